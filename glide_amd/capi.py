@@ -1,0 +1,180 @@
+"""ctypes binding of libglide_hip.so (the C ABI declared in include/glide_hip.h).
+
+The library is the product; this module only marshals arguments.  There is no CPU fallback: if the shared
+library is missing or a call fails, an exception is raised.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libglide_hip.so")
+_lib = None
+
+EUCLIDEAN, COSINE = 0, 1
+INVALID = 0xFFFFFFFF
+
+u32, f32, vp = C.c_uint32, C.c_float, C.c_void_p
+
+
+class GlideHipError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__("%s failed: %s (code %d)" % (what, error_string(code), code))
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libglide_hip.so is not built: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                               "or `make -C glide_amd/csrc`")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.glide_hip_version.restype = C.c_char_p
+        _lib.glide_hip_error_string.restype = C.c_char_p
+    return _lib
+
+
+def error_string(code):
+    return lib().glide_hip_error_string(C.c_int(code)).decode()
+
+
+def check(code, what):
+    if code != 0:
+        raise GlideHipError(code, what)
+
+
+def version():
+    return lib().glide_hip_version().decode()
+
+
+def set_device(device=0):
+    check(lib().glide_hip_set_device(C.c_int(device)), "glide_hip_set_device")
+
+
+def device_info():
+    name = C.create_string_buffer(256)
+    cus, mem = C.c_int(0), C.c_size_t(0)
+    check(lib().glide_hip_device_info(name, C.c_size_t(256), C.byref(cus), C.byref(mem)), "glide_hip_device_info")
+    return dict(name=name.value.decode(), compute_units=cus.value, total_mem=mem.value)
+
+
+class DeviceArray:
+    """A typed device allocation owned through glide_hip_malloc / glide_hip_free."""
+
+    def __init__(self, shape, dtype):
+        self.shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = vp()
+        check(lib().glide_hip_malloc(C.byref(p), C.c_size_t(self.nbytes)), "glide_hip_malloc")
+        self.ptr = p.value
+
+    @classmethod
+    def from_numpy(cls, arr, dtype=None):
+        arr = np.ascontiguousarray(arr, dtype=dtype)
+        d = cls(arr.shape, arr.dtype)
+        d.upload(arr)
+        return d
+
+    @classmethod
+    def full(cls, shape, value, dtype=np.uint32):
+        d = cls(shape, dtype)
+        assert d.dtype.itemsize == 4
+        v = int(np.array([value], dtype=d.dtype).view(np.uint32)[0])
+        check(lib().glide_hip_fill_u32(vp(d.ptr), u32(v), C.c_size_t(d.nbytes // 4), None), "glide_hip_fill_u32")
+        return d
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr, dtype=self.dtype)
+        assert arr.nbytes == self.nbytes
+        check(lib().glide_hip_memcpy_h2d(vp(self.ptr), arr.ctypes.data_as(vp), C.c_size_t(self.nbytes), None),
+              "glide_hip_memcpy_h2d")
+
+    def numpy(self):
+        out = np.empty(self.shape, dtype=self.dtype)
+        check(lib().glide_hip_memcpy_d2h(out.ctypes.data_as(vp), vp(self.ptr), C.c_size_t(self.nbytes), None),
+              "glide_hip_memcpy_d2h")
+        return out
+
+    def free(self):
+        if self.ptr:
+            lib().glide_hip_free(vp(self.ptr))
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _ptr(x):
+    """Device pointer of a DeviceArray, a torch tensor, a raw int, or None."""
+    if x is None:
+        return vp(None)
+    if isinstance(x, DeviceArray):
+        return vp(x.ptr)
+    if isinstance(x, int):
+        return vp(x)
+    if hasattr(x, "data_ptr"):
+        return vp(x.data_ptr())
+    raise TypeError("not a device buffer: %r" % type(x))
+
+
+def synchronize(stream=None):
+    check(lib().glide_hip_stream_synchronize(vp(stream)), "glide_hip_stream_synchronize")
+
+
+class Event:
+    def __init__(self):
+        p = vp()
+        check(lib().glide_hip_event_create(C.byref(p)), "glide_hip_event_create")
+        self.ptr = p.value
+
+    def record(self, stream=None):
+        check(lib().glide_hip_event_record(vp(self.ptr), vp(stream)), "glide_hip_event_record")
+
+    def elapsed_ms(self, stop):
+        ms = f32(0)
+        check(lib().glide_hip_event_elapsed_ms(vp(self.ptr), vp(stop.ptr), C.byref(ms)), "glide_hip_event_elapsed_ms")
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib().glide_hip_event_destroy(vp(self.ptr))
+        except Exception:
+            pass
+
+
+# ------------------------------------------------------------------------------------------- entry points
+def search(data, num, dim, graph, graph_degree, centroids, centroid_num, start_points, queries, query_num, top_k,
+           beam, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric, result_ids, result_dists,
+           counters=None, stream=None):
+    check(lib().glide_hip_search(_ptr(data), u32(num), u32(dim), _ptr(graph), u32(graph_degree), _ptr(centroids),
+                                 u32(centroid_num), _ptr(start_points), _ptr(queries), u32(query_num), u32(top_k),
+                                 u32(beam), u32(max_iterations), u32(min_iterations), u32(hash_bit),
+                                 u32(hash_reset_interval), C.c_int(metric), _ptr(result_ids), _ptr(result_dists),
+                                 _ptr(counters), vp(stream)), "glide_hip_search")
+
+
+def distance_batch(a, b, n, dim, metric, out, stream=None):
+    check(lib().glide_hip_distance_batch(_ptr(a), _ptr(b), u32(n), u32(dim), C.c_int(metric), _ptr(out), vp(stream)),
+          "glide_hip_distance_batch")
+
+
+def bitonic_sort_kv(keys, vals, m, batch, stream=None):
+    check(lib().glide_hip_bitonic_sort_kv(_ptr(keys), _ptr(vals), u32(m), u32(batch), vp(stream)),
+          "glide_hip_bitonic_sort_kv")
+
+
+def bitonic_merge_kv(keys, vals, m, batch, stream=None):
+    check(lib().glide_hip_bitonic_merge_kv(_ptr(keys), _ptr(vals), u32(m), u32(batch), vp(stream)),
+          "glide_hip_bitonic_merge_kv")
+
+
+def hashmap_insert_seq(table, bitlen, keys, n, flags, stream=None):
+    check(lib().glide_hip_hashmap_insert_seq(_ptr(table), u32(bitlen), _ptr(keys), u32(n), _ptr(flags), vp(stream)),
+          "glide_hip_hashmap_insert_seq")

@@ -1,0 +1,264 @@
+// Beam-search core for one item per 64-lane wavefront (search, sub-graph build, refine all use it).
+//
+// Reference semantics: search_kernel.cuh:433-482 / graph_kernel.cuh:16-63 (one iteration), :9-37 and :97-148
+// (candidate sort, beam merge), :292-325 (parent selection), :327-334 (hash restore), :336-391 (expansion).
+//
+// Layout: the beam (MAX_BEAM entries) lives in registers, element e = NB*lane + r, ascending, explored flag in
+// the id's MSB.  The D candidates of one expansion are produced into LDS by graph-row slot, pulled into
+// registers with the reference's strided->blocked permutation, sorted by the wave network and staged back to
+// LDS so that beam element e can pick candidate MAX_BEAM-1-e (the half-cleaner).  The visited set is an LDS
+// open-addressing table.  Data rows are gathered two at a time (one 32-lane half each, 16 B per lane).
+#pragma once
+#include "bitonic.hpp"
+
+namespace glide {
+
+struct BeamParams {
+    uint32_t beam, degree, dim, hash_bit, reset_interval, max_iterations, min_iterations;
+    int metric;
+};
+
+struct BeamCounters {  // wave-uniform tallies for traffic accounting
+    uint32_t iterations = 0, rows_scored = 0, graph_rows = 0;
+};
+
+template <int MAX_CAND>
+struct BeamLds {  // per-wave LDS (the hash table follows, 1 << hash_bit words)
+    uint32_t cand_id[MAX_CAND];
+    float cand_dist[MAX_CAND];
+    uint32_t vlist[MAX_CAND];
+};
+
+__device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
+
+template <int MAX_CAND, int MAX_BEAM, int DIMV>
+struct Beam {
+    static constexpr int NB = MAX_BEAM / 64;
+    static constexpr int NC = MAX_CAND / 64;
+    static constexpr int NC32 = MAX_CAND / 32;  // items per lane in the reference's 32-lane layout
+
+    float bk[NB];
+    uint32_t bv[NB];
+    RowRegs<DIMV> q;
+    BeamLds<MAX_CAND>* lds;
+    uint32_t* hash;
+    BeamParams p;
+    BeamCounters cnt;
+    int lane;
+
+    __device__ __forceinline__ void init(BeamLds<MAX_CAND>* lds_, uint32_t* hash_, const BeamParams& p_, const float* query) {
+        lds = lds_;
+        hash = hash_;
+        p = p_;
+        lane = lane_id();
+        load_row<DIMV>(q, query, p.dim, lane & 31);
+        hash_clear(hash, p.hash_bit, lane);
+        wave_sync();
+    }
+
+    // Expansion of `parent` (reference compute_distance / get_init / result_init second half):
+    // every neighbour not yet in the visited set becomes a candidate; `exclude_insert` is never inserted,
+    // `exclude_score` is inserted and kept as a candidate id but gets distance FLT_MAX.
+    __device__ __forceinline__ void expand(uint32_t parent, const uint32_t* graph, const float* data,
+                                           uint32_t exclude_insert, uint32_t exclude_score) {
+        uint32_t nv = 0;
+        if (parent != kInvalid) cnt.graph_rows++;
+#pragma unroll
+        for (int s0 = 0; s0 < MAX_CAND; s0 += 64) {
+            const uint32_t s = s0 + lane;
+            uint32_t nid = kInvalid;
+            if (s < p.degree && parent != kInvalid) nid = graph[static_cast<size_t>(parent) * p.degree + s];
+            const uint32_t flag = (nid != kInvalid && nid != exclude_insert) ? hash_insert(hash, p.hash_bit, nid) : 0;
+            const uint32_t cid = flag ? nid : kInvalid;
+            lds->cand_id[s] = cid;
+            lds->cand_dist[s] = FLT_MAX;
+            const bool score = cid != kInvalid && cid != exclude_score;
+            const uint64_t m = ballot(score);
+            if (score) lds->vlist[nv + prefix_count(m)] = s;
+            nv += __popcll(m);
+        }
+        wave_sync();
+        cnt.rows_scored += nv;
+        const int half = lane >> 5, t = lane & 31;
+        constexpr int U = DIMV == 1 ? 4 : (DIMV == 2 ? 2 : 1);  // row pairs in flight per trip
+        for (uint32_t base = 0; base < nv; base += 2 * U) {
+            RowRegs<DIMV> rows[U];
+            uint32_t slot[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const uint32_t idx = base + 2 * u + half;
+                const bool active = idx < nv;
+                slot[u] = active ? lds->vlist[idx] : kInvalid;
+                const uint32_t id = active ? lds->cand_id[slot[u]] : 0u;
+                const float* row = data + static_cast<size_t>(id) * p.dim;
+                if (active) {
+                    load_row<DIMV>(rows[u], row, p.dim, t);
+                } else {
+                    rows[u] = q;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float d = finish_distance(half_wave_sum(partial_sqdist<DIMV>(q, rows[u])), p.metric);
+                if (t == 0 && slot[u] != kInvalid) lds->cand_dist[slot[u]] = d;
+            }
+        }
+        wave_sync();
+    }
+
+    // reference update_result_buffer: sort the candidates, then fold them into the beam
+    __device__ __forceinline__ void absorb(bool first) {
+        float ck[NC];
+        uint32_t cv[NC];
+#pragma unroll
+        for (int r = 0; r < NC; r++) {
+            const uint32_t e = NC * lane + r;          // element index in the network
+            const uint32_t l32 = e / NC32, i = e % NC32;
+            const uint32_t slot = l32 + 32 * i;        // reference loads strided: j = lane + 32*i
+            ck[r] = slot < p.degree ? lds->cand_dist[slot] : FLT_MAX;
+            cv[r] = slot < p.degree ? lds->cand_id[slot] : kInvalid;
+        }
+        WaveNet<MAX_CAND>::sort(ck, cv, lane);
+        wave_sync();
+#pragma unroll
+        for (int r = 0; r < NC; r++) {
+            const uint32_t e = NC * lane + r;
+            lds->cand_dist[e] = ck[r];
+            lds->cand_id[e] = cv[r];
+        }
+        wave_sync();
+        if (first) {
+#pragma unroll
+            for (int r = 0; r < NB; r++) {
+                const uint32_t e = NB * lane + r;
+                const bool take = e < p.beam && e < p.degree;
+                bk[r] = take ? lds->cand_dist[e] : FLT_MAX;
+                bv[r] = take ? lds->cand_id[e] : kInvalid;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < NB; r++) {
+                const uint32_t e = NB * lane + r;
+                const uint32_t k = MAX_BEAM - 1 - e;
+                if (k < p.beam && k < p.degree) {
+                    const float c = lds->cand_dist[k];
+                    if (bk[r] > c) {
+                        bk[r] = c;
+                        bv[r] = lds->cand_id[k];
+                    }
+                }
+            }
+            WaveNet<MAX_BEAM>::merge(bk, bv, lane);
+#pragma unroll
+            for (int r = 0; r < NB; r++) {
+                const uint32_t e = NB * lane + r;
+                if (e >= p.beam) {
+                    bk[r] = FLT_MAX;
+                    bv[r] = kInvalid;
+                }
+            }
+        }
+        wave_sync();
+    }
+
+    // first unexplored beam entry (reference select_current_point); marks it explored
+    __device__ __forceinline__ uint32_t select_parent() {
+        int rsel = NB;
+#pragma unroll
+        for (int r = NB - 1; r >= 0; r--) {
+            const uint32_t e = NB * lane + r;
+            if (e < p.beam && (bv[r] & kExplored) == 0) rsel = r;
+        }
+        const uint64_t m = ballot(rsel < NB);
+        if (m == 0) return kInvalid;
+        const int src = __builtin_ctzll(m);
+        const int r_src = __builtin_amdgcn_readlane(rsel, src);
+        uint32_t mine = 0;
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            if (r == r_src) {
+                mine = bv[r];
+                if (lane == src) bv[r] |= kExplored;
+            }
+        }
+        return read_lane(mine, src);
+    }
+
+    __device__ __forceinline__ void restore_hash() {
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t e = NB * lane + r;
+            if (e < p.beam) hash_insert(hash, p.hash_bit, bv[r] & kClean);
+        }
+    }
+
+    // main loop; candidates of the entry expansion must already be in LDS
+    __device__ __forceinline__ void run(const uint32_t* graph, const float* data, uint32_t self_id) {
+        uint32_t iter = 0;
+        bool terminate = false;
+        while (true) {
+            absorb(iter == 0);
+            cnt.iterations++;
+            const bool reset_now = ((iter + 1) % p.reset_interval) == 0;
+            if (reset_now) {
+                hash_clear(hash, p.hash_bit, lane);
+                wave_sync();
+            }
+            if (iter + 1 == p.max_iterations) break;
+            const uint32_t parent = select_parent();
+            if (parent == kInvalid) terminate = true;
+            if (reset_now) {
+                restore_hash();
+                wave_sync();
+            }
+            if (terminate && iter >= p.min_iterations) break;
+            expand(parent, graph, data, self_id, kInvalid);
+            iter++;
+        }
+    }
+
+    __device__ __forceinline__ void flush_counters(unsigned long long* counters) {
+        if (counters != nullptr && lane == 0) {
+            atomicAdd(&counters[0], static_cast<unsigned long long>(cnt.iterations));
+            atomicAdd(&counters[1], static_cast<unsigned long long>(cnt.rows_scored));
+            atomicAdd(&counters[2], static_cast<unsigned long long>(cnt.graph_rows));
+        }
+    }
+};
+
+// Nearest centroid by the reference's sort network (search_kernel.cuh:259-268, distance.cuh:29-60):
+// strided load, blocked store, element 0 is the winner.  One wavefront; scratch holds `centroid_num` pairs.
+template <int MAX_CENTROID, int DIMV>
+__device__ __forceinline__ uint32_t nearest_centroid(const RowRegs<DIMV>& q, const float* centroids, uint32_t centroid_num,
+                                                     uint32_t dim, int metric, float* cent_dist, int lane) {
+    const int half = lane >> 5, t = lane & 31;
+    for (uint32_t c0 = 0; c0 < centroid_num; c0 += 2) {
+        const uint32_t c = c0 + half;
+        RowRegs<DIMV> row;
+        if (c < centroid_num) {
+            load_row<DIMV>(row, centroids + static_cast<size_t>(c) * dim, dim, t);
+        } else {
+            row = q;
+        }
+        const float d = finish_distance(half_wave_sum(partial_sqdist<DIMV>(q, row)), metric);
+        if (t == 0 && c < centroid_num) cent_dist[c] = d;
+    }
+    wave_sync();
+    constexpr int NR = WaveNet<MAX_CENTROID>::NR;
+    constexpr int N32 = MAX_CENTROID / 32;
+    float k[NR];
+    uint32_t v[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        const uint32_t j = (e / N32) + 32 * (e % N32);
+        const bool ok = (MAX_CENTROID >= 64 || lane < 32) && j < centroid_num;
+        k[r] = ok ? cent_dist[j] : FLT_MAX;
+        v[r] = ok ? j : kInvalid;
+    }
+    WaveNet<MAX_CENTROID>::sort(k, v, lane);
+    wave_sync();
+    return read_lane(v[0], 0);
+}
+
+}  // namespace glide

@@ -1,0 +1,77 @@
+// Bitonic sort / merge of (float key, u32 value) pairs held in the registers of one 64-lane wavefront.
+//
+// The reference (bitonic.cuh:24-212) runs the standard bitonic network over M = 32*N elements with element
+// index e = N*lane32 + i and a compare-exchange that does nothing on equal keys.  The network is a property of
+// the element indices, not of the lane width, so the same comparator sequence is executed here with
+// e = NR*lane64 + r, NR = M/64 (M = 32 uses lanes 0..31 with NR = 1; lanes 32..63 run a private copy).
+// Same comparators in the same stage order => identical output sequence, ties included.
+#pragma once
+#include "common.hpp"
+
+namespace glide {
+
+template <int M>
+struct WaveNet {
+    static_assert(M == 32 || M == 64 || M == 128 || M == 256 || M == 512, "network size");
+    static constexpr int NR = M >= 64 ? M / 64 : 1;
+
+    // compare-exchange of two registers of the same lane (bitonic.cuh:25-34)
+    static __device__ __forceinline__ void cmpx_reg(float& k0, uint32_t& v0, float& k1, uint32_t& v1, bool asc) {
+        if ((k0 != k1) && ((k0 < k1) != asc)) {
+            float tk = k0; k0 = k1; k1 = tk;
+            uint32_t tv = v0; v0 = v1; v1 = tv;
+        }
+    }
+    // compare-exchange with the lane `lane ^ LM` (bitonic.cuh:36-44); keep_min: this lane keeps the smaller key
+    template <int LM>
+    static __device__ __forceinline__ void cmpx_lane(float& k, uint32_t& v, bool keep_min) {
+        const float ok = lane_xor<LM>(k);
+        const uint32_t ov = lane_xor<LM>(v);
+        if ((k != ok) && ((k < ok) != keep_min)) {
+            k = ok;
+            v = ov;
+        }
+    }
+
+    // one network stage: partner distance J (elements), direction block K (elements); K == M means all ascending
+    template <int K, int J>
+    static __device__ __forceinline__ void stage(float (&k)[NR], uint32_t (&v)[NR], int lane) {
+        if constexpr (J < NR) {
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                if ((r & J) == 0) {
+                    const int e = NR * lane + r;
+                    const bool asc = (K >= M) ? true : ((e & K) == 0);
+                    cmpx_reg(k[r], v[r], k[r | J], v[r | J], asc);
+                }
+            }
+        } else {
+            constexpr int LM = J / NR;
+            const bool lower = (lane & LM) == 0;
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                const int e = NR * lane + r;
+                const bool asc = (K >= M) ? true : ((e & K) == 0);
+                cmpx_lane<LM>(k[r], v[r], lower == asc);
+            }
+        }
+    }
+
+    template <int K, int J>
+    static __device__ __forceinline__ void merge_from(float (&k)[NR], uint32_t (&v)[NR], int lane) {
+        stage<K, J>(k, v, lane);
+        if constexpr (J > 1) merge_from<K, J / 2>(k, v, lane);
+    }
+    template <int K>
+    static __device__ __forceinline__ void sort_from(float (&k)[NR], uint32_t (&v)[NR], int lane) {
+        merge_from<K, K / 2>(k, v, lane);
+        if constexpr (K < M) sort_from<K * 2>(k, v, lane);
+    }
+
+    // full ascending sort (reference warp_sort, bitonic.cuh:207-212)
+    static __device__ __forceinline__ void sort(float (&k)[NR], uint32_t (&v)[NR], int lane) { sort_from<2>(k, v, lane); }
+    // final ascending merge of a bitonic sequence (reference warp_merge with range 32, bitonic.cuh:202-205)
+    static __device__ __forceinline__ void merge(float (&k)[NR], uint32_t (&v)[NR], int lane) { merge_from<M, M / 2>(k, v, lane); }
+};
+
+}  // namespace glide

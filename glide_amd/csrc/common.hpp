@@ -1,0 +1,130 @@
+// Wave64 device primitives shared by every GLIDE kernel on gfx950 (CDNA4).
+//
+// One wavefront = 64 lanes.  All per-item kernels (search, sub-graph build, refine) give one item to one
+// wavefront, so the "warp 0 / other warps" split and the block barriers of the reference collapse into
+// straight-line wave code.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <float.h>
+
+namespace glide {
+
+constexpr uint32_t kInvalid = 0xffffffffu;
+constexpr uint32_t kExplored = 0x80000000u;  // reference utils.cuh:5-8
+constexpr uint32_t kClean = 0x7fffffffu;
+constexpr int kWave = 64;
+
+enum Metric : int { kEuclidean = 0, kCosine = 1 };  // reference params.cuh:5-8
+
+__host__ __device__ constexpr uint32_t round_up32(uint32_t p) { return (p + 31u) & ~31u; }  // utils.cuh:21-23
+__host__ __device__ constexpr uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+__device__ __forceinline__ int lane_id() { return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))); }
+
+// ---------------------------------------------------------------- cross-lane exchange, compile-time xor mask
+// xor 1,2: DPP quad_perm; xor 4: two banked DPP row shifts; xor 8: DPP row_ror:8; xor 16: ds_swizzle (LDS
+// crossbar, no memory); xor 32: ds_bpermute.
+template <int MASK>
+__device__ __forceinline__ int lane_xor_i(int v) {
+    static_assert(MASK == 1 || MASK == 2 || MASK == 4 || MASK == 8 || MASK == 16 || MASK == 32, "xor mask");
+    if constexpr (MASK == 1) {
+        return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false);  // quad_perm:[1,0,3,2]
+    } else if constexpr (MASK == 2) {
+        return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false);  // quad_perm:[2,3,0,1]
+    } else if constexpr (MASK == 4) {
+        int r = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xf, 0x5, false);  // row_shl:4 -> banks 0,2 read lane+4
+        r = __builtin_amdgcn_update_dpp(r, v, 0x114, 0xf, 0xA, false);      // row_shr:4 -> banks 1,3 read lane-4
+        return r;
+    } else if constexpr (MASK == 8) {
+        return __builtin_amdgcn_update_dpp(v, v, 0x128, 0xf, 0xf, false);  // row_ror:8
+    } else if constexpr (MASK == 16) {
+        return __builtin_amdgcn_ds_swizzle(v, 0x401F);  // BITMODE and=0x1f or=0 xor=0x10
+    } else {
+        return __builtin_amdgcn_ds_bpermute((lane_id() ^ 32) << 2, v);
+    }
+}
+template <int MASK>
+__device__ __forceinline__ float lane_xor(float v) { return __builtin_bit_cast(float, lane_xor_i<MASK>(__builtin_bit_cast(int, v))); }
+template <int MASK>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v) { return static_cast<uint32_t>(lane_xor_i<MASK>(static_cast<int>(v))); }
+
+__device__ __forceinline__ float read_lane(float v, int lane) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane)); }
+__device__ __forceinline__ uint32_t read_lane(uint32_t v, int lane) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane)); }
+__device__ __forceinline__ uint32_t shfl_u32(uint32_t v, int src_lane) { return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(src_lane << 2, static_cast<int>(v))); }
+__device__ __forceinline__ float shfl_f32(float v, int src_lane) { return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src_lane << 2, __builtin_bit_cast(int, v))); }
+
+__device__ __forceinline__ uint64_t ballot(bool p) { return __ballot(p); }
+// number of set bits of `mask` strictly below this lane
+__device__ __forceinline__ uint32_t prefix_count(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+}
+
+// Sum over each 32-lane half of the wave; every lane of a half ends with that half's total.
+__device__ __forceinline__ float half_wave_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));  // row_mirror
+    v += lane_xor<16>(v);
+    return v;
+}
+// Sum over the whole wave; every lane ends with the total.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = half_wave_sum(v);
+    v += lane_xor<32>(v);
+    return v;
+}
+
+// ---------------------------------------------------------------- LDS open-addressing hash set (reference hashmap.cuh:23-56)
+__device__ __forceinline__ void hash_clear(uint32_t* table, uint32_t bitlen, int lane) {
+    for (uint32_t i = lane; i < (1u << bitlen); i += kWave) table[i] = kInvalid;
+}
+// returns 1 iff `key` was newly stored; 0 if present or the table is full
+__device__ __forceinline__ uint32_t hash_insert(uint32_t* table, uint32_t bitlen, uint32_t key) {
+    const uint32_t size = 1u << bitlen;
+    const uint32_t mask = size - 1;
+    uint32_t index = (key ^ (key >> bitlen)) & mask;
+    for (uint32_t i = 0; i < size; i++) {
+        const uint32_t old = atomicCAS(&table[index], kInvalid, key);
+        if (old == kInvalid) return 1;
+        if (old == key) return 0;
+        index = (index + 1) & mask;
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------- row distance with a 32-lane half per row
+// Lane t of a half owns dims [c*128 + 4t, c*128 + 4t + 4) of chunk c.  DIMV = number of 128-dim chunks.
+template <int DIMV>
+struct RowRegs {
+    float4 v[DIMV];
+};
+
+template <int DIMV>
+__device__ __forceinline__ void load_row(RowRegs<DIMV>& r, const float* row, uint32_t dim, int t) {
+#pragma unroll
+    for (int c = 0; c < DIMV; c++) {
+        const uint32_t d0 = c * 128 + t * 4;
+        r.v[c] = d0 < dim ? *reinterpret_cast<const float4*>(row + d0) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+
+template <int DIMV>
+__device__ __forceinline__ float partial_sqdist(const RowRegs<DIMV>& a, const RowRegs<DIMV>& b) {
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < DIMV; c++) {
+        float dx = a.v[c].x - b.v[c].x, dy = a.v[c].y - b.v[c].y, dz = a.v[c].z - b.v[c].z, dw = a.v[c].w - b.v[c].w;
+        acc = fmaf(dx, dx, acc);
+        acc = fmaf(dy, dy, acc);
+        acc = fmaf(dz, dz, acc);
+        acc = fmaf(dw, dw, acc);
+    }
+    return acc;
+}
+
+// reference distance.cuh:22-26: Euclidean reports sqrt, Cosine the squared L2 of pre-normalised rows
+__device__ __forceinline__ float finish_distance(float sq, int metric) { return metric == kEuclidean ? sqrtf(sq) : sq; }
+
+}  // namespace glide

@@ -1,0 +1,119 @@
+// Test hooks exposing the device primitives one at a time (distance, bitonic network, hash set).
+#include "beam.hpp"
+#include "host_util.hpp"
+
+namespace glide {
+
+// one 32-lane half per row pair; generic dim (any multiple of 4, looped in 128-dim chunks)
+__global__ __launch_bounds__(64) void distance_batch_kernel(const float* a, const float* b, uint32_t n, uint32_t dim,
+                                                            int metric, float* out) {
+    const int lane = lane_id();
+    const int half = lane >> 5, t = lane & 31;
+    const uint32_t i = blockIdx.x * 2 + half;
+    float acc = 0.f;
+    if (i < n) {
+        const float* x = a + static_cast<size_t>(i) * dim;
+        const float* y = b + static_cast<size_t>(i) * dim;
+        for (uint32_t d0 = t * 4; d0 < dim; d0 += 128) {
+            RowRegs<1> rx, ry;
+            rx.v[0] = *reinterpret_cast<const float4*>(x + d0);
+            ry.v[0] = *reinterpret_cast<const float4*>(y + d0);
+            acc += partial_sqdist<1>(rx, ry);
+        }
+    }
+    const float d = finish_distance(half_wave_sum(acc), metric);
+    if (i < n && t == 0) out[i] = d;
+}
+
+template <int M, bool MERGE_ONLY>
+__global__ __launch_bounds__(64) void bitonic_kernel(float* keys, uint32_t* vals, uint32_t batch) {
+    constexpr int NR = WaveNet<M>::NR;
+    const int lane = lane_id();
+    const uint32_t b = blockIdx.x;
+    if (b >= batch) return;
+    float k[NR];
+    uint32_t v[NR];
+    const bool live = (M >= 64) || lane < 32;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        k[r] = live ? keys[static_cast<size_t>(b) * M + e] : FLT_MAX;
+        v[r] = live ? vals[static_cast<size_t>(b) * M + e] : kInvalid;
+    }
+    if (MERGE_ONLY) {
+        WaveNet<M>::merge(k, v, lane);
+    } else {
+        WaveNet<M>::sort(k, v, lane);
+    }
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        if (live) {
+            keys[static_cast<size_t>(b) * M + e] = k[r];
+            vals[static_cast<size_t>(b) * M + e] = v[r];
+        }
+    }
+}
+
+// keys are inserted strictly one after another (lane 0 only), so flags match a sequential host model; the
+// table is staged through LDS to exercise the same ds atomics as the search kernels.
+__global__ __launch_bounds__(64) void hashmap_seq_kernel(uint32_t* table, uint32_t bitlen, const uint32_t* keys, uint32_t n,
+                                                         uint32_t* flags) {
+    extern __shared__ uint32_t lds_table[];
+    const int lane = lane_id();
+    for (uint32_t i = lane; i < (1u << bitlen); i += 64) lds_table[i] = table[i];
+    __syncthreads();
+    if (lane == 0)
+        for (uint32_t i = 0; i < n; i++) flags[i] = hash_insert(lds_table, bitlen, keys[i]);
+    __syncthreads();
+    for (uint32_t i = lane; i < (1u << bitlen); i += 64) table[i] = lds_table[i];
+}
+
+template <bool MERGE_ONLY>
+int launch_bitonic(float* keys, uint32_t* vals, uint32_t m, uint32_t batch, hipStream_t s) {
+    switch (m) {
+        case 32: hipLaunchKernelGGL((bitonic_kernel<32, MERGE_ONLY>), dim3(batch), dim3(64), 0, s, keys, vals, batch); break;
+        case 64: hipLaunchKernelGGL((bitonic_kernel<64, MERGE_ONLY>), dim3(batch), dim3(64), 0, s, keys, vals, batch); break;
+        case 128: hipLaunchKernelGGL((bitonic_kernel<128, MERGE_ONLY>), dim3(batch), dim3(64), 0, s, keys, vals, batch); break;
+        case 256: hipLaunchKernelGGL((bitonic_kernel<256, MERGE_ONLY>), dim3(batch), dim3(64), 0, s, keys, vals, batch); break;
+        case 512: hipLaunchKernelGGL((bitonic_kernel<512, MERGE_ONLY>), dim3(batch), dim3(64), 0, s, keys, vals, batch); break;
+        default: return GLIDE_ERR_UNSUPPORTED;
+    }
+    return launch_status();
+}
+
+}  // namespace glide
+
+using namespace glide;
+
+extern "C" {
+
+int glide_hip_distance_batch(const float* a, const float* b, uint32_t n, uint32_t dim, int metric, float* out, void* stream) {
+    if (!a || !b || !out || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    if (n == 0) return GLIDE_OK;
+    hipLaunchKernelGGL(distance_batch_kernel, dim3((n + 1) / 2), dim3(64), 0, as_stream(stream), a, b, n, dim, metric, out);
+    return launch_status();
+}
+
+int glide_hip_bitonic_sort_kv(float* keys, uint32_t* vals, uint32_t m, uint32_t batch, void* stream) {
+    if (!keys || !vals) return GLIDE_ERR_BAD_ARGUMENT;
+    if (batch == 0) return GLIDE_OK;
+    return launch_bitonic<false>(keys, vals, m, batch, as_stream(stream));
+}
+
+int glide_hip_bitonic_merge_kv(float* keys, uint32_t* vals, uint32_t m, uint32_t batch, void* stream) {
+    if (!keys || !vals) return GLIDE_ERR_BAD_ARGUMENT;
+    if (batch == 0) return GLIDE_OK;
+    return launch_bitonic<true>(keys, vals, m, batch, as_stream(stream));
+}
+
+int glide_hip_hashmap_insert_seq(uint32_t* table, uint32_t bitlen, const uint32_t* keys, uint32_t n, uint32_t* flags, void* stream) {
+    if (!table || !keys || !flags) return GLIDE_ERR_BAD_ARGUMENT;
+    if (bitlen < 1 || bitlen > 13) return GLIDE_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(hashmap_seq_kernel, dim3(1), dim3(64), (size_t{1} << bitlen) * sizeof(uint32_t), as_stream(stream), table,
+                       bitlen, keys, n, flags);
+    return launch_status();
+}
+
+}  // extern "C"

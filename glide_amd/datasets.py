@@ -1,0 +1,97 @@
+"""Seeded synthetic datasets with the shapes of the benchmark configurations, and the fbin file format.
+
+File formats follow the reference's load.cuh:8-128: fbin = u32 num, u32 dim, then num*dim values row-major.
+"""
+import numpy as np
+
+
+def gmm_clipped(num, dim=128, components=64, mean_hi=160.0, sigma=25.0, seed=1234, mixture_seed=99):
+    """Gaussian mixture with means uniform in [0, mean_hi], clipped to [0, 255] and rounded to integers.
+
+    The mixture (means) depends only on `mixture_seed`, so base vectors and queries drawn with different
+    `seed`s come from the same distribution.
+    """
+    means = np.random.default_rng(mixture_seed).uniform(0.0, mean_hi, size=(components, dim)).astype(np.float32)
+    rng = np.random.default_rng(seed)
+    out = np.empty((num, dim), dtype=np.float32)
+    step = 1 << 18
+    for s in range(0, num, step):
+        e = min(num, s + step)
+        comp = rng.integers(0, components, size=e - s)
+        x = means[comp] + rng.standard_normal((e - s, dim), dtype=np.float32) * np.float32(sigma)
+        out[s:e] = np.rint(np.clip(x, 0.0, 255.0))
+    return out
+
+
+def gmm_normalized(num, dim=96, components=256, sigma=0.3, seed=1234, mixture_seed=98):
+    """Gaussian mixture with N(0,1) means, each row L2-normalised (cosine configuration)."""
+    means = np.random.default_rng(mixture_seed).standard_normal((components, dim)).astype(np.float32)
+    rng = np.random.default_rng(seed)
+    comp = rng.integers(0, components, size=num)
+    x = means[comp] + rng.standard_normal((num, dim), dtype=np.float32) * np.float32(sigma)
+    x /= np.linalg.norm(x, axis=1, keepdims=True).astype(np.float32)
+    return x.astype(np.float32)
+
+
+def beta_scaled(num, dim=960, components=128, seed=1234, mixture_seed=97):
+    """Beta(0.5, 2) per dimension, modulated by a per-cluster dimension-wise scale vector; values in [0, 1]."""
+    scales = np.random.default_rng(mixture_seed).uniform(0.05, 1.0, size=(components, dim)).astype(np.float32)
+    rng = np.random.default_rng(seed)
+    out = np.empty((num, dim), dtype=np.float32)
+    step = 1 << 16
+    for s in range(0, num, step):
+        e = min(num, s + step)
+        comp = rng.integers(0, components, size=e - s)
+        out[s:e] = rng.beta(0.5, 2.0, size=(e - s, dim)).astype(np.float32) * scales[comp]
+    return out
+
+
+def write_fbin(path, matrix):
+    matrix = np.ascontiguousarray(matrix)
+    with open(path, "wb") as f:
+        np.array(matrix.shape, dtype=np.uint32).tofile(f)
+        matrix.tofile(f)
+
+
+def read_fbin(path, dtype=np.float32):
+    with open(path, "rb") as f:
+        num, dim = np.fromfile(f, dtype=np.uint32, count=2)
+        return np.fromfile(f, dtype=dtype, count=int(num) * int(dim)).reshape(int(num), int(dim))
+
+
+def write_vector(path, vec):
+    vec = np.ascontiguousarray(vec, dtype=np.uint32)
+    with open(path, "wb") as f:
+        np.array([vec.size], dtype=np.uint32).tofile(f)
+        vec.tofile(f)
+
+
+def read_vector(path):
+    with open(path, "rb") as f:
+        n = int(np.fromfile(f, dtype=np.uint32, count=1)[0])
+        return np.fromfile(f, dtype=np.uint32, count=n)
+
+
+def write_segment(path, starts, lengths):
+    starts = np.ascontiguousarray(starts, dtype=np.uint32)
+    lengths = np.ascontiguousarray(lengths, dtype=np.uint32)
+    with open(path, "wb") as f:
+        np.array([starts.size], dtype=np.uint32).tofile(f)
+        starts.tofile(f)
+        lengths.tofile(f)
+
+
+def read_segment(path):
+    with open(path, "rb") as f:
+        n = int(np.fromfile(f, dtype=np.uint32, count=1)[0])
+        starts = np.fromfile(f, dtype=np.uint32, count=n)
+        lengths = np.fromfile(f, dtype=np.uint32, count=n)
+    return starts, lengths
+
+
+def recall(result_ids, truth_ids, k):
+    """Mean fraction of the true top-k found among the returned top-k (small_search.cu:14-36)."""
+    hit = 0
+    for r, t in zip(result_ids[:, :k], truth_ids[:, :k]):
+        hit += len(set(r.tolist()) & set(t.tolist()))
+    return hit / float(result_ids.shape[0] * k)
