@@ -178,3 +178,50 @@ def bitonic_merge_kv(keys, vals, m, batch, stream=None):
 def hashmap_insert_seq(table, bitlen, keys, n, flags, stream=None):
     check(lib().glide_hip_hashmap_insert_seq(_ptr(table), u32(bitlen), _ptr(keys), u32(n), _ptr(flags), vp(stream)),
           "glide_hip_hashmap_insert_seq")
+
+
+def build_subgraph(reorder_data, num, dim, knn_graph, knn_degree, mp, segment_starts, segment_lengths, segment_num,
+                   start_points, graph_degree, beam, max_iterations, min_iterations, hash_bit, hash_reset_interval,
+                   relaxant, metric, graph, counters=None, stream=None):
+    check(lib().glide_hip_build_subgraph(_ptr(reorder_data), u32(num), u32(dim), _ptr(knn_graph), u32(knn_degree),
+                                         _ptr(mp), _ptr(segment_starts), _ptr(segment_lengths), u32(segment_num),
+                                         _ptr(start_points), u32(graph_degree), u32(beam), u32(max_iterations),
+                                         u32(min_iterations), u32(hash_bit), u32(hash_reset_interval), f32(relaxant),
+                                         C.c_int(metric), _ptr(graph), _ptr(counters), vp(stream)),
+          "glide_hip_build_subgraph")
+
+
+def build_boundary(reorder_data, num, reorder_num, dim, knn_graph, knn_degree, mp, start_point, graph_degree, beam,
+                   max_iterations, min_iterations, hash_bit, hash_reset_interval, relaxant, metric, graph,
+                   counters=None, stream=None):
+    check(lib().glide_hip_build_boundary(_ptr(reorder_data), u32(num), u32(reorder_num), u32(dim), _ptr(knn_graph),
+                                         u32(knn_degree), _ptr(mp), u32(start_point), u32(graph_degree), u32(beam),
+                                         u32(max_iterations), u32(min_iterations), u32(hash_bit),
+                                         u32(hash_reset_interval), f32(relaxant), C.c_int(metric), _ptr(graph),
+                                         _ptr(counters), vp(stream)), "glide_hip_build_boundary")
+
+
+def reverse_edges_workspace_bytes(num, graph_degree):
+    f = lib().glide_hip_reverse_edges_workspace_bytes
+    f.restype = C.c_size_t
+    return int(f(u32(num), u32(graph_degree)))
+
+
+def reverse_edges(graph, num, graph_degree, reverse_graph, reverse_counts, workspace, workspace_bytes, stream=None):
+    check(lib().glide_hip_reverse_edges(_ptr(graph), u32(num), u32(graph_degree), _ptr(reverse_graph),
+                                        _ptr(reverse_counts), _ptr(workspace), C.c_size_t(workspace_bytes),
+                                        vp(stream)), "glide_hip_reverse_edges")
+
+
+def insert_reverse(graph, reverse_graph, reverse_counts, num, graph_degree, stream=None):
+    check(lib().glide_hip_insert_reverse(_ptr(graph), _ptr(reverse_graph), _ptr(reverse_counts), u32(num),
+                                         u32(graph_degree), vp(stream)), "glide_hip_insert_reverse")
+
+
+def refine(data, num, dim, graph_in, graph_out, graph_degree, centroids, centroid_num, start_points, beam,
+           max_iterations, min_iterations, hash_bit, hash_reset_interval, relaxant, metric, counters=None,
+           stream=None):
+    check(lib().glide_hip_refine(_ptr(data), u32(num), u32(dim), _ptr(graph_in), _ptr(graph_out), u32(graph_degree),
+                                 _ptr(centroids), u32(centroid_num), _ptr(start_points), u32(beam),
+                                 u32(max_iterations), u32(min_iterations), u32(hash_bit), u32(hash_reset_interval),
+                                 f32(relaxant), C.c_int(metric), _ptr(counters), vp(stream)), "glide_hip_refine")

@@ -31,6 +31,33 @@ struct BeamLds {  // per-wave LDS (the hash table follows, 1 << hash_bit words)
 
 __device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
 
+// Distances from `ref` to `count` listed rows, two rows per step (one per 32-lane half), U steps in flight.
+// id_of(idx) -> row id of list entry idx; out(idx, dist) is called by one lane per scored row.
+template <int DIMV, class IdFn, class OutFn>
+__device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float* data, uint32_t dim, int metric,
+                                           uint32_t first, uint32_t count, int lane, IdFn id_of, OutFn out) {
+    const int half = lane >> 5, t = lane & 31;
+    constexpr int U = DIMV == 1 ? 4 : (DIMV == 2 ? 2 : 1);
+    for (uint32_t base = first; base < count; base += 2 * U) {
+        RowRegs<DIMV> rows[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t idx = base + 2 * u + half;
+            if (idx < count) {
+                load_row<DIMV>(rows[u], data + static_cast<size_t>(id_of(idx)) * dim, dim, t);
+            } else {
+                rows[u] = ref;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t idx = base + 2 * u + half;
+            const float d = finish_distance(half_wave_sum(partial_sqdist<DIMV>(ref, rows[u])), metric);
+            if (t == 0 && idx < count) out(idx, d);
+        }
+    }
+}
+
 template <int MAX_CAND, int MAX_BEAM, int DIMV>
 struct Beam {
     static constexpr int NB = MAX_BEAM / 64;
@@ -79,30 +106,10 @@ struct Beam {
         }
         wave_sync();
         cnt.rows_scored += nv;
-        const int half = lane >> 5, t = lane & 31;
-        constexpr int U = DIMV == 1 ? 4 : (DIMV == 2 ? 2 : 1);  // row pairs in flight per trip
-        for (uint32_t base = 0; base < nv; base += 2 * U) {
-            RowRegs<DIMV> rows[U];
-            uint32_t slot[U];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const uint32_t idx = base + 2 * u + half;
-                const bool active = idx < nv;
-                slot[u] = active ? lds->vlist[idx] : kInvalid;
-                const uint32_t id = active ? lds->cand_id[slot[u]] : 0u;
-                const float* row = data + static_cast<size_t>(id) * p.dim;
-                if (active) {
-                    load_row<DIMV>(rows[u], row, p.dim, t);
-                } else {
-                    rows[u] = q;
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const float d = finish_distance(half_wave_sum(partial_sqdist<DIMV>(q, rows[u])), p.metric);
-                if (t == 0 && slot[u] != kInvalid) lds->cand_dist[slot[u]] = d;
-            }
-        }
+        BeamLds<MAX_CAND>* l = lds;
+        score_list<DIMV>(q, data, p.dim, p.metric, 0, nv, lane,
+                         [l](uint32_t idx) { return l->cand_id[l->vlist[idx]]; },
+                         [l](uint32_t idx, float d) { l->cand_dist[l->vlist[idx]] = d; });
         wave_sync();
     }
 

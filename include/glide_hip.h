@@ -68,6 +68,59 @@ int glide_hip_search(const float *data, uint32_t num, uint32_t dim, const uint32
                      uint32_t hash_reset_interval, int metric, uint32_t *result_ids, float *result_dists,
                      unsigned long long *counters, void *stream);
 
+/* ---- graph construction (subsystem 3) ----------------------------------------------------------------------
+ * All kernels give one point to one wavefront.  Limits as for glide_hip_search (knn_degree, graph_degree <= 128,
+ * beam <= 256, dim % 4 == 0, dim <= 1024).  `counters` as in glide_hip_search (prune distances count as rows). */
+
+/* Replaces build_kernel (graph_kernel.cuh:249-316) as launched by GLIDE::subgraph_build_and_merge
+ * (glide_impl.cuh:77-147): for every reorder id p < num, beam search on the partition-local kNN graph from the
+ * partition's start point, relaxed-RNG prune to graph_degree, row graph[map[p]] written in original ids
+ * (0xffffffff = empty).  knn_graph is reorder_num x knn_degree with partition-local ids; start_points holds one
+ * partition-local id per segment. */
+int glide_hip_build_subgraph(const float *reorder_data, uint32_t num, uint32_t dim, const uint32_t *knn_graph,
+                             uint32_t knn_degree, const uint32_t *map, const uint32_t *segment_starts,
+                             const uint32_t *segment_lengths, uint32_t segment_num, const uint32_t *start_points,
+                             uint32_t graph_degree, uint32_t beam, uint32_t max_iterations,
+                             uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
+                             float relaxant, int metric, uint32_t *graph, unsigned long long *counters,
+                             void *stream);
+
+/* Replaces build_boundary_kernel + map_to_graph_boundary (graph_kernel.cuh:318-376, 160-247; launch
+ * glide_impl.cuh:149-191): the same on the boundary segment [num, reorder_num), merging each result into the
+ * row of the original point.  Must run after glide_hip_build_subgraph on the same stream.  start_point is the
+ * boundary segment's local start id. */
+int glide_hip_build_boundary(const float *reorder_data, uint32_t num, uint32_t reorder_num, uint32_t dim,
+                             const uint32_t *knn_graph, uint32_t knn_degree, const uint32_t *map,
+                             uint32_t start_point, uint32_t graph_degree, uint32_t beam, uint32_t max_iterations,
+                             uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
+                             float relaxant, int metric, uint32_t *graph, unsigned long long *counters,
+                             void *stream);
+
+/* Replaces the graph_degree launches of reverse_graph_kernel (graph_kernel.cuh:378-414; glide_impl.cuh:194-233).
+ * reverse_graph (num x graph_degree) receives, for every node, the sources of edges pointing at it that it does
+ * not point back to, capped at graph_degree; reverse_counts the uncapped count.  Where the reference keeps
+ * whichever sources win its atomics, the list here is the first graph_degree in (column, source) order, i.e.
+ * what a sequential sweep produces.  workspace: glide_hip_reverse_edges_workspace_bytes(), 8-byte aligned. */
+size_t glide_hip_reverse_edges_workspace_bytes(uint32_t num, uint32_t graph_degree);
+int glide_hip_reverse_edges(const uint32_t *graph, uint32_t num, uint32_t graph_degree, uint32_t *reverse_graph,
+                            uint32_t *reverse_counts, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Replaces insert_reverse_kernel (graph_kernel.cuh:416-453; glide_impl.cuh:235-256): the empty slots of each
+ * row take, in order, the first entries of its reverse list. */
+int glide_hip_insert_reverse(uint32_t *graph, const uint32_t *reverse_graph, const uint32_t *reverse_counts,
+                             uint32_t num, uint32_t graph_degree, void *stream);
+
+/* Replaces refine_kernel (graph_kernel.cuh:580-673; GLIDE::refine glide_impl.cuh:258-316): rows with empty
+ * slots search the whole graph from the nearest centroid's start point and fill the slots after a prune that
+ * skips existing neighbours.  Reads graph_in, writes every row of graph_out (graph_in != graph_out): the
+ * reference refines in place while other blocks still traverse the rows; here all searches see the
+ * pre-refinement graph. */
+int glide_hip_refine(const float *data, uint32_t num, uint32_t dim, const uint32_t *graph_in, uint32_t *graph_out,
+                     uint32_t graph_degree, const float *centroids, uint32_t centroid_num,
+                     const uint32_t *start_points, uint32_t beam, uint32_t max_iterations,
+                     uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant,
+                     int metric, unsigned long long *counters, void *stream);
+
 /* ---- test hooks for the device primitives (subsystems 5, 6 and the hash set) ------------------------------ */
 /* compute_similarity_warp (distance.cuh:9-27): out[i] = dist(a[i], b[i]) for n row pairs */
 int glide_hip_distance_batch(const float *a, const float *b, uint32_t n, uint32_t dim, int metric, float *out,
