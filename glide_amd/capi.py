@@ -225,3 +225,41 @@ def refine(data, num, dim, graph_in, graph_out, graph_degree, centroids, centroi
                                  _ptr(centroids), u32(centroid_num), _ptr(start_points), u32(beam),
                                  u32(max_iterations), u32(min_iterations), u32(hash_bit), u32(hash_reset_interval),
                                  f32(relaxant), C.c_int(metric), _ptr(counters), vp(stream)), "glide_hip_refine")
+
+
+def _size_fn(name):
+    f = getattr(lib(), name)
+    f.restype = C.c_size_t
+    return f
+
+
+def partition_assign_workspace_bytes(num, centroid_num):
+    return int(_size_fn("glide_hip_partition_assign_workspace_bytes")(u32(num), u32(centroid_num)))
+
+
+def partition_assign(data, num, dim, centroids, centroid_num, boundary_factor, metric, segment_indexes,
+                     segment_lengths, nearest_dists, workspace, workspace_bytes, stream=None):
+    check(lib().glide_hip_partition_assign(_ptr(data), u32(num), u32(dim), _ptr(centroids), u32(centroid_num),
+                                           f32(boundary_factor), C.c_int(metric), _ptr(segment_indexes),
+                                           _ptr(segment_lengths), _ptr(nearest_dists), _ptr(workspace),
+                                           C.c_size_t(workspace_bytes), vp(stream)), "glide_hip_partition_assign")
+
+
+def reorder(data, num, dim, segment_indexes, segment_starts, reorder_data, mp, stream=None):
+    check(lib().glide_hip_reorder(_ptr(data), u32(num), u32(dim), _ptr(segment_indexes), _ptr(segment_starts),
+                                  _ptr(reorder_data), _ptr(mp), vp(stream)), "glide_hip_reorder")
+
+
+def sample_rows(data, dim, sample_ids, sample_num, sample, stream=None):
+    check(lib().glide_hip_sample_rows(_ptr(data), u32(dim), _ptr(sample_ids), u32(sample_num), _ptr(sample),
+                                      vp(stream)), "glide_hip_sample_rows")
+
+
+def kmeans_workspace_bytes(cluster_num, dim):
+    return int(_size_fn("glide_hip_kmeans_workspace_bytes")(u32(cluster_num), u32(dim)))
+
+
+def kmeans_fit(sample, sample_num, dim, cluster_num, iterations, centroids, workspace, workspace_bytes, stream=None):
+    check(lib().glide_hip_kmeans_fit(_ptr(sample), u32(sample_num), u32(dim), u32(cluster_num), u32(iterations),
+                                     _ptr(centroids), _ptr(workspace), C.c_size_t(workspace_bytes), vp(stream)),
+          "glide_hip_kmeans_fit")

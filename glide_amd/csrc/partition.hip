@@ -1,0 +1,419 @@
+// Locality partitioning: point -> centroid assignment (fp32 MFMA tile + norm-trick ranking, exact rescoring of
+// the best few), stable slot numbering, row reordering, row sampling and a small Lloyd k-means.
+// Reference: define_partition_kernel (partition_kernel.cuh:22-66), reorder_kernel (:68-100), sample_kernel
+// (:7-20), host sequencing partition.cuh:8-193.
+#include "common.hpp"
+#include "host_util.hpp"
+
+namespace glide {
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int kTilePoints = 128;   // points per workgroup (4 wavefronts x 32)
+constexpr int kChunk = 32;         // dims staged per step
+constexpr int kLdsStride = 36;     // floats per staged row (32 + 4 pad keeps 16-byte alignment, spreads banks)
+constexpr int kTop = 4;            // candidates kept from the ranking pass and rescored exactly
+
+struct AssignArgs {
+    const float* data;
+    const float* centroids;
+    const float* centroid_norms;   // ||c||^2, fp32
+    uint32_t* segment_indexes;     // num x 3: segment, (slot filled later), boundary flag as 0 / 0xffffffff
+    uint32_t* tile_hist;           // tiles x (C + 1)
+    float* nearest_dists;          // num x 2 or null
+    uint32_t num, dim, centroid_num;
+    float boundary_factor;
+    int metric;
+};
+
+// exact distance of one point row to one centroid, one 32-lane half per pair (same arithmetic as the search kernels)
+__device__ __forceinline__ float exact_distance_half(const float* x, const float* c, uint32_t dim, int t) {
+    float acc = 0.f;
+    for (uint32_t d0 = t * 4; d0 < dim; d0 += 128) {
+        const float4 a = *reinterpret_cast<const float4*>(x + d0);
+        const float4 b = *reinterpret_cast<const float4*>(c + d0);
+        float dx = a.x - b.x, dy = a.y - b.y, dz = a.z - b.z, dw = a.w - b.w;
+        acc = fmaf(dx, dx, acc);
+        acc = fmaf(dy, dy, acc);
+        acc = fmaf(dz, dz, acc);
+        acc = fmaf(dw, dw, acc);
+    }
+    return half_wave_sum(acc);
+}
+
+// CB = number of 32-centroid column blocks held in accumulators (centroid_num <= 32*CB)
+template <int CB>
+__global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
+    extern __shared__ __align__(16) float smem[];
+    float* cent_tile = smem;                                   // [32*CB][kLdsStride]
+    float* x_tile = cent_tile + 32 * CB * kLdsStride;          // [4 waves][32][kLdsStride]
+    float* score_tile = x_tile + 4 * 32 * kLdsStride;          // [4 waves][32][33]
+    uint32_t* hist = reinterpret_cast<uint32_t*>(score_tile + 4 * 32 * 33);  // [C + 1]
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int half = lane >> 5, t = lane & 31;
+    const uint32_t tile_base = blockIdx.x * kTilePoints;
+    const uint32_t wave_base = tile_base + wave * 32;
+    float* xw = x_tile + wave * 32 * kLdsStride;
+    float* sw = score_tile + wave * 32 * 33;
+
+    for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256) hist[i] = 0;
+
+    float16v acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[cb][r] = 0.f;
+
+    for (uint32_t k0 = 0; k0 < a.dim; k0 += kChunk) {
+        __syncthreads();
+        // centroid chunk: 8 lanes x float4 per row
+        for (uint32_t idx = threadIdx.x; idx < 32u * CB * 8; idx += 256) {
+            const uint32_t row = idx >> 3, q = idx & 7;
+            const uint32_t d0 = k0 + q * 4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row < a.centroid_num && d0 < a.dim) v = *reinterpret_cast<const float4*>(a.centroids + static_cast<size_t>(row) * a.dim + d0);
+            *reinterpret_cast<float4*>(cent_tile + row * kLdsStride + q * 4) = v;
+        }
+        // this wave's 32 points
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const uint32_t row = it * 8 + (lane >> 3), q = lane & 7;
+            const uint32_t p = wave_base + row, d0 = k0 + q * 4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (p < a.num && d0 < a.dim) v = *reinterpret_cast<const float4*>(a.data + static_cast<size_t>(p) * a.dim + d0);
+            *reinterpret_cast<float4*>(xw + row * kLdsStride + q * 4) = v;
+        }
+        __syncthreads();
+        // v_mfma_f32_32x32x2_f32: lane supplies A[i = lane%32][k-slot = lane/32] and B[k-slot][j = lane%32].
+        // A k-slot pair is fed from one float4 per half (dims kk+4*half .. +3), component by component.
+#pragma unroll
+        for (int kk = 0; kk < kChunk; kk += 8) {
+            const float4 av = *reinterpret_cast<const float4*>(xw + t * kLdsStride + kk + 4 * half);
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++) {
+                const float4 bv = *reinterpret_cast<const float4*>(cent_tile + (cb * 32 + t) * kLdsStride + kk + 4 * half);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc[cb], 0, 0, 0);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc[cb], 0, 0, 0);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc[cb], 0, 0, 0);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc[cb], 0, 0, 0);
+            }
+        }
+    }
+
+    // ranking epilogue: score = ||c||^2 - 2 x.c (the ||x||^2 term is constant per point); lane i < 32 keeps the
+    // kTop smallest scores of point i
+    float best_s[kTop];
+    uint32_t best_c[kTop];
+#pragma unroll
+    for (int k = 0; k < kTop; k++) {
+        best_s[k] = FLT_MAX;
+        best_c[k] = kInvalid;
+    }
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        const uint32_t j = cb * 32 + t;
+        const float cn = j < a.centroid_num ? a.centroid_norms[j] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int i = 8 * (r / 4) + 4 * half + (r % 4);   // accumulator layout of the 32x32 tile
+            sw[i * 33 + t] = j < a.centroid_num ? cn - 2.f * acc[cb][r] : FLT_MAX;
+        }
+        __syncthreads();
+        if (lane < 32) {
+            for (int jj = 0; jj < 32; jj++) {
+                float s = sw[lane * 33 + jj];
+                uint32_t c = cb * 32 + jj;
+#pragma unroll
+                for (int k = 0; k < kTop; k++) {
+                    if (s < best_s[k]) {
+                        const float ts = best_s[k];
+                        const uint32_t tc = best_c[k];
+                        best_s[k] = s;
+                        best_c[k] = c;
+                        s = ts;
+                        c = tc;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // exact rescoring of the kept candidates; lanes 0..31 own the points, halves do the row pairs
+    float d0 = FLT_MAX, d1 = FLT_MAX;
+    uint32_t c0 = kInvalid, c1 = kInvalid;
+    for (int i = 0; i < 32; i++) {
+        const uint32_t p = wave_base + i;
+        if (p >= a.num) break;   // wave-uniform
+        const float* x = a.data + static_cast<size_t>(p) * a.dim;
+        float dd[kTop];
+        uint32_t cc[kTop];
+#pragma unroll
+        for (int k = 0; k < kTop; k += 2) {
+            const uint32_t ca = read_lane(best_c[k], i), cb2 = read_lane(best_c[k + 1], i);
+            const uint32_t mine = half ? cb2 : ca;
+            const float sq = exact_distance_half(x, a.centroids + static_cast<size_t>(mine != kInvalid ? mine : 0u) * a.dim, a.dim, t);
+            const float da = read_lane(sq, 0), db = read_lane(sq, 32);
+            dd[k] = ca != kInvalid ? finish_distance(da, a.metric) : FLT_MAX;
+            dd[k + 1] = cb2 != kInvalid ? finish_distance(db, a.metric) : FLT_MAX;
+            cc[k] = ca;
+            cc[k + 1] = cb2;
+        }
+        // smallest two by (distance, centroid id)
+        float m0 = FLT_MAX, m1 = FLT_MAX;
+        uint32_t i0 = kInvalid, i1 = kInvalid;
+#pragma unroll
+        for (int k = 0; k < kTop; k++) {
+            const bool lt0 = dd[k] < m0 || (dd[k] == m0 && cc[k] < i0);
+            const bool lt1 = dd[k] < m1 || (dd[k] == m1 && cc[k] < i1);
+            if (lt0) {
+                m1 = m0; i1 = i0;
+                m0 = dd[k]; i0 = cc[k];
+            } else if (lt1) {
+                m1 = dd[k]; i1 = cc[k];
+            }
+        }
+        if (lane == i) {
+            d0 = m0; d1 = m1; c0 = i0; c1 = i1;
+        }
+    }
+    (void) c1;
+
+    const uint32_t p = wave_base + lane;
+    if (lane < 32 && p < a.num) {
+        // reference partition_kernel.cuh:55-64: boundary iff a second centroid exists and d(2)/d(1) <= factor
+        const bool boundary = a.centroid_num > 1 && (d1 / d0 <= a.boundary_factor);
+        a.segment_indexes[static_cast<size_t>(p) * 3] = c0;
+        a.segment_indexes[static_cast<size_t>(p) * 3 + 2] = boundary ? 0u : kInvalid;
+        if (a.nearest_dists) {
+            a.nearest_dists[static_cast<size_t>(p) * 2] = d0;
+            a.nearest_dists[static_cast<size_t>(p) * 2 + 1] = d1;
+        }
+        atomicAdd(&hist[c0], 1u);
+        if (boundary) atomicAdd(&hist[a.centroid_num], 1u);
+    }
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256)
+        a.tile_hist[static_cast<size_t>(blockIdx.x) * (a.centroid_num + 1) + i] = hist[i];
+}
+
+// exclusive scan over tiles, one workgroup per bin; also emits the bin totals (segment lengths)
+__global__ __launch_bounds__(256) void tile_scan_kernel(uint32_t* tile_hist, uint32_t tiles, uint32_t bins, uint32_t* totals) {
+    __shared__ uint32_t partial[256];
+    const uint32_t bin = blockIdx.x;
+    const uint32_t per = ceil_div(tiles, 256);
+    const uint32_t begin = threadIdx.x * per, end = begin + per < tiles ? begin + per : tiles;
+    uint32_t sum = 0;
+    for (uint32_t i = begin; i < end; i++) sum += tile_hist[static_cast<size_t>(i) * bins + bin];
+    partial[threadIdx.x] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t run = 0;
+        for (int i = 0; i < 256; i++) {
+            const uint32_t v = partial[i];
+            partial[i] = run;
+            run += v;
+        }
+        totals[bin] = run;
+    }
+    __syncthreads();
+    uint32_t run = partial[threadIdx.x];
+    for (uint32_t i = begin; i < end; i++) {
+        const uint32_t v = tile_hist[static_cast<size_t>(i) * bins + bin];
+        tile_hist[static_cast<size_t>(i) * bins + bin] = run;
+        run += v;
+    }
+}
+
+// slot = number of earlier points (in point order) of the same segment; same for the boundary list
+__global__ __launch_bounds__(kTilePoints) void slot_kernel(uint32_t* segment_indexes, const uint32_t* tile_base_counts, uint32_t num,
+                                                           uint32_t centroid_num) {
+    __shared__ uint32_t seg[kTilePoints];
+    __shared__ uint32_t bnd[kTilePoints];
+    const uint32_t p = blockIdx.x * kTilePoints + threadIdx.x;
+    const bool live = p < num;
+    const uint32_t my_seg = live ? segment_indexes[static_cast<size_t>(p) * 3] : kInvalid;
+    const uint32_t my_b = live ? segment_indexes[static_cast<size_t>(p) * 3 + 2] : kInvalid;
+    seg[threadIdx.x] = my_seg;
+    bnd[threadIdx.x] = my_b;
+    __syncthreads();
+    if (!live) return;
+    uint32_t rank = 0, brank = 0;
+    for (uint32_t j = 0; j < threadIdx.x; j++) {
+        rank += seg[j] == my_seg;
+        brank += bnd[j] != kInvalid;
+    }
+    const uint32_t* base = tile_base_counts + static_cast<size_t>(blockIdx.x) * (centroid_num + 1);
+    segment_indexes[static_cast<size_t>(p) * 3 + 1] = base[my_seg] + rank;
+    if (my_b != kInvalid) segment_indexes[static_cast<size_t>(p) * 3 + 2] = base[centroid_num] + brank;
+}
+
+// reorder_kernel (partition_kernel.cuh:68-100): one wavefront per point
+__global__ __launch_bounds__(256) void reorder_kernel(const float* data, float* reorder_data, const uint32_t* segment_indexes,
+                                                      uint32_t* map, const uint32_t* segment_starts, uint32_t num, uint32_t dim) {
+    const int lane = lane_id();
+    const uint32_t p = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (p >= num) return;
+    const uint32_t seg = segment_indexes[static_cast<size_t>(p) * 3];
+    const uint32_t slot = segment_indexes[static_cast<size_t>(p) * 3 + 1];
+    const uint32_t bslot = segment_indexes[static_cast<size_t>(p) * 3 + 2];
+    const uint32_t rid = segment_starts[seg] + slot;
+    const float* src = data + static_cast<size_t>(p) * dim;
+    float* dst = reorder_data + static_cast<size_t>(rid) * dim;
+    float* bdst = bslot != kInvalid ? reorder_data + static_cast<size_t>(num + bslot) * dim : nullptr;
+    for (uint32_t d0 = lane * 4; d0 < dim; d0 += 256) {
+        const float4 v = *reinterpret_cast<const float4*>(src + d0);
+        *reinterpret_cast<float4*>(dst + d0) = v;
+        if (bdst) *reinterpret_cast<float4*>(bdst + d0) = v;
+    }
+    if (lane == 0) {
+        map[rid] = p;
+        if (bdst) map[num + bslot] = p;
+    }
+}
+
+// sample_kernel (partition_kernel.cuh:7-20)
+__global__ __launch_bounds__(256) void sample_rows_kernel(const float* data, float* sample, const uint32_t* ids, uint32_t count, uint32_t dim) {
+    const int lane = lane_id();
+    const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= count) return;
+    const float* src = data + static_cast<size_t>(ids[i]) * dim;
+    float* dst = sample + static_cast<size_t>(i) * dim;
+    for (uint32_t d0 = lane * 4; d0 < dim; d0 += 256) *reinterpret_cast<float4*>(dst + d0) = *reinterpret_cast<const float4*>(src + d0);
+}
+
+__global__ __launch_bounds__(256) void row_norms_kernel(const float* rows, uint32_t count, uint32_t dim, float* norms) {
+    const int lane = lane_id();
+    const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= count) return;
+    float acc = 0.f;
+    for (uint32_t d = lane; d < dim; d += 64) {
+        const float v = rows[static_cast<size_t>(i) * dim + d];
+        acc = fmaf(v, v, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) norms[i] = acc;
+}
+
+// ---- Lloyd k-means on a sample (stand-in for cuvs::cluster::kmeans::fit, reference partition.cuh:48-54) ----
+// one wavefront per sample point: nearest centroid by direct distances, then atomic accumulation
+__global__ __launch_bounds__(256) void kmeans_accumulate_kernel(const float* sample, uint32_t n, uint32_t dim, const float* centroids,
+                                                                uint32_t k, float* sums, uint32_t* counts) {
+    const int lane = lane_id();
+    const int half = lane >> 5, t = lane & 31;
+    const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= n) return;
+    const float* x = sample + static_cast<size_t>(i) * dim;
+    float best = FLT_MAX;
+    uint32_t bc = 0;
+    for (uint32_t c0 = 0; c0 < k; c0 += 2) {
+        const uint32_t c = c0 + half < k ? c0 + half : c0;
+        const float sq = exact_distance_half(x, centroids + static_cast<size_t>(c) * dim, dim, t);
+        const float da = read_lane(sq, 0), db = read_lane(sq, 32);
+        if (da < best) { best = da; bc = c0; }
+        if (c0 + 1 < k && db < best) { best = db; bc = c0 + 1; }
+    }
+    for (uint32_t d = lane; d < dim; d += 64) atomicAdd(&sums[static_cast<size_t>(bc) * dim + d], x[d]);
+    if (lane == 0) atomicAdd(&counts[bc], 1u);
+}
+
+__global__ void kmeans_update_kernel(float* centroids, const float* sums, const uint32_t* counts, uint32_t k, uint32_t dim) {
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= k * dim) return;
+    const uint32_t c = idx / dim;
+    if (counts[c]) centroids[idx] = sums[idx] / static_cast<float>(counts[c]);   // an empty cluster keeps its centroid
+}
+
+size_t assign_lds_bytes(int cb, uint32_t centroid_num) {
+    return (static_cast<size_t>(32) * cb * kLdsStride + 4 * 32 * kLdsStride + 4 * 32 * 33) * sizeof(float) + (centroid_num + 1) * sizeof(uint32_t);
+}
+
+}  // namespace glide
+
+using namespace glide;
+
+extern "C" {
+
+size_t glide_hip_partition_assign_workspace_bytes(uint32_t num, uint32_t centroid_num) {
+    const size_t tiles = ceil_div(num, kTilePoints);
+    return tiles * (centroid_num + 1) * 4 + static_cast<size_t>(centroid_num) * 4 + 256;
+}
+
+int glide_hip_partition_assign(const float* data, uint32_t num, uint32_t dim, const float* centroids, uint32_t centroid_num,
+                               float boundary_factor, int metric, uint32_t* segment_indexes, uint32_t* segment_lengths,
+                               float* nearest_dists, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!data || !centroids || !segment_indexes || !segment_lengths || !workspace) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim == 0 || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
+    if (centroid_num > 256 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // reference buckets: kernel_config.cuh:224-234
+    if (workspace_bytes < glide_hip_partition_assign_workspace_bytes(num, centroid_num)) return GLIDE_ERR_BAD_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    if (num == 0) return glide_hip_fill_u32(segment_lengths, 0u, centroid_num + 1, stream);
+    const uint32_t tiles = ceil_div(num, kTilePoints);
+    float* norms = static_cast<float*>(workspace);
+    uint32_t* tile_hist = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(workspace) + ((static_cast<size_t>(centroid_num) * 4 + 255) / 256) * 256);
+    hipLaunchKernelGGL(row_norms_kernel, dim3(ceil_div(centroid_num, 4)), dim3(256), 0, s, centroids, centroid_num, dim, norms);
+    AssignArgs a{data, centroids, norms, segment_indexes, tile_hist, nearest_dists, num, dim, centroid_num, boundary_factor, metric};
+    const int cb = centroid_num <= 32 ? 1 : centroid_num <= 64 ? 2 : centroid_num <= 128 ? 4 : 8;
+    const size_t lds = assign_lds_bytes(cb, centroid_num);
+    if (lds > 64 * 1024) {
+        GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&assign_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          static_cast<int>(lds)));
+    }
+    switch (cb) {
+        case 1: hipLaunchKernelGGL(assign_kernel<1>, dim3(tiles), dim3(256), lds, s, a); break;
+        case 2: hipLaunchKernelGGL(assign_kernel<2>, dim3(tiles), dim3(256), lds, s, a); break;
+        case 4: hipLaunchKernelGGL(assign_kernel<4>, dim3(tiles), dim3(256), lds, s, a); break;
+        default: hipLaunchKernelGGL(assign_kernel<8>, dim3(tiles), dim3(256), lds, s, a); break;
+    }
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(256), 0, s, tile_hist, tiles, centroid_num + 1, segment_lengths);
+    hipLaunchKernelGGL(slot_kernel, dim3(tiles), dim3(kTilePoints), 0, s, segment_indexes, tile_hist, num, centroid_num);
+    return launch_status();
+}
+
+int glide_hip_reorder(const float* data, uint32_t num, uint32_t dim, const uint32_t* segment_indexes, const uint32_t* segment_starts,
+                      float* reorder_data, uint32_t* map, void* stream) {
+    if (!data || !segment_indexes || !segment_starts || !reorder_data || !map || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    if (num == 0) return GLIDE_OK;
+    hipLaunchKernelGGL(reorder_kernel, dim3(ceil_div(num, 4)), dim3(256), 0, as_stream(stream), data, reorder_data, segment_indexes, map,
+                       segment_starts, num, dim);
+    return launch_status();
+}
+
+int glide_hip_sample_rows(const float* data, uint32_t dim, const uint32_t* sample_ids, uint32_t sample_num, float* sample, void* stream) {
+    if (!data || !sample_ids || !sample || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    if (sample_num == 0) return GLIDE_OK;
+    hipLaunchKernelGGL(sample_rows_kernel, dim3(ceil_div(sample_num, 4)), dim3(256), 0, as_stream(stream), data, sample, sample_ids,
+                       sample_num, dim);
+    return launch_status();
+}
+
+size_t glide_hip_kmeans_workspace_bytes(uint32_t cluster_num, uint32_t dim) {
+    return static_cast<size_t>(cluster_num) * dim * 4 + static_cast<size_t>(cluster_num) * 4 + 256;
+}
+
+int glide_hip_kmeans_fit(const float* sample, uint32_t sample_num, uint32_t dim, uint32_t cluster_num, uint32_t iterations,
+                         float* centroids, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!sample || !centroids || !workspace || dim == 0 || cluster_num == 0 || sample_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    if (workspace_bytes < glide_hip_kmeans_workspace_bytes(cluster_num, dim)) return GLIDE_ERR_BAD_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    float* sums = static_cast<float*>(workspace);
+    uint32_t* counts = reinterpret_cast<uint32_t*>(sums + static_cast<size_t>(cluster_num) * dim);
+    const size_t words = static_cast<size_t>(cluster_num) * dim + cluster_num;
+    for (uint32_t it = 0; it < iterations; it++) {
+        int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(sums), 0u, words, stream);
+        if (rc != GLIDE_OK) return rc;
+        hipLaunchKernelGGL(kmeans_accumulate_kernel, dim3(ceil_div(sample_num, 4)), dim3(256), 0, s, sample, sample_num, dim, centroids,
+                           cluster_num, sums, counts);
+        hipLaunchKernelGGL(kmeans_update_kernel, dim3(ceil_div(cluster_num * dim, 256)), dim3(256), 0, s, centroids, sums, counts,
+                           cluster_num, dim);
+    }
+    return launch_status();
+}
+
+}  // extern "C"

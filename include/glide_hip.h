@@ -7,8 +7,8 @@
  * Each declaration cites the interface of the reference implementation (owlet-hub/GLIDE, paths relative to its
  * src/ directory) that it replaces.
  *
- * Unless stated otherwise the kernels allocate nothing; entry points that need scratch memory say so and
- * allocate/free it with hipMallocAsync/hipFreeAsync on `stream`.
+ * No entry point allocates device memory: those that need scratch take a caller-provided `workspace` whose
+ * size a companion *_workspace_bytes() function reports.
  */
 #ifndef GLIDE_HIP_H
 #define GLIDE_HIP_H
@@ -67,6 +67,38 @@ int glide_hip_search(const float *data, uint32_t num, uint32_t dim, const uint32
                      uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
                      uint32_t hash_reset_interval, int metric, uint32_t *result_ids, float *result_dists,
                      unsigned long long *counters, void *stream);
+
+/* ---- locality partitioning (subsystem 1) --------------------------------------------------------------------
+ * Replaces define_partition_kernel (partition_kernel.cuh:22-66) + the host prefix sum of define_partition
+ * (partition.cuh:61-116).  Distances to all centroids are ranked with an fp32 MFMA tile (||c||^2 - 2 x.c), the
+ * best four are re-evaluated with the direct sum of squared differences, and the reference's rule is applied to
+ * those: segment = nearest centroid; boundary iff centroid_num > 1 and d(2nd)/d(1st) <= boundary_factor (sqrt
+ * distances for Euclidean).  segment_indexes is num x 3: {segment, slot in segment, boundary slot or
+ * 0xffffffff}.  Slots are numbered in point order (the reference numbers them in atomicAdd arrival order).
+ * segment_lengths receives centroid_num + 1 counts, the last one being the boundary list.  nearest_dists
+ * (nullable, num x 2) receives the two smallest distances.  Limits: centroid_num <= 256, dim % 4 == 0. */
+size_t glide_hip_partition_assign_workspace_bytes(uint32_t num, uint32_t centroid_num);
+int glide_hip_partition_assign(const float *data, uint32_t num, uint32_t dim, const float *centroids,
+                               uint32_t centroid_num, float boundary_factor, int metric,
+                               uint32_t *segment_indexes, uint32_t *segment_lengths, float *nearest_dists,
+                               void *workspace, size_t workspace_bytes, void *stream);
+
+/* Replaces reorder_kernel (partition_kernel.cuh:68-100; partition.cuh:118-157): row p goes to
+ * segment_starts[segment] + slot, boundary copies to num + boundary slot; map[reorder id] = p.
+ * segment_starts: centroid_num + 1 device words (exclusive prefix sum of segment_lengths). */
+int glide_hip_reorder(const float *data, uint32_t num, uint32_t dim, const uint32_t *segment_indexes,
+                      const uint32_t *segment_starts, float *reorder_data, uint32_t *map, void *stream);
+
+/* Replaces sample_kernel (partition_kernel.cuh:7-20; partition.cuh:31-45): sample[i] = data[sample_ids[i]]. */
+int glide_hip_sample_rows(const float *data, uint32_t dim, const uint32_t *sample_ids, uint32_t sample_num,
+                          float *sample, void *stream);
+
+/* Stands in for cuvs::cluster::kmeans::fit (third-party; call site partition.cuh:48-54): `iterations` Lloyd
+ * steps from the centroids passed in (the caller seeds them, e.g. with sampled rows). */
+size_t glide_hip_kmeans_workspace_bytes(uint32_t cluster_num, uint32_t dim);
+int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim, uint32_t cluster_num,
+                         uint32_t iterations, float *centroids, void *workspace, size_t workspace_bytes,
+                         void *stream);
 
 /* ---- graph construction (subsystem 3) ----------------------------------------------------------------------
  * All kernels give one point to one wavefront.  Limits as for glide_hip_search (knn_degree, graph_degree <= 128,
