@@ -263,3 +263,15 @@ def kmeans_fit(sample, sample_num, dim, cluster_num, iterations, centroids, work
     check(lib().glide_hip_kmeans_fit(_ptr(sample), u32(sample_num), u32(dim), u32(cluster_num), u32(iterations),
                                      _ptr(centroids), _ptr(workspace), C.c_size_t(workspace_bytes), vp(stream)),
           "glide_hip_kmeans_fit")
+
+
+def nnd_workspace_bytes(reorder_num, dim, knn_degree):
+    return int(_size_fn("glide_hip_nnd_workspace_bytes")(u32(reorder_num), u32(dim), u32(knn_degree)))
+
+
+def nnd_build(reorder_data, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, iterations,
+              seed, knn_graph, workspace, workspace_bytes, stats=None, stream=None):
+    check(lib().glide_hip_nnd_build(_ptr(reorder_data), u32(reorder_num), u32(dim), _ptr(segment_starts),
+                                    _ptr(segment_lengths), u32(segment_num), u32(knn_degree), u32(iterations),
+                                    u32(seed), _ptr(knn_graph), _ptr(workspace), C.c_size_t(workspace_bytes),
+                                    _ptr(stats), vp(stream)), "glide_hip_nnd_build")

@@ -1,0 +1,677 @@
+// NN-descent kNN-graph construction, entirely on the device.
+//
+// Reference: nn_descent.cuh -- preprocess_data_kernel (:445-488), sampling on the host (GnndGraph::sample_graph
+// :1040-1071, sample_graph_new :973-1001), add_rev_edges_kernel (:490-507), local_join_kernel (:668-914),
+// insert_to_global_graph (:509-579), host merge update_graph (:1106-1126) and the shrink step (:1376-1402).
+//
+// What is kept: fp16 rows with fp32 squared norms, <= 32 new + <= 32 old forward samples per node, reverse
+// samples capped at 32, a 64 x 64 distance tile per phase (new x new, new x old) computed on the matrix cores
+// with the norm-trick epilogue, and one offer per row / column (its nearest partner) per phase.
+// What is different: the kNN lists, flags and samples never leave HBM.  Offers are appended to a per-node inbox
+// (one atomic counter per node, no locks, no cross-workgroup read-after-write inside a kernel) and a merge kernel
+// folds each inbox into the node's sorted list with a wave-wide bitonic sort; sampling uses the new/old flag kept
+// in the list instead of a host-side Bloom filter.  All ids are partition-local.
+#include "common.hpp"
+#include "host_util.hpp"
+
+namespace glide {
+
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kSamples = 32;     // NUM_SAMPLES (nn_descent.cuh:391)
+constexpr uint32_t kBi = 64;          // MAX_NUM_BI_SAMPLES (:392)
+constexpr uint32_t kOld = 0x80000000u;  // "old" flag in a list entry (the reference uses the sign bit, :53-72)
+constexpr int kRowHalfs = 128 + 8;    // LDS row stride in halfs for a 128-dim chunk
+constexpr int kDStride = 65;
+
+struct Segments {
+    const uint32_t* starts;
+    const uint32_t* lengths;
+    uint32_t count;
+};
+
+__device__ __forceinline__ void locate(const Segments& s, uint32_t node, uint32_t& start, uint32_t& len) {
+    uint32_t i = 0;
+    for (; i + 1 < s.count; i++)
+        if (node < s.starts[i] + s.lengths[i]) break;
+    start = s.starts[i];
+    len = s.lengths[i];
+}
+
+// ---- prepare: fp32 rows -> fp16 rows (stride dim_pad, zero padded) + squared norms of the fp32 input
+__global__ __launch_bounds__(256) void nnd_prepare_kernel(const float* data, uint32_t num, uint32_t dim, uint32_t dim_pad, _Float16* half_rows,
+                                                          float* norms) {
+    const int lane = lane_id();
+    const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= num) return;
+    float acc = 0.f;
+    for (uint32_t d = lane; d < dim_pad; d += 64) {
+        const float v = d < dim ? data[static_cast<size_t>(i) * dim + d] : 0.f;
+        acc = fmaf(v, v, acc);
+        half_rows[static_cast<size_t>(i) * dim_pad + d] = static_cast<_Float16>(v);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) norms[i] = acc;
+}
+
+// ---- random initial lists (reference init_random_graph :1003-1038 uses shuffled sequences on the host)
+__device__ __forceinline__ uint32_t mix32(uint32_t x) {
+    x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    return x;
+}
+
+__global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, uint32_t num, uint32_t width,
+                                                       Segments segs, uint32_t seed) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t node = idx / width, j = idx % width;
+    if (node >= num) return;
+    uint32_t start, len;
+    locate(segs, node, start, len);
+    const uint32_t local = node - start;
+    // pseudo-random partition-local neighbour, never the node itself; a repeated id in a row is harmless (the
+    // join and the merge both drop repeats)
+    uint32_t id = kInvalid;
+    if (len > 1) {
+        id = mix32(mix32(node + seed * 0x9E3779B9u) ^ (j * 0x85EBCA6Bu + 1u)) % len;
+        if (id == local) id = (id + 1) % len;
+    }
+    list_ids[static_cast<size_t>(node) * width + j] = id;   // new (flag clear)
+    list_dists[static_cast<size_t>(node) * width + j] = FLT_MAX;
+    if (j == 0) inbox_counts[node] = 0;
+}
+
+// ---- sampling: first <= 32 new entries (marked old afterwards) and first <= 32 entries that were already old
+__global__ __launch_bounds__(256) void nnd_sample_kernel(uint32_t* list_ids, uint32_t num, uint32_t width, Segments segs, uint32_t* fwd_new,
+                                                         uint32_t* fwd_old, uint32_t* counts /* num x 4: fwd_new, fwd_old, rev_new, rev_old */) {
+    const int lane = lane_id();
+    const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (node >= num) return;
+    uint32_t start, len;
+    locate(segs, node, start, len);
+    uint32_t nn = 0, no = 0;
+    for (uint32_t base = 0; base < width; base += 64) {
+        const uint32_t j = base + lane;
+        uint32_t e = j < width ? list_ids[static_cast<size_t>(node) * width + j] : kInvalid;
+        const uint32_t id = e & ~kOld;
+        const bool valid = e != kInvalid && id < len;
+        const bool is_new = valid && (e & kOld) == 0;
+        const bool is_old = valid && (e & kOld) != 0;
+        const uint64_t mn = ballot(is_new), mo = ballot(is_old);
+        const uint32_t pn = nn + prefix_count(mn), po = no + prefix_count(mo);
+        if (is_new && pn < kSamples) {
+            fwd_new[static_cast<size_t>(node) * kSamples + pn] = id;
+            list_ids[static_cast<size_t>(node) * width + j] = e | kOld;
+        }
+        if (is_old && po < kSamples) fwd_old[static_cast<size_t>(node) * kSamples + po] = id;
+        nn += __popcll(mn);
+        no += __popcll(mo);
+    }
+    if (lane == 0) {
+        counts[static_cast<size_t>(node) * 4 + 0] = nn < kSamples ? nn : kSamples;
+        counts[static_cast<size_t>(node) * 4 + 1] = no < kSamples ? no : kSamples;
+        counts[static_cast<size_t>(node) * 4 + 2] = 0;
+        counts[static_cast<size_t>(node) * 4 + 3] = 0;
+    }
+}
+
+// ---- reverse samples (add_rev_edges_kernel :490-507): list u appends itself to the reverse list of each sample
+__global__ __launch_bounds__(256) void nnd_reverse_kernel(const uint32_t* fwd_new, const uint32_t* fwd_old, uint32_t* counts, uint32_t* rev_new,
+                                                          uint32_t* rev_old, uint32_t num, Segments segs) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t node = idx / 64, j = idx % 64;
+    if (node >= num) return;
+    uint32_t start, len;
+    locate(segs, node, start, len);
+    const uint32_t which = j / kSamples, k = j % kSamples;   // 0: new, 1: old
+    if (k >= counts[static_cast<size_t>(node) * 4 + which]) return;
+    const uint32_t v = (which ? fwd_old : fwd_new)[static_cast<size_t>(node) * kSamples + k];
+    const uint32_t target = start + v;
+    const uint32_t pos = atomicAdd(&counts[static_cast<size_t>(target) * 4 + 2 + which], 1u);
+    if (pos < kSamples) (which ? rev_old : rev_new)[static_cast<size_t>(target) * kSamples + pos] = node - start;
+}
+
+// ---- local join ---------------------------------------------------------------------------------------------
+struct JoinArgs {
+    const _Float16* half_rows;
+    const float* norms;
+    const uint32_t* fwd_new;
+    const uint32_t* fwd_old;
+    const uint32_t* rev_new;
+    const uint32_t* rev_old;
+    const uint32_t* counts;
+    const float* list_dists;    // thresholds: a node's current worst distance
+    uint32_t* inbox_counts;
+    uint2* inbox;               // num x inbox_cap (dist bits, id)
+    unsigned long long* stats;  // [0] offers emitted, [1] offers dropped by a full inbox (nullable)
+    uint32_t num, dim_pad, width, inbox_cap;
+    Segments segs;
+};
+
+struct JoinLds {
+    _Float16 xn[kBi][kRowHalfs];
+    _Float16 xo[kBi][kRowHalfs];
+    float dist[kBi][kDStride];
+    uint32_t new_ids[kBi], old_ids[kBi];
+    float new_norms[kBi], old_norms[kBi];
+    uint32_t hash_new[128], hash_old[128];
+    uint32_t n_new, n_old;
+};
+
+__device__ __forceinline__ bool lds_set_insert(uint32_t* table, uint32_t key) {   // 128-slot open addressing
+    uint32_t idx = (key * 0x9E3779B1u) >> 25;
+    for (int i = 0; i < 128; i++) {
+        const uint32_t old = atomicCAS(&table[idx], kInvalid, key);
+        if (old == kInvalid) return true;
+        if (old == key) return false;
+        idx = (idx + 1) & 127;
+    }
+    return false;
+}
+
+__device__ __forceinline__ void emit_offer(const JoinArgs& a, uint32_t seg_start, uint32_t seg_len, uint32_t target, uint32_t cand, float d) {
+    if (cand == kInvalid || cand == target || cand >= seg_len || !(d < FLT_MAX)) return;
+    // No filtering against the target's current list: the reference also explores offers that do not enter the
+    // list (they are the "new" samples of the next round, nn_descent.cuh:973-1001).
+    const uint32_t g = seg_start + target;
+    const uint32_t pos = atomicAdd(&a.inbox_counts[g], 1u);
+    if (pos < a.inbox_cap) {
+        a.inbox[static_cast<size_t>(g) * a.inbox_cap + pos] = make_uint2(__float_as_uint(d), cand);
+    }
+}
+
+// A (rows) x B (rows) dot products of a 128-dim chunk for this wave's 32 x 32 quadrant.
+// v_mfma_f32_32x32x8_f16: lane supplies A[i = lane%32][k = 4*(lane/32) .. +3] and B[k = same][j = lane%32].
+__device__ __forceinline__ void mfma_chunk(float16v& acc, const _Float16 (*A)[kRowHalfs], const _Float16 (*B)[kRowHalfs], int rb, int cb, int lane) {
+    const int t = lane & 31, kh = lane >> 5;
+#pragma unroll
+    for (int kk = 0; kk < 128; kk += 8) {
+        const half4v av = *reinterpret_cast<const half4v*>(&A[rb * 32 + t][kk + 4 * kh]);
+        const half4v bv = *reinterpret_cast<const half4v*>(&B[cb * 32 + t][kk + 4 * kh]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x8f16(av, bv, acc, 0, 0, 0);
+    }
+}
+
+__global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    JoinLds& L = *reinterpret_cast<JoinLds*>(smem);
+    const uint32_t node = blockIdx.x;
+    if (node >= a.num) return;
+    const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    uint32_t seg_start, seg_len;
+    locate(a.segs, node, seg_start, seg_len);
+
+    const uint32_t c_fn = a.counts[static_cast<size_t>(node) * 4 + 0], c_fo = a.counts[static_cast<size_t>(node) * 4 + 1];
+    uint32_t c_rn = a.counts[static_cast<size_t>(node) * 4 + 2], c_ro = a.counts[static_cast<size_t>(node) * 4 + 3];
+    c_rn = c_rn < kSamples ? c_rn : kSamples;
+    c_ro = c_ro < kSamples ? c_ro : kSamples;
+    if (c_fn + c_rn == 0) return;
+
+    if (tid < 128) {
+        L.hash_new[tid] = kInvalid;
+        L.hash_old[tid] = kInvalid;
+    }
+    if (tid == 0) {
+        L.n_new = 0;
+        L.n_old = 0;
+    }
+    __syncthreads();
+    // forward then reverse samples, duplicates removed with an LDS hash set (reference: sort + binary search, :625-666)
+    if (tid < 128) {
+        const bool is_old = tid >= 64;
+        const uint32_t k = tid & 63;
+        const uint32_t cf = is_old ? c_fo : c_fn, cr = is_old ? c_ro : c_rn;
+        uint32_t id = kInvalid;
+        if (k < cf) id = (is_old ? a.fwd_old : a.fwd_new)[static_cast<size_t>(node) * kSamples + k];
+        else if (k >= kSamples && k - kSamples < cr) id = (is_old ? a.rev_old : a.rev_new)[static_cast<size_t>(node) * kSamples + (k - kSamples)];
+        bool keep = id != kInvalid && id < seg_len && lds_set_insert(is_old ? L.hash_old : L.hash_new, id);
+        // forward entries first: rank within the wave keeps that order (wave 0 = new, wave 1 = old)
+        const uint64_t m = ballot(keep);
+        if (keep) {
+            const uint32_t pos = prefix_count(m);
+            (is_old ? L.old_ids : L.new_ids)[pos] = id;
+            (is_old ? L.old_norms : L.new_norms)[pos] = a.norms[seg_start + id];
+        }
+        if (lane == 0) (is_old ? L.n_old : L.n_new) = __popcll(m);
+    }
+    __syncthreads();
+    const uint32_t n_new = L.n_new, n_old = L.n_old;
+    if (n_new == 0) return;
+
+    const int rb = wave >> 1, cb = wave & 1;
+    float16v acc_nn, acc_no;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        acc_nn[r] = 0.f;
+        acc_no[r] = 0.f;
+    }
+    const bool need_nn = (rb * 32 < static_cast<int>(n_new)) && (cb * 32 < static_cast<int>(n_new));
+    const bool need_no = (rb * 32 < static_cast<int>(n_new)) && (cb * 32 < static_cast<int>(n_old));
+
+    for (uint32_t k0 = 0; k0 < a.dim_pad; k0 += 128) {
+        if (k0) __syncthreads();
+        // gather: 16 lanes x 16 B per 128-dim chunk row, 16 rows per pass, new rows then old rows
+        for (uint32_t r0 = 0; r0 < 128; r0 += 16) {
+            const uint32_t r = r0 + (tid >> 4), q = tid & 15;
+            const bool is_old = r >= 64;
+            const uint32_t rr = r & 63;
+            const uint32_t n = is_old ? n_old : n_new;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            const uint32_t d0 = k0 + q * 8;
+            if (rr < n && d0 < a.dim_pad) {
+                const uint32_t id = (is_old ? L.old_ids : L.new_ids)[rr];
+                v = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
+            }
+            *reinterpret_cast<float4*>(&(is_old ? L.xo : L.xn)[rr][q * 8]) = v;
+        }
+        __syncthreads();
+        if (need_nn) mfma_chunk(acc_nn, L.xn, L.xn, rb, cb, lane);
+        if (need_no) mfma_chunk(acc_no, L.xn, L.xo, rb, cb, lane);
+    }
+
+    const int t = lane & 31, kh = lane >> 5;
+    // ---- phase 1: new x new
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
+        float d = FLT_MAX;
+        if (i < n_new && j < n_new) d = fmaxf((L.new_norms[i] + L.new_norms[j]) - 2.f * acc_nn[r], 0.f);
+        L.dist[i][j] = d;
+    }
+    __syncthreads();
+    if (tid < 64 && static_cast<uint32_t>(tid) < n_new) {   // get_min_item (:581-623): nearest partner with a different id
+        const uint32_t me = L.new_ids[tid];
+        float best = FLT_MAX;
+        uint32_t bid = kInvalid;
+        for (uint32_t j = 0; j < n_new; j++) {
+            const float d = L.dist[tid][j];
+            if (j != static_cast<uint32_t>(tid) && d < best) {
+                best = d;
+                bid = L.new_ids[j];
+            }
+        }
+        emit_offer(a, seg_start, seg_len, me, bid, best);
+    }
+    if (n_old == 0) return;
+    // ---- phase 2: new x old (rows: new, columns: old)
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
+        float d = FLT_MAX;
+        if (i < n_new && j < n_old) d = fmaxf((L.new_norms[i] + L.old_norms[j]) - 2.f * acc_no[r], 0.f);
+        L.dist[i][j] = d;
+    }
+    __syncthreads();
+    if (tid < 64) {
+        if (static_cast<uint32_t>(tid) < n_new) {
+            const uint32_t me = L.new_ids[tid];
+            float best = FLT_MAX;
+            uint32_t bid = kInvalid;
+            for (uint32_t j = 0; j < n_old; j++) {
+                const float d = L.dist[tid][j];
+                if (L.old_ids[j] != me && d < best) {
+                    best = d;
+                    bid = L.old_ids[j];
+                }
+            }
+            emit_offer(a, seg_start, seg_len, me, bid, best);
+        }
+    } else if (tid < 128) {
+        const uint32_t c = tid - 64;
+        if (c < n_old) {
+            const uint32_t me = L.old_ids[c];
+            float best = FLT_MAX;
+            uint32_t bid = kInvalid;
+            for (uint32_t i = 0; i < n_new; i++) {
+                const float d = L.dist[i][c];
+                if (L.new_ids[i] != me && d < best) {
+                    best = d;
+                    bid = L.new_ids[i];
+                }
+            }
+            emit_offer(a, seg_start, seg_len, me, bid, best);
+        }
+    }
+}
+
+// ---- merge: list (width) + inbox (<= cap) -> sorted, de-duplicated list of `width`; one wavefront per node
+// key = dist bits : id (31 bits) : source (0 = already in the list, 1 = offer); payload = old flag
+template <int M>
+struct Net64 {
+    static constexpr int NR = M / 64;
+    template <int LM>
+    static __device__ __forceinline__ unsigned long long xor_lane(unsigned long long v) {
+        const uint32_t lo = lane_xor<LM>(static_cast<uint32_t>(v)), hi = lane_xor<LM>(static_cast<uint32_t>(v >> 32));
+        return (static_cast<unsigned long long>(hi) << 32) | lo;
+    }
+    template <int K, int J>
+    static __device__ __forceinline__ void stage(unsigned long long (&k)[NR], uint32_t (&v)[NR], int lane) {
+        if constexpr (J < NR) {
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                if ((r & J) == 0) {
+                    const int e = NR * lane + r;
+                    const bool asc = (K >= M) ? true : ((e & K) == 0);
+                    if ((k[r] > k[r | J]) == asc) {
+                        const unsigned long long tk = k[r]; k[r] = k[r | J]; k[r | J] = tk;
+                        const uint32_t tv = v[r]; v[r] = v[r | J]; v[r | J] = tv;
+                    }
+                }
+            }
+        } else {
+            constexpr int LM = J / NR;
+            const bool lower = (lane & LM) == 0;
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                const int e = NR * lane + r;
+                const bool asc = (K >= M) ? true : ((e & K) == 0);
+                const unsigned long long ok = xor_lane<LM>(k[r]);
+                const uint32_t ov = lane_xor<LM>(v[r]);
+                const bool keep_min = lower == asc;
+                if (keep_min ? (ok < k[r]) : (ok > k[r])) {
+                    k[r] = ok;
+                    v[r] = ov;
+                }
+            }
+        }
+    }
+    template <int K, int J>
+    static __device__ __forceinline__ void merge_from(unsigned long long (&k)[NR], uint32_t (&v)[NR], int lane) {
+        stage<K, J>(k, v, lane);
+        if constexpr (J > 1) merge_from<K, J / 2>(k, v, lane);
+    }
+    template <int K>
+    static __device__ __forceinline__ void sort_from(unsigned long long (&k)[NR], uint32_t (&v)[NR], int lane) {
+        merge_from<K, K / 2>(k, v, lane);
+        if constexpr (K < M) sort_from<K * 2>(k, v, lane);
+    }
+    static __device__ __forceinline__ void sort(unsigned long long (&k)[NR], uint32_t (&v)[NR], int lane) { sort_from<2>(k, v, lane); }
+};
+
+// Bloom filter of ids already used as "new" samples (reference BloomFilter :203-276: 512-bit sets, 3 hashes)
+__device__ __forceinline__ uint32_t bloom_h0(uint32_t v) { v *= 1103515245u; v += 12345u; v ^= v << 13; v ^= v >> 17; v ^= v << 5; return v; }
+__device__ __forceinline__ uint32_t bloom_h1(uint32_t v) { v *= 1664525u; v += 1013904223u; v ^= v << 13; v ^= v >> 17; v ^= v << 5; return v; }
+
+__device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane, uint32_t& total) {
+    uint32_t incl = value;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t o = __shfl_up(incl, off);
+        if (lane >= off) incl += o;
+    }
+    total = __shfl(incl, 63);
+    return incl - value;
+}
+
+// Merge + resample.  The list and this round's offers are sorted together by (distance, id); repeats of an id are
+// dropped; the first `width` survive as the new list.  Samples for the next join:
+//   new = the best <= 32 offers of this round (what the reference's 32-wide device list would hold) that the
+//         Bloom filter has not seen (sample_graph_new :973-1001); those that made the list are flagged old;
+//   old = the first <= 32 list entries that were already flagged old (sample_segment_graph :1073-1104).
+template <int M>
+__global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t num,
+                                                        uint32_t width, uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new,
+                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats) {
+    constexpr int NR = M / 64;
+    __shared__ uint32_t filter_lds[4][64];
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (node >= num) return;
+    uint32_t* filter = filter_lds[wave];
+    const uint32_t bloom_words = bloom_sets * 16;
+    if (static_cast<uint32_t>(lane) < bloom_words) filter[lane] = bloom[static_cast<size_t>(node) * bloom_words + lane];
+    const uint32_t raw = inbox_counts[node];
+    const uint32_t n_in = raw < inbox_cap ? raw : inbox_cap;
+    unsigned long long k[NR];
+    uint32_t v[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        k[r] = ~0ull;
+        v[r] = 0;
+        if (e < width) {
+            const uint32_t id = list_ids[static_cast<size_t>(node) * width + e];
+            const float d = list_dists[static_cast<size_t>(node) * width + e];
+            if (id != kInvalid) {
+                k[r] = (static_cast<unsigned long long>(__float_as_uint(d)) << 32) | (static_cast<unsigned long long>(id & ~kOld) << 1);
+                v[r] = id & kOld;
+            }
+        } else if (e - width < n_in) {
+            const uint2 o = inbox[static_cast<size_t>(node) * inbox_cap + (e - width)];
+            k[r] = (static_cast<unsigned long long>(o.x) << 32) | (static_cast<unsigned long long>(o.y) << 1) | 1ull;
+            v[r] = 0;   // offers enter as new
+        }
+    }
+    Net64<M>::sort(k, v, lane);
+    // drop repeats of an id (equal id => equal distance => adjacent after the sort; the list's own copy sorts first)
+    uint32_t keep_count = 0, offer_count = 0, old_count = 0;
+    bool keep[NR], offer[NR];
+    const unsigned long long last_of_prev = __shfl_up(k[NR - 1], 1);
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const unsigned long long prev = r == 0 ? last_of_prev : k[r - 1];
+        const bool first = (r == 0 && lane == 0);
+        keep[r] = k[r] != ~0ull && (first || (prev >> 1) != (k[r] >> 1));
+        offer[r] = keep[r] && (k[r] & 1ull);
+        keep_count += keep[r];
+        offer_count += offer[r];
+    }
+    uint32_t total_keep, total_offer, total_new, total_old;
+    uint32_t pos = wave_exclusive_scan(keep_count, lane, total_keep);
+    uint32_t orank = wave_exclusive_scan(offer_count, lane, total_offer);
+    // Bloom check of the best 32 offers against the filter as it was before this round
+    bool fresh[NR];
+    uint32_t fresh_count = 0;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        fresh[r] = false;
+        if (offer[r]) {
+            if (orank < kSamples) {
+                const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+                const uint32_t base = (id % bloom_sets) * 512;
+                uint32_t h = bloom_h0(id);
+                const uint32_t b0 = base + h % 512;
+                h += bloom_h1(id);
+                const uint32_t b1 = base + h % 512;
+                h += bloom_h1(id);
+                const uint32_t b2 = base + h % 512;
+                const bool seen = ((filter[b0 >> 5] >> (b0 & 31)) & (filter[b1 >> 5] >> (b1 & 31)) & (filter[b2 >> 5] >> (b2 & 31)) & 1u) != 0;
+                fresh[r] = !seen;
+            }
+            orank++;
+        }
+        fresh_count += fresh[r];
+    }
+    uint32_t nrank = wave_exclusive_scan(fresh_count, lane, total_new);
+    // old samples: list entries (final position < width) that were flagged old before this round
+    uint32_t p2 = pos;
+    bool oldf[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        oldf[r] = keep[r] && p2 < width && (v[r] & kOld) != 0;
+        old_count += oldf[r];
+        p2 += keep[r];
+    }
+    uint32_t orank_old = wave_exclusive_scan(old_count, lane, total_old);
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+        uint32_t flag = v[r];
+        if (fresh[r]) {
+            if (nrank < kSamples) {
+                fwd_new[static_cast<size_t>(node) * kSamples + nrank] = id;
+                flag = kOld;
+                const uint32_t base = (id % bloom_sets) * 512;
+                uint32_t h = bloom_h0(id);
+                const uint32_t b0 = base + h % 512;
+                h += bloom_h1(id);
+                const uint32_t b1 = base + h % 512;
+                h += bloom_h1(id);
+                const uint32_t b2 = base + h % 512;
+                atomicOr(&filter[b0 >> 5], 1u << (b0 & 31));
+                atomicOr(&filter[b1 >> 5], 1u << (b1 & 31));
+                atomicOr(&filter[b2 >> 5], 1u << (b2 & 31));
+            }
+            nrank++;
+        }
+        if (oldf[r]) {
+            if (orank_old < kSamples) fwd_old[static_cast<size_t>(node) * kSamples + orank_old] = id;
+            orank_old++;
+        }
+        if (keep[r]) {
+            if (pos < width) {
+                list_ids[static_cast<size_t>(node) * width + pos] = id | flag;
+                list_dists[static_cast<size_t>(node) * width + pos] = __uint_as_float(static_cast<uint32_t>(k[r] >> 32));
+            }
+            pos++;
+        }
+    }
+    for (uint32_t e = total_keep + lane; e < width; e += 64) {
+        list_ids[static_cast<size_t>(node) * width + e] = kInvalid;
+        list_dists[static_cast<size_t>(node) * width + e] = FLT_MAX;
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (static_cast<uint32_t>(lane) < bloom_words) bloom[static_cast<size_t>(node) * bloom_words + lane] = filter[lane];
+    if (lane == 0) {
+        inbox_counts[node] = 0;
+        counts[static_cast<size_t>(node) * 4 + 0] = total_new < kSamples ? total_new : kSamples;
+        counts[static_cast<size_t>(node) * 4 + 1] = total_old < kSamples ? total_old : kSamples;
+        counts[static_cast<size_t>(node) * 4 + 2] = 0;
+        counts[static_cast<size_t>(node) * 4 + 3] = 0;
+        if (stats) {
+            atomicAdd(&stats[0], static_cast<unsigned long long>(raw));
+            if (raw > inbox_cap) atomicAdd(&stats[1], static_cast<unsigned long long>(raw - inbox_cap));
+        }
+    }
+}
+
+// ---- finalize (shrink step :1376-1402): first `degree` ids of each list; unfilled slots get a pseudo-random id
+__host__ __device__ inline uint32_t xorshift32(uint32_t u) {   // reference utils.cuh:14-19
+    u ^= u >> 13;
+    u ^= u << 27;
+    u ^= u >> 5;
+    return u * 0x9E3779B9u;
+}
+
+__global__ __launch_bounds__(256) void nnd_finalize_kernel(const uint32_t* list_ids, uint32_t num, uint32_t width, uint32_t degree, Segments segs,
+                                                           uint32_t* knn_graph) {
+    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+    const uint32_t node = idx / degree, j = idx % degree;
+    if (node >= num) return;
+    uint32_t start, len;
+    locate(segs, node, start, len);
+    const uint32_t e = list_ids[static_cast<size_t>(node) * width + j];
+    const uint32_t id = e & ~kOld;
+    knn_graph[static_cast<size_t>(node) * degree + j] = (e != kInvalid && id < len) ? id : xorshift32(node * width + j) % (len ? len : 1);
+}
+
+}  // namespace glide
+
+using namespace glide;
+
+namespace {
+uint32_t nnd_width(uint32_t degree) { return round_up32(static_cast<uint32_t>(degree * (degree <= 32 ? 1.0 : 1.3))); }  // nn_descent.cuh:1427-1428
+uint32_t nnd_inbox_cap(uint32_t width) { return 256 - width; }   // list + inbox fill one 256-element sort
+size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
+struct NndLayout {
+    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, counts, inbox_counts, inbox, bloom, stats, total;
+    uint32_t width, cap, dim_pad, bloom_sets;
+};
+NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
+    NndLayout l;
+    l.width = nnd_width(degree);
+    l.cap = nnd_inbox_cap(l.width);
+    l.dim_pad = (dim + 7) / 8 * 8;
+    l.bloom_sets = nnd_width(static_cast<uint32_t>(1.5 * degree)) / 32;   // internal degree / 32 (nn_descent.cuh:962, params.cuh:23-24)
+    const size_t n = num;
+    size_t off = 0;
+    auto take = [&off](size_t bytes) { size_t o = off; off += align256(bytes); return o; };
+    l.half_rows = take(n * l.dim_pad * 2);
+    l.norms = take(n * 4);
+    l.list_ids = take(n * l.width * 4);
+    l.list_dists = take(n * l.width * 4);
+    l.fwd_new = take(n * kSamples * 4);
+    l.fwd_old = take(n * kSamples * 4);
+    l.rev_new = take(n * kSamples * 4);
+    l.rev_old = take(n * kSamples * 4);
+    l.counts = take(n * 16);
+    l.inbox_counts = take(n * 4);
+    l.inbox = take(n * l.cap * 8);
+    l.bloom = take(n * l.bloom_sets * 64);
+    l.stats = take(64);
+    l.total = off;
+    return l;
+}
+}  // namespace
+
+extern "C" {
+
+size_t glide_hip_nnd_workspace_bytes(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree) {
+    return nnd_layout(reorder_num, dim, knn_degree).total;
+}
+
+int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts,
+                        const uint32_t* segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations, uint32_t seed,
+                        uint32_t* knn_graph, void* workspace, size_t workspace_bytes, unsigned long long* stats_out, void* stream) {
+    if (!reorder_data || !segment_starts || !segment_lengths || !knn_graph || !workspace) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim == 0 || segment_num == 0 || knn_degree == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // also keeps the Bloom filter within 64 words
+    if (reorder_num == 0) return GLIDE_OK;
+    const NndLayout l = nnd_layout(reorder_num, dim, knn_degree);
+    if (l.bloom_sets > 4) return GLIDE_ERR_UNSUPPORTED;
+    if (workspace_bytes < l.total || reinterpret_cast<uintptr_t>(workspace) % 16) return GLIDE_ERR_BAD_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    unsigned char* w = static_cast<unsigned char*>(workspace);
+    _Float16* half_rows = reinterpret_cast<_Float16*>(w + l.half_rows);
+    float* norms = reinterpret_cast<float*>(w + l.norms);
+    uint32_t* list_ids = reinterpret_cast<uint32_t*>(w + l.list_ids);
+    float* list_dists = reinterpret_cast<float*>(w + l.list_dists);
+    uint32_t* fwd_new = reinterpret_cast<uint32_t*>(w + l.fwd_new);
+    uint32_t* fwd_old = reinterpret_cast<uint32_t*>(w + l.fwd_old);
+    uint32_t* rev_new = reinterpret_cast<uint32_t*>(w + l.rev_new);
+    uint32_t* rev_old = reinterpret_cast<uint32_t*>(w + l.rev_old);
+    uint32_t* counts = reinterpret_cast<uint32_t*>(w + l.counts);
+    uint32_t* inbox_counts = reinterpret_cast<uint32_t*>(w + l.inbox_counts);
+    uint2* inbox = reinterpret_cast<uint2*>(w + l.inbox);
+    uint32_t* bloom = reinterpret_cast<uint32_t*>(w + l.bloom);
+    unsigned long long* stats = stats_out ? reinterpret_cast<unsigned long long*>(w + l.stats) : nullptr;
+    const Segments segs{segment_starts, segment_lengths, segment_num};
+    const uint32_t n = reorder_num;
+
+    if (stats) {
+        int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(stats), 0u, 4, stream);
+        if (rc != GLIDE_OK) return rc;
+    }
+    hipLaunchKernelGGL(nnd_prepare_kernel, dim3(ceil_div(n, 4)), dim3(256), 0, s, reorder_data, n, dim, l.dim_pad, half_rows, norms);
+    hipLaunchKernelGGL(nnd_init_kernel, dim3(ceil_div(n * l.width, 256)), dim3(256), 0, s, list_ids, list_dists, inbox_counts, n, l.width, segs, seed);
+    JoinArgs ja{half_rows, norms, fwd_new, fwd_old, rev_new, rev_old, counts, list_dists, inbox_counts, inbox, stats, n, l.dim_pad, l.width, l.cap, segs};
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(sizeof(JoinLds))));
+    {
+        int rc = glide_hip_fill_u32(bloom, 0u, static_cast<size_t>(n) * l.bloom_sets * 16, stream);
+        if (rc != GLIDE_OK) return rc;
+    }
+    // first samples come from the random lists (sample_graph(true), nn_descent.cuh:1266); later ones from the merge
+    hipLaunchKernelGGL(nnd_sample_kernel, dim3(ceil_div(n, 4)), dim3(256), 0, s, list_ids, n, l.width, segs, fwd_new, fwd_old, counts);
+    for (uint32_t it = 0; it < iterations; it++) {
+        hipLaunchKernelGGL(nnd_reverse_kernel, dim3(ceil_div(n * 64, 256)), dim3(256), 0, s, fwd_new, fwd_old, counts, rev_new, rev_old, n, segs);
+        hipLaunchKernelGGL(nnd_join_kernel, dim3(n), dim3(256), sizeof(JoinLds), s, ja);
+        const uint32_t m = l.width + l.cap;
+        if (m <= 128) {
+            hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(n, 4)), dim3(256), 0, s, list_ids, list_dists, inbox_counts, inbox, n, l.width, l.cap,
+                               bloom, l.bloom_sets, fwd_new, fwd_old, counts, stats);
+        } else {
+            hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(n, 4)), dim3(256), 0, s, list_ids, list_dists, inbox_counts, inbox, n, l.width, l.cap,
+                               bloom, l.bloom_sets, fwd_new, fwd_old, counts, stats);
+        }
+    }
+    hipLaunchKernelGGL(nnd_finalize_kernel, dim3(ceil_div(n * knn_degree, 256)), dim3(256), 0, s, list_ids, n, l.width, knn_degree, segs, knn_graph);
+    if (stats_out) GLIDE_HIP_TRY(hipMemcpyAsync(stats_out, stats, 16, hipMemcpyDeviceToDevice, s));
+    return launch_status();
+}
+
+}  // extern "C"

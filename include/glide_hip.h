@@ -100,6 +100,22 @@ int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim,
                          uint32_t iterations, float *centroids, void *workspace, size_t workspace_bytes,
                          void *stream);
 
+/* ---- NN-descent kNN graph (subsystem 2) ---------------------------------------------------------------------
+ * Replaces build_nnd / GNND::build (nn_descent.cuh:1238-1467) together with its device kernels
+ * (preprocess_data_kernel :445, add_rev_edges_kernel :490, local_join_kernel :668) and the host-side sampling
+ * and list merging (GnndGraph :973-1149).  Builds, for every partition given by segment_starts/segment_lengths
+ * (device arrays, segment_num entries, the boundary segment included), a knn_degree-regular graph of
+ * partition-local ids: knn_graph is reorder_num x knn_degree, nearest first.  `iterations` rounds of
+ * sample -> reverse sample -> local join (64 x 64 fp16 matrix-core tiles, fp32 accumulate, norm-trick
+ * epilogue, one offer per row/column) -> merge are run; lists, flags and samples stay in `workspace`.
+ * stats_out (nullable, 2 device u64): offers received by the merge step, offers dropped by a full inbox.
+ * Limits: knn_degree <= 65 (list width round_up32(1.3 * knn_degree) <= 96, Bloom filter <= 2048 bits), dim % 4 == 0. */
+size_t glide_hip_nnd_workspace_bytes(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree);
+int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim,
+                        const uint32_t *segment_starts, const uint32_t *segment_lengths, uint32_t segment_num,
+                        uint32_t knn_degree, uint32_t iterations, uint32_t seed, uint32_t *knn_graph,
+                        void *workspace, size_t workspace_bytes, unsigned long long *stats_out, void *stream);
+
 /* ---- graph construction (subsystem 3) ----------------------------------------------------------------------
  * All kernels give one point to one wavefront.  Limits as for glide_hip_search (knn_degree, graph_degree <= 128,
  * beam <= 256, dim % 4 == 0, dim <= 1024).  `counters` as in glide_hip_search (prune distances count as rows). */

@@ -1,0 +1,108 @@
+"""GPU NN-descent against exact kNN and the CPU restatement (statistical parity: graph recall)."""
+import numpy as np
+import pytest
+
+from conftest import lowdim_data, lowdim_float_data
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from glide_amd import capi
+    capi.set_device(0)
+    return capi
+
+
+def gpu_nnd(hip, rdata, seg_start, seg_len, k, iterations, seed=0):
+    n, dim = rdata.shape
+    d_data = hip.DeviceArray.from_numpy(rdata, np.float32)
+    d_ss, d_sl = hip.DeviceArray.from_numpy(seg_start, np.uint32), hip.DeviceArray.from_numpy(seg_len, np.uint32)
+    knn = hip.DeviceArray((n, k), np.uint32)
+    wb = hip.nnd_workspace_bytes(n, dim, k)
+    ws = hip.DeviceArray(wb // 16 + 1, np.dtype("V16"))
+    stats = hip.DeviceArray.from_numpy(np.zeros(2, np.uint64))
+    hip.nnd_build(d_data, n, dim, d_ss, d_sl, seg_start.size, k, iterations, seed, knn, ws, wb, stats)
+    hip.synchronize()
+    return knn.numpy(), stats.numpy()
+
+
+def partition_recall(knn, rdata, seg_start, seg_len, k, sample=400, metric=0):
+    from glide_amd.datasets import recall
+    from oracle import oracle as O
+    out = []
+    for s, l in zip(seg_start.tolist(), seg_len.tolist()):
+        if l <= k + 1:
+            continue
+        sub = rdata[s:s + l]
+        m = min(sample, l)
+        gt, _ = O.bruteforce_knn(sub, sub[:m], k, metric, exclude_self=True)
+        out.append(recall(knn[s:s + m], gt, k))
+    return float(np.mean(out))
+
+
+def test_nnd_structure_and_recall(hip):
+    from oracle import oracle as O
+    data = lowdim_data(12000, 128, seed=21)
+    seg_len = np.array([5000, 4000, 2990, 10], dtype=np.uint32)       # the last one stands in for a tiny boundary list
+    seg_start = O.segment_starts(np.append(seg_len, 0))[:4]
+    k = 32
+    knn, stats = gpu_nnd(hip, data, seg_start, seg_len, k, 10)
+    # structure: ids are partition-local, no self loops, no repeated neighbour in partitions larger than k
+    for s, l in zip(seg_start.tolist(), seg_len.tolist()):
+        rows = knn[s:s + l]
+        assert (rows < l).all()
+        if l > 4 * k:   # partitions with fewer points than slots are padded with pseudo-random ids, like the reference's shrink step
+            assert (rows != np.arange(l, dtype=np.uint32)[:, None]).all()
+            srt = np.sort(rows, axis=1)
+            assert (np.diff(srt.astype(np.int64), axis=1) != 0).all()
+    r_gpu = partition_recall(knn, data, seg_start, seg_len, k)
+    cpu = O.nnd_build(data, seg_start, seg_len, k, 10).astype(np.uint32)
+    r_cpu = partition_recall(cpu, data, seg_start, seg_len, k)
+    print("graph recall@32 after 10 iterations: gpu %.4f cpu-restatement %.4f; offers %d dropped %d" % (r_gpu, r_cpu, stats[0], stats[1]))
+    assert r_gpu >= 0.95
+    assert r_gpu >= r_cpu - 0.005      # within half a point of the reference algorithm at equal degree / iterations
+
+
+def test_nnd_rows_are_sorted_by_distance(hip):
+    from oracle import oracle as O
+    data = lowdim_data(4000, 128, seed=22)
+    seg_len = np.array([4000], dtype=np.uint32)
+    seg_start = np.array([0], dtype=np.uint32)
+    knn, _ = gpu_nnd(hip, data, seg_start, seg_len, 32, 12)
+    d = np.sqrt(((data[knn[:200].astype(np.int64)] - data[:200, None, :]) ** 2).sum(-1))
+    assert (np.diff(d, axis=1) >= -1e-3).all()       # ascending (fp16 tile distances; integer data is exact)
+
+
+def test_nnd_k64_cosine_dim96(hip):
+    from oracle import oracle as O
+    data = lowdim_float_data(6000, 96, seed=23)
+    seg_len = np.array([3500, 2500], dtype=np.uint32)
+    seg_start = np.array([0, 3500], dtype=np.uint32)
+    knn, _ = gpu_nnd(hip, data, seg_start, seg_len, 64, 12)
+    assert knn.shape == (6000, 64)
+    r = partition_recall(knn, data, seg_start, seg_len, 64, sample=200, metric=1)
+    print("graph recall@64 (cosine, dim 96): %.4f" % r)
+    assert r >= 0.93
+
+
+def test_nnd_dim960(hip):
+    rng = np.random.default_rng(5)
+    base = rng.random((40, 960)).astype(np.float32)
+    data = (base[rng.integers(0, 40, 3000)] + rng.random((3000, 960)).astype(np.float32) * 0.3).astype(np.float32)
+    seg_len = np.array([3000], dtype=np.uint32)
+    seg_start = np.array([0], dtype=np.uint32)
+    knn, _ = gpu_nnd(hip, data, seg_start, seg_len, 32, 10)
+    r = partition_recall(knn, data, seg_start, seg_len, 32, sample=200)
+    print("graph recall@32 (dim 960): %.4f" % r)
+    assert r >= 0.85
+
+
+def test_nnd_rejects_unsupported(hip):
+    d = hip.DeviceArray(1024, np.float32)
+    with pytest.raises(hip.GlideHipError) as e:
+        hip.nnd_build(d, 8, 128, d, d, 1, 100, 1, 0, d, d, 1 << 30)
+    assert e.value.code == -1
+    with pytest.raises(hip.GlideHipError) as e:
+        hip.nnd_build(d, 8, 128, d, d, 1, 32, 1, 0, d, d, 16)      # workspace too small
+    assert e.value.code == -2
