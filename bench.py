@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the GLIDE hot path on one MI355X: index build seconds + graph recall@32, search QPS.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-navigable|cfg0] [--no-cpu]
+
+A "step" is one beam-search pass of the whole query batch (10 000 queries, top-10) over the finished index.
+Before the timed steps the index is built once on the GPU (partition -> NN-descent -> sub-graph build + boundary
+merge -> reverse edges -> refine) and its stage times, the kNN-graph recall@32 against exact neighbours and the
+recall@10 of the whole beam sweep are measured.  One JSON line is printed.
+
+Everything on the product path goes through libglide_hip.so.  torch is imported only to compute exact ground
+truth on the GPU (a checker); the CPU oracle is used only for the cpu_baseline leg.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg1-navigable"])
+    ap.add_argument("--nnd-iterations", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-navigable", action="store_true", help="skip the extra navigable-data variant")
+    return ap.parse_args()
+
+
+WORKLOADS = {
+    # name: (num, partitions, knn degree, NN-descent iterations, queries, description)
+    "cfg0": (100_000, 10, 64, 8, 1_000, "cfg0: 100k x 128 fp32 clipped/rounded 64-component GMM, L2, degree 32, NN-descent k=64 x 8 iterations, 1k queries"),
+    "cfg1": (1_000_000, 16, 32, 20, 10_000, "cfg1: 1M x 128 fp32 clipped/rounded 64-component GMM, L2, 16 partitions, degree 32, 10k queries top-10, beams 32/64/128/256"),
+    "cfg1-navigable": (1_000_000, 16, 32, 20, 10_000, "cfg1 shapes on integer-valued data of low intrinsic dimension (12-d latent, 0..255): 1M x 128, 16 partitions, degree 32, 10k queries top-10"),
+}
+
+
+def make_data(workload, num, nq):
+    import numpy as np
+    from glide_amd import datasets as D
+    if workload == "cfg1-navigable":
+        a = np.random.default_rng(0).standard_normal((12, 128)).astype(np.float32)
+
+        def gen(m, seed):
+            r = np.random.default_rng(seed)
+            out = np.empty((m, 128), dtype=np.float32)
+            for s in range(0, m, 1 << 18):
+                e = min(m, s + (1 << 18))
+                z = r.standard_normal((e - s, 12)).astype(np.float32)
+                out[s:e] = np.rint(np.clip(z @ a * 20 + 128 + r.standard_normal((e - s, 128)).astype(np.float32) * 3, 0, 255))
+            return out
+        return gen(num, 1234), gen(nq, 4321)
+    return D.gmm_clipped(num, 128, seed=1234), D.gmm_clipped(nq, 128, seed=4321)
+
+
+def exact_knn(torch, base, queries, k, exclude_self_offset=None, chunk=2048):
+    """Exact top-k by brute force on the GPU (checker).  Integer-valued inputs below 2^24 make the norm trick exact."""
+    b = torch.from_numpy(base).cuda()
+    bn = (b * b).sum(1)
+    out = []
+    for s in range(0, queries.shape[0], chunk):
+        q = torch.from_numpy(queries[s:s + chunk]).cuda()
+        d = (q * q).sum(1, keepdim=True) + bn[None] - 2.0 * (q @ b.T)
+        if exclude_self_offset is not None:
+            idx = torch.arange(q.shape[0], device="cuda")
+            d[idx, idx + s + exclude_self_offset] = float("inf")
+        out.append(d.topk(k, largest=False).indices.cpu())
+    return torch.cat(out).numpy()
+
+
+def run_workload(args, workload, torch, want_cpu):
+    import numpy as np
+    from glide_amd import capi, datasets as D, index as G
+
+    num, parts, knn_degree, nnd_iters, nq, desc = WORKLOADS[workload]
+    if args.nnd_iterations:
+        nnd_iters = args.nnd_iterations
+    degree, top_k = 32, 10
+    t0 = time.time()
+    data, queries = make_data(workload, num, nq)
+    gen_s = time.time() - t0
+
+    d_data = capi.DeviceArray.from_numpy(data)
+    res = {}
+    pp = G.PartitionParameter(centroid_num=parts, boundary_factor=1.04, sample_factor=0.01)   # reference test.sh:10-12
+    d_re, d_map, h_start, h_len, d_cent = G.preprocess(pp, d_data, res)
+    nn = G.NNDescentParameter(graph_degree=knn_degree, max_iterations=nnd_iters)
+    d_knn = G.build_nnd(nn, d_re, h_start, h_len, res, stats=True)
+
+    # graph recall@k of the kNN graph inside each partition (what NN-descent is asked to find) on 500 nodes per partition
+    knn = d_knn.numpy()
+    rdata = d_re.numpy()
+    h_map = d_map.numpy()
+    k_eval = min(32, knn_degree)
+    per_part, glob = [], []
+    sample_global_ids, sample_rows = [], []
+    for s, l in zip(h_start.tolist(), h_len.tolist()):
+        if l <= 2 * knn_degree:
+            continue
+        m = min(500, l)
+        sub = rdata[s:s + l]
+        gt = exact_knn(torch, sub, sub[:m], k_eval, exclude_self_offset=0)
+        per_part.append(D.recall(knn[s:s + m, :k_eval], gt, k_eval))
+        if s < num:
+            sample_global_ids.append(h_map[s:s + m])
+            sample_rows.append((s, m))
+    # the same nodes against exact neighbours over the whole data set (capped by partition locality)
+    if sample_global_ids:
+        gids = np.concatenate(sample_global_ids)
+        b = torch.from_numpy(data).cuda()
+        bn = (b * b).sum(1)
+        q = b[torch.from_numpy(gids.astype(np.int64)).cuda()]
+        d = (q * q).sum(1, keepdim=True) + bn[None] - 2.0 * (q @ b.T)
+        d[torch.arange(q.shape[0], device="cuda"), torch.from_numpy(gids.astype(np.int64)).cuda()] = float("inf")
+        gt_glob = d.topk(k_eval, largest=False).indices.cpu().numpy()
+        found = np.concatenate([h_map[s + knn[s:s + m, :k_eval].astype(np.int64)] for s, m in sample_rows])
+        glob.append(D.recall(found, gt_glob, k_eval))
+        del b, bn, q, d
+    graph_recall_partition = float(np.mean(per_part))
+    graph_recall_global = float(glob[0]) if glob else None
+    del rdata, knn
+
+    index = G.GLIDE(degree, d_data, d_cent, G.Metric.Euclidean)
+    bp = G.IndexParameter(graph_degree=degree, knn_degree=knn_degree, relaxant_factor=1.05)   # test.sh:16
+    sp_knn = G.make_search_parameter(64, knn_degree)         # test.sh:17 build beam
+    sp_ref = G.make_search_parameter(128, knn_degree)        # test.sh:18 refine beam (hash sized with knn_degree, small_build.cu:76-82)
+    index.build(bp, sp_knn, sp_ref, d_knn, h_start, h_len, d_map, d_re, res, counters=True)
+    build_sec = res["pre_time"] + res["knn_time"] + res["index_time"] + res["refine_time"]
+    graph = index.d_graph.numpy()
+    holes = float((graph == 0xFFFFFFFF).mean())
+
+    # ---- search sweep
+    gt = exact_knn(torch, data, queries, top_k)
+    d_q = capi.DeviceArray.from_numpy(queries)
+    d_ids, d_dists = capi.DeviceArray((nq, top_k), np.uint32), capi.DeviceArray((nq, top_k), np.float32)
+    sweep = []
+    for beam in (32, 64, 128, 256):
+        sp = G.make_search_parameter(beam, degree, top_k)
+        cnt = capi.DeviceArray.from_numpy(np.zeros(3, np.uint64))
+        index.search(sp, d_q, counters=cnt, out=(d_ids, d_dists))
+        capi.synchronize()
+        c = cnt.numpy()
+        r = {}
+        index.search(sp, d_q, result=r, out=(d_ids, d_dists))
+        rec = D.recall(d_ids.numpy(), gt, top_k)
+        # algorithmic bytes of one launch: query rows + centroid table once + graph rows + scored data rows + results
+        alg = nq * 128 * 4 + parts * 128 * 4 + int(c[2]) * degree * 4 + int(c[1]) * 128 * 4 + nq * top_k * 8
+        sweep.append(dict(beam=beam, recall_at_10=rec, qps=r["QPS"], ms=r["search_time"] * 1e3, iterations_per_query=c[0] / nq,
+                          rows_per_query=c[1] / nq, algorithmic_bytes=alg))
+    ok = [s for s in sweep if s["recall_at_10"] >= 0.95]
+    chosen = min(ok, key=lambda s: s["beam"]) if ok else sweep[-1]
+
+    # ---- timed steps at the chosen beam: HIP events on the launch stream, warm-up first
+    sp = G.make_search_parameter(chosen["beam"], degree, top_k)
+    for _ in range(args.warmup):
+        index.search(sp, d_q, out=(d_ids, d_dists))
+    capi.synchronize()
+    e0, e1 = capi.Event(), capi.Event()
+    w0 = time.time()
+    e0.record()
+    for _ in range(args.steps):
+        capi.search(index.d_data, num, 128, index.d_graph, degree, index.d_centroids, parts, index.d_start_points, d_q, nq, top_k,
+                    sp.beam, sp.max_iterations, sp.min_iterations, sp.hash_bit, sp.hash_reset_interval, 0, d_ids, d_dists)
+    e1.record()
+    gpu_ms = e0.elapsed_ms(e1)
+    capi.synchronize()
+    wall_ms = (time.time() - w0) * 1e3
+    ms_per_step = wall_ms / args.steps
+    kernel_ms = gpu_ms / args.steps
+    achieved = chosen["algorithmic_bytes"] / (kernel_ms * 1e-3) / 1e9
+
+    out = dict(
+        workload=desc, gen_sec=gen_s, build_sec=build_sec,
+        build_stages=dict(pre=res["pre_time"], knn=res["knn_time"], index=res["index_time"], refine=res["refine_time"],
+                          detail={**res["pre_stages"], **res["build_stages"]}),
+        nnd_iterations=nnd_iters, nnd_offers=res["nnd_stats"][0], nnd_offers_dropped=res["nnd_stats"][1],
+        graph_recall_at_32=graph_recall_partition, graph_recall_at_32_global=graph_recall_global,
+        partition_sizes=[int(x) for x in h_len], empty_slots_fraction=holes,
+        sweep=sweep, beam=chosen["beam"], recall_at_10=chosen["recall_at_10"], recall_target_met=bool(ok),
+        qps=nq * args.steps / (wall_ms * 1e-3), ms_per_step=ms_per_step, kernel_ms=kernel_ms,
+        roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS, traffic=None,
+                      kernel="search_kernel<64,%d,1>" % (64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256),
+                      algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
+    )
+
+    if want_cpu:
+        out["cpu_baseline"] = cpu_baseline(data, queries, graph, d_cent.numpy(), index.d_start_points.numpy(), sp, top_k, gt)
+    return out
+
+
+def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt):
+    """The CPU restatement of the reference algorithm, timed on this box's host cores on a bounded sample."""
+    import numpy as np
+    from glide_amd import datasets as D
+    from oracle import oracle as O
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except Exception:
+        pass
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    nq = min(queries.shape[0], 4000)
+    t = time.time()
+    ids, _, _ = O.search(data, graph, centroids, start_points, queries[:nq], top_k, sp.beam, sp.max_iterations, sp.min_iterations,
+                         sp.hash_bit, sp.hash_reset_interval, 0, threads=cores)
+    search_s = time.time() - t
+    # NN-descent build of one 30k-point partition-sized sample with the same degree / 10 iterations
+    n_s = min(30_000, data.shape[0])
+    t = time.time()
+    O.nnd_build(data[:n_s], np.array([0], np.uint32), np.array([n_s], np.uint32), 32, 10, 0, threads=cores)
+    nnd_s = time.time() - t
+    t = time.time()
+    O.bruteforce_knn(data[:200_000], queries[:200], top_k, threads=cores)
+    bf_s = time.time() - t
+    return dict(value=nq / search_s, unit="queries/s", cores=cores, kind="port",
+                sample="beam search of the first %d queries (same index, beam %d) with the CPU restatement, %d threads" % (nq, sp.beam, cores),
+                recall_at_10=D.recall(ids, gt[:nq], top_k),
+                nnd_points_per_sec=n_s / nnd_s, nnd_sample="NN-descent k=32 x 10 iterations on the first %d points as one partition" % n_s,
+                bruteforce_qps=200 / bf_s * (200_000 / data.shape[0]), bruteforce_sample="exact top-10 of 200 queries over 200k rows, scaled to the full set")
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch   # first: libglide_hip.so then binds to the HIP runtime torch has already loaded
+    assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    from glide_amd import capi
+    capi.set_device(0)
+    info = capi.device_info()
+
+    main_res = run_workload(args, args.workload, torch, want_cpu=not args.no_cpu)
+    line = {
+        "metric": "search QPS at recall@10 >= 0.95 (index build sec and graph recall@32 alongside), 1 MI355X",
+        "value": main_res["qps"], "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": main_res["workload"], "graph_degree": 32, "top_k": 10, "beam": main_res["beam"],
+                   "build_beam": 64, "refine_beam": 128, "relaxant": 1.05, "boundary_factor": 1.04, "sample_factor": 0.01,
+                   "nnd_iterations": main_res["nnd_iterations"]},
+        "device": info["name"],
+    }
+    for k in ("build_sec", "build_stages", "graph_recall_at_32", "graph_recall_at_32_global", "recall_at_10", "recall_target_met",
+              "empty_slots_fraction", "sweep", "kernel_ms", "nnd_offers", "nnd_offers_dropped", "roofline"):
+        line[k] = main_res[k]
+    if "cpu_baseline" in main_res:
+        line["cpu_baseline"] = main_res["cpu_baseline"]
+    if args.workload == "cfg1" and not args.no_navigable:
+        nav = run_workload(args, "cfg1-navigable", torch, want_cpu=False)
+        line["navigable_variant"] = {k: nav[k] for k in ("workload", "build_sec", "build_stages", "graph_recall_at_32", "beam", "recall_at_10",
+                                                         "recall_target_met", "qps", "kernel_ms", "sweep", "roofline")}
+    print(json.dumps(line, default=float))
+
+
+if __name__ == "__main__":
+    main()
