@@ -33,6 +33,8 @@ def parse():
     ap.add_argument("--nnd-iterations", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-navigable", action="store_true", help="skip the extra navigable-data variant")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run the plain copy kernel on 1 GiB x steps (yardstick for rocprofv3 byte counters) and exit")
     return ap.parse_args()
 
 
@@ -238,6 +240,21 @@ def main():
     from glide_amd import capi
     capi.set_device(0)
     info = capi.device_info()
+
+    if args.copy_calibration:
+        import numpy as np
+        nbytes = 1 << 30
+        src, dst = capi.DeviceArray(nbytes // 4, np.uint32), capi.DeviceArray(nbytes // 4, np.uint32)
+        capi.copy_bytes(dst, src, nbytes)
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record()
+        for _ in range(args.steps):
+            capi.copy_bytes(dst, src, nbytes)
+        e1.record()
+        ms = e0.elapsed_ms(e1) / args.steps
+        print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes, "ms": ms,
+                          "GBps_read_plus_write": 2 * nbytes / ms / 1e6}))
+        return
 
     main_res = run_workload(args, args.workload, torch, want_cpu=not args.no_cpu)
     line = {

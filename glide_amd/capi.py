@@ -275,3 +275,7 @@ def nnd_build(reorder_data, reorder_num, dim, segment_starts, segment_lengths, s
                                     _ptr(segment_lengths), u32(segment_num), u32(knn_degree), u32(iterations),
                                     u32(seed), _ptr(knn_graph), _ptr(workspace), C.c_size_t(workspace_bytes),
                                     _ptr(stats), vp(stream)), "glide_hip_nnd_build")
+
+
+def copy_bytes(dst, src, nbytes, stream=None):
+    check(lib().glide_hip_copy_bytes(_ptr(dst), _ptr(src), C.c_size_t(nbytes), vp(stream)), "glide_hip_copy_bytes")

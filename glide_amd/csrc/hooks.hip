@@ -69,6 +69,13 @@ __global__ __launch_bounds__(64) void hashmap_seq_kernel(uint32_t* table, uint32
     for (uint32_t i = lane; i < (1u << bitlen); i += 64) table[i] = lds_table[i];
 }
 
+// plain streaming copy of known size: the yardstick that hardware byte counters are scaled with
+__global__ __launch_bounds__(256) void copy_kernel(const uint4* src, uint4* dst, size_t n16) {
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
 template <bool MERGE_ONLY>
 int launch_bitonic(float* keys, uint32_t* vals, uint32_t m, uint32_t batch, hipStream_t s) {
     switch (m) {
@@ -93,6 +100,13 @@ int glide_hip_distance_batch(const float* a, const float* b, uint32_t n, uint32_
     if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
     if (n == 0) return GLIDE_OK;
     hipLaunchKernelGGL(distance_batch_kernel, dim3((n + 1) / 2), dim3(64), 0, as_stream(stream), a, b, n, dim, metric, out);
+    return launch_status();
+}
+
+int glide_hip_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {
+    if (!dst || !src || bytes % 16 || reinterpret_cast<uintptr_t>(dst) % 16 || reinterpret_cast<uintptr_t>(src) % 16) return GLIDE_ERR_BAD_ARGUMENT;
+    if (bytes == 0) return GLIDE_OK;
+    hipLaunchKernelGGL(copy_kernel, dim3(8192), dim3(256), 0, as_stream(stream), static_cast<const uint4*>(src), static_cast<uint4*>(dst), bytes / 16);
     return launch_status();
 }
 

@@ -1,0 +1,189 @@
+// class GLIDE<Data_t, Index_t>: the small-path index.  Reference: glide.cuh:14-189, glide_impl.cuh:15-454.
+#pragma once
+#include <fstream>
+#include <iostream>
+#include <optional>
+#include <random>
+#include <string>
+
+#include "mdarray.hpp"
+#include "params.hpp"
+
+namespace glide {
+
+template <typename Data_t, typename Index_t>
+class GLIDE {
+    static_assert(sizeof(Data_t) == 4 && sizeof(Index_t) == 4, "the small path is float / uint32_t (reference mains instantiate only that)");
+
+public:
+    // glide_impl.cuh:15-30
+    GLIDE(device_resources& handle, uint32_t graph_degree, host_matrix_view<Data_t, Index_t> h_data_view,
+          host_matrix_view<float> h_centroid_view, Metric metric)
+        : handle(handle), metric(metric), d_graph(h_data_view.extent(0), graph_degree), d_data(h_data_view.extent(0), h_data_view.extent(1)),
+          d_centroids(h_centroid_view.extent(0), h_centroid_view.extent(1)) {
+        copy_to_device(d_data.data_handle(), h_data_view.data_handle(), h_data_view.size());
+        copy_to_device(d_centroids.data_handle(), h_centroid_view.data_handle(), h_centroid_view.size());
+    }
+
+    // glide_impl.cuh:32-41
+    void load(host_matrix_view<uint32_t, Index_t> h_graph_view, host_vector_view<uint32_t> h_start_point_view) {
+        d_start_points.emplace(h_start_point_view.size());
+        copy_to_device(d_graph.data_handle(), h_graph_view.data_handle(), h_graph_view.size());
+        copy_to_device(d_start_points->data_handle(), h_start_point_view.data_handle(), h_start_point_view.size());
+    }
+
+    // glide_impl.cuh:319-368.  The optionals are consumed.
+    void build(IndexParameter& build_param, SearchParameter& search_param_knn, SearchParameter& search_param_refine,
+               std::optional<device_matrix<uint32_t, Index_t>>& d_knn_graph, std::optional<device_vector<uint32_t>>& d_segment_start,
+               std::optional<device_vector<uint32_t>>& d_segment_length, std::optional<device_vector<uint32_t>>& d_map,
+               host_vector_view<uint32_t> h_segment_start_view, host_vector_view<uint32_t> h_segment_length_view,
+               host_vector_view<uint32_t> h_map_view, std::optional<device_matrix<Data_t, Index_t>>& d_reorder_data, std::string& result_file) {
+        float build_time = 0.0f;
+        host_vector<uint32_t> h_start_point(centroid_num());
+        host_vector<uint32_t> h_reorder_start_point(d_segment_start->size());
+        start_point_select(h_segment_start_view, h_segment_length_view, h_map_view, h_reorder_start_point.view(), h_start_point.view(),
+                           build_param.seed);
+        d_start_points.emplace(h_reorder_start_point.size());
+        copy_to_device(d_start_points->data_handle(), h_reorder_start_point.data_handle(), h_reorder_start_point.size());
+
+        subgraph_build_and_merge(search_param_knn, build_param.relaxant_factor, d_reorder_data->view(), d_map->view(), d_segment_start->view(),
+                                 d_segment_length->view(), d_knn_graph->view(), h_reorder_start_point(centroid_num()), build_time);
+        handle.sync();
+        d_knn_graph.reset();
+        d_segment_start.reset();
+        d_segment_length.reset();
+        d_map.reset();
+        d_reorder_data.reset();
+
+        d_start_points.reset();
+        d_start_points.emplace(h_start_point.size());
+        copy_to_device(d_start_points->data_handle(), h_start_point.data_handle(), h_start_point.size());
+
+        reverse_graph(build_time);
+        if (search_param_refine.beam != 0) refine(search_param_refine, build_param.relaxant_factor, build_time);
+
+        std::cout << "index build time: " << build_time << " s" << std::endl;
+        std::ofstream result_out(result_file, std::ios::app);
+        result_out << build_time << ",";
+    }
+
+    // glide_impl.cuh:370-454
+    void search(SearchParameter& param, device_matrix_view<Data_t> d_query_view, host_matrix<uint32_t>& result_ids,
+                host_matrix<float>& result_dists, std::string& result_file) {
+        const uint32_t query_number = d_query_view.extent(0), top_k = param.top_k;
+        device_matrix<uint32_t> d_result_ids(query_number, top_k);
+        device_matrix<float> d_result_dists(query_number, top_k);
+        gpu_timer timer;
+        timer.start();
+        hip_try(glide_hip_search(d_data.data_handle(), num(), dim(), d_graph.data_handle(), graph_degree(), d_centroids.data_handle(),
+                                 centroid_num(), d_start_points->data_handle(), d_query_view.data_handle(), query_number, top_k, param.beam,
+                                 param.max_iterations, param.min_iterations, param.hash_bit, param.hash_reset_interval, metric_code(metric),
+                                 d_result_ids.data_handle(), d_result_dists.data_handle(), nullptr, handle.stream()),
+                "glide_hip_search");
+        const float seconds = timer.stop();
+        std::cout << "query time: " << seconds << " s" << "   " << "QPS: " << static_cast<float>(query_number) / seconds << std::endl;
+        std::ofstream result;
+        result.setf(std::ios::fixed);
+        result.open(result_file, std::ios::app);
+        result << seconds << "," << static_cast<float>(query_number) / seconds << ",";
+        result.close();
+        copy_to_host(result_ids.data_handle(), d_result_ids.data_handle(), d_result_ids.size());
+        copy_to_host(result_dists.data_handle(), d_result_dists.data_handle(), d_result_dists.size());
+    }
+
+    // accessors (glide.cuh:81-125)
+    uint32_t dim() const { return d_data.extent(1); }
+    Index_t num() const { return d_data.extent(0); }
+    uint32_t graph_degree() const { return d_graph.extent(1); }
+    uint32_t start_point_num() const { return d_start_points->size(); }
+    uint32_t centroid_num() const { return d_centroids.extent(0); }
+    device_matrix_view<Data_t, Index_t> data_view() const { return d_data.view(); }
+    device_vector_view<uint32_t> start_point_view() const { return d_start_points->view(); }
+    device_matrix_view<uint32_t, Index_t> graph_view() const { return d_graph.view(); }
+    device_matrix_view<float> centroid_view() const { return d_centroids.view(); }
+
+private:
+    // glide_impl.cuh:43-75: one random local id per segment; original-id copy for the first centroid_num segments
+    void start_point_select(host_vector_view<uint32_t> h_segment_start_view, host_vector_view<uint32_t> h_segment_length_view,
+                            host_vector_view<uint32_t> h_map_view, host_vector_view<uint32_t> h_reorder_start_points,
+                            host_vector_view<uint32_t> h_start_points, uint32_t seed) {
+        std::mt19937 generator(seed);
+        for (uint32_t i = 0; i < h_segment_start_view.extent(0); i++) {
+            const uint32_t length = h_segment_length_view(i);
+            uint32_t id = 0;
+            if (length > 0) {   // the reference's distribution underflows on an empty segment (glide_impl.cuh:60)
+                std::uniform_int_distribution<uint32_t> dist(0, length - 1);
+                id = dist(generator);
+            }
+            h_reorder_start_points(i) = id;
+            if (i != centroid_num()) h_start_points(i) = length > 0 ? h_map_view(h_segment_start_view(i) + id) : 0;
+        }
+    }
+
+    // glide_impl.cuh:77-192
+    void subgraph_build_and_merge(SearchParameter& param, float relaxant_factor, device_matrix_view<Data_t, Index_t> d_reorder_data_view,
+                                  device_vector_view<uint32_t> d_map_view, device_vector_view<uint32_t> d_segment_start_view,
+                                  device_vector_view<uint32_t> d_segment_length_view, device_matrix_view<uint32_t, Index_t> d_knn_graph_view,
+                                  uint32_t boundary_start_point, float& build_time) {
+        const uint32_t knn_degree = d_knn_graph_view.extent(1), segment_num = d_segment_start_view.extent(0);
+        const uint32_t reorder_num = d_reorder_data_view.extent(0);
+        gpu_timer timer;
+        timer.start();
+        hip_try(glide_hip_build_subgraph(d_reorder_data_view.data_handle(), num(), dim(), d_knn_graph_view.data_handle(), knn_degree,
+                                         d_map_view.data_handle(), d_segment_start_view.data_handle(), d_segment_length_view.data_handle(),
+                                         segment_num, d_start_points->data_handle(), graph_degree(), param.beam, param.max_iterations,
+                                         param.min_iterations, param.hash_bit, param.hash_reset_interval, relaxant_factor,
+                                         metric_code(metric), d_graph.data_handle(), nullptr, handle.stream()),
+                "glide_hip_build_subgraph");
+        build_time += timer.stop();
+        timer.start();
+        hip_try(glide_hip_build_boundary(d_reorder_data_view.data_handle(), num(), reorder_num, dim(), d_knn_graph_view.data_handle(), knn_degree,
+                                         d_map_view.data_handle(), boundary_start_point, graph_degree(), param.beam, param.max_iterations,
+                                         param.min_iterations, param.hash_bit, param.hash_reset_interval, relaxant_factor,
+                                         metric_code(metric), d_graph.data_handle(), nullptr, handle.stream()),
+                "glide_hip_build_boundary");
+        build_time += timer.stop();
+    }
+
+    // glide_impl.cuh:194-256
+    void reverse_graph(float& build_time) {
+        device_matrix<uint32_t> d_reverse_graph(num(), graph_degree());
+        device_vector<uint32_t> d_reverse_graph_degree(num());
+        const size_t wb = glide_hip_reverse_edges_workspace_bytes(num(), graph_degree());
+        device_buffer ws(wb);
+        gpu_timer timer;
+        timer.start();
+        hip_try(glide_hip_reverse_edges(d_graph.data_handle(), num(), graph_degree(), d_reverse_graph.data_handle(),
+                                        d_reverse_graph_degree.data_handle(), ws.get(), wb, handle.stream()),
+                "glide_hip_reverse_edges");
+        build_time += timer.stop();
+        timer.start();
+        hip_try(glide_hip_insert_reverse(d_graph.data_handle(), d_reverse_graph.data_handle(), d_reverse_graph_degree.data_handle(), num(),
+                                         graph_degree(), handle.stream()),
+                "glide_hip_insert_reverse");
+        build_time += timer.stop();
+    }
+
+    // glide_impl.cuh:258-316
+    void refine(SearchParameter& param, float relaxant_factor, float& build_time) {
+        device_matrix<uint32_t, Index_t> d_refined(num(), graph_degree());
+        gpu_timer timer;
+        timer.start();
+        hip_try(glide_hip_refine(d_data.data_handle(), num(), dim(), d_graph.data_handle(), d_refined.data_handle(), graph_degree(),
+                                 d_centroids.data_handle(), centroid_num(), d_start_points->data_handle(), param.beam, param.max_iterations,
+                                 param.min_iterations, param.hash_bit, param.hash_reset_interval, relaxant_factor, metric_code(metric),
+                                 nullptr, handle.stream()),
+                "glide_hip_refine");
+        build_time += timer.stop();
+        d_graph = std::move(d_refined);
+    }
+
+    device_resources& handle;
+    Metric metric;
+    device_matrix<uint32_t, Index_t> d_graph;
+    device_matrix<Data_t, Index_t> d_data;
+    device_matrix<float, uint32_t> d_centroids;
+    std::optional<device_vector<uint32_t>> d_start_points;
+};
+
+}  // namespace glide

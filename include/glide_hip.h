@@ -170,6 +170,9 @@ int glide_hip_refine(const float *data, uint32_t num, uint32_t dim, const uint32
                      int metric, unsigned long long *counters, void *stream);
 
 /* ---- test hooks for the device primitives (subsystems 5, 6 and the hash set) ------------------------------ */
+/* A plain copy kernel (bytes % 16 == 0, 16-byte aligned): no counterpart in the reference; it is the transfer
+ * of known size against which hardware byte counters (FETCH_SIZE / WRITE_SIZE) are calibrated. */
+int glide_hip_copy_bytes(void *dst, const void *src, size_t bytes, void *stream);
 /* compute_similarity_warp (distance.cuh:9-27): out[i] = dist(a[i], b[i]) for n row pairs */
 int glide_hip_distance_batch(const float *a, const float *b, uint32_t n, uint32_t dim, int metric, float *out,
                              void *stream);
