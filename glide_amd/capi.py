@@ -279,3 +279,37 @@ def nnd_build(reorder_data, reorder_num, dim, segment_starts, segment_lengths, s
 
 def copy_bytes(dst, src, nbytes, stream=None):
     check(lib().glide_hip_copy_bytes(_ptr(dst), _ptr(src), C.c_size_t(nbytes), vp(stream)), "glide_hip_copy_bytes")
+
+
+def build_segment(segment_data, num, dim, knn_graph, knn_degree, start_point, graph_degree, beam, max_iterations,
+                  min_iterations, hash_bit, hash_reset_interval, relaxant, metric, graph, counters=None, stream=None):
+    check(lib().glide_hip_build_segment(_ptr(segment_data), u32(num), u32(dim), _ptr(knn_graph), u32(knn_degree),
+                                        u32(start_point), u32(graph_degree), u32(beam), u32(max_iterations),
+                                        u32(min_iterations), u32(hash_bit), u32(hash_reset_interval), f32(relaxant),
+                                        C.c_int(metric), _ptr(graph), _ptr(counters), vp(stream)), "glide_hip_build_segment")
+
+
+def refine_segment(segment_data, num, dim, graph_in, graph_out, graph_degree, start_point, beam, max_iterations,
+                   min_iterations, hash_bit, hash_reset_interval, relaxant, metric, counters=None, stream=None):
+    check(lib().glide_hip_refine_segment(_ptr(segment_data), u32(num), u32(dim), _ptr(graph_in), _ptr(graph_out),
+                                         u32(graph_degree), u32(start_point), u32(beam), u32(max_iterations),
+                                         u32(min_iterations), u32(hash_bit), u32(hash_reset_interval), f32(relaxant),
+                                         C.c_int(metric), _ptr(counters), vp(stream)), "glide_hip_refine_segment")
+
+
+def select_segments(queries, query_num, dim, centroids, centroid_num, min_segment_num, boundary_factor, metric,
+                    segment_ids, stream=None):
+    check(lib().glide_hip_select_segments(_ptr(queries), u32(query_num), u32(dim), _ptr(centroids), u32(centroid_num),
+                                          u32(min_segment_num), f32(boundary_factor), C.c_int(metric),
+                                          _ptr(segment_ids), vp(stream)), "glide_hip_select_segments")
+
+
+def search_sub(segment_data, dim, segment_graph, graph_degree, segment_map, queries, query_num, segment_ids,
+               centroid_num, segment_id, start_point, top_k, beam, max_iterations, min_iterations, hash_bit,
+               hash_reset_interval, metric, final_ids, final_dists, counters=None, stream=None):
+    check(lib().glide_hip_search_sub(_ptr(segment_data), u32(dim), _ptr(segment_graph), u32(graph_degree),
+                                     _ptr(segment_map), _ptr(queries), u32(query_num), _ptr(segment_ids),
+                                     u32(centroid_num), u32(segment_id), u32(start_point), u32(top_k), u32(beam),
+                                     u32(max_iterations), u32(min_iterations), u32(hash_bit), u32(hash_reset_interval),
+                                     C.c_int(metric), _ptr(final_ids), _ptr(final_dists), _ptr(counters), vp(stream)),
+          "glide_hip_search_sub")

@@ -34,8 +34,12 @@ __global__ __launch_bounds__(64) void build_kernel(BuildArgs a) {
     const uint32_t point = a.first_point + blockIdx.x;
     const bool boundary = a.boundary_start != kInvalid;
 
+    const bool segment_mode = a.map == nullptr;   // one staged partition: local ids in and out (build_for_large_kernel)
     uint32_t seg_start, entry;
-    if (boundary) {
+    if (segment_mode) {
+        seg_start = 0;
+        entry = a.boundary_start_point;
+    } else if (boundary) {
         seg_start = a.boundary_start;
         entry = a.boundary_start_point;
     } else {
@@ -59,6 +63,12 @@ __global__ __launch_bounds__(64) void build_kernel(BuildArgs a) {
     prune_pool<MAX_BEAM, DIMV>(pl, pool, a.reorder_data, a.p.dim, seg_start, a.graph_degree, a.relaxant, a.p.metric, b.lane,
                                b.cnt.rows_scored);
     wave_sync();
+    if (segment_mode) {   // map_to_graph (graph_kernel.cuh:145-150)
+        uint32_t* row = a.graph + static_cast<size_t>(point) * a.graph_degree;
+        for (uint32_t i = b.lane; i < a.graph_degree; i += 64) row[i] = pl->neighbor[i];
+        b.flush_counters(a.counters);
+        return;
+    }
     uint32_t* row = a.graph + static_cast<size_t>(a.map[point]) * a.graph_degree;
     if (boundary) {
         merge_boundary_row<MAX_BEAM>(pl, row, a.map, a.graph_degree, b.lane);
@@ -78,7 +88,7 @@ struct RefineArgs {
     const float* centroids;
     const uint32_t* start_points;
     unsigned long long* counters;
-    uint32_t num, centroid_num, max_centroid;
+    uint32_t num, centroid_num, max_centroid, segment_start_point;
     float relaxant;
     BeamParams p;   // p.degree = graph_degree
 };
@@ -123,8 +133,12 @@ __global__ __launch_bounds__(64) void refine_kernel(RefineArgs a) {
 
     Beam<MAX_CAND, MAX_BEAM, DIMV> b;
     b.init(lds, hash, a.p, a.data + static_cast<size_t>(point) * a.p.dim);
-    const uint32_t c0 = pick_centroid_refine<DIMV>(a.max_centroid, b.q, a.centroids, a.centroid_num, a.p.dim, a.p.metric, cent, lane);
-    b.expand(a.start_points[c0], a.graph_in, a.data, kInvalid, kInvalid);
+    if (a.centroids != nullptr) {
+        const uint32_t c0 = pick_centroid_refine<DIMV>(a.max_centroid, b.q, a.centroids, a.centroid_num, a.p.dim, a.p.metric, cent, lane);
+        b.expand(a.start_points[c0], a.graph_in, a.data, kInvalid, kInvalid);
+    } else {   // refine_for_large_kernel (graph_kernel.cuh:796-798): get_init from the segment's start point
+        b.expand(a.segment_start_point, a.graph_in, a.data, kInvalid, point);
+    }
     b.run(a.graph_in, a.data, point);
 
     uint32_t pool = beam_to_pool(b, pl);
@@ -362,6 +376,67 @@ int glide_hip_build_boundary(const float* reorder_data, uint32_t num, uint32_t r
     return launch_build(a, as_stream(stream));
 }
 
+int glide_hip_build_segment(const float* segment_data, uint32_t num, uint32_t dim, const uint32_t* knn_graph, uint32_t knn_degree,
+                            uint32_t start_point, uint32_t graph_degree, uint32_t beam, uint32_t max_iterations, uint32_t min_iterations,
+                            uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant, int metric, uint32_t* graph,
+                            unsigned long long* counters, void* stream) {
+    if (!segment_data || !knn_graph || !graph) return GLIDE_ERR_BAD_ARGUMENT;
+    if (max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    int rc = check_beam_sizes(knn_degree, graph_degree, beam, dim, hash_bit, metric);
+    if (rc != GLIDE_OK) return rc;
+    if (num == 0) return GLIDE_OK;
+    if (start_point >= num) return GLIDE_ERR_BAD_ARGUMENT;
+    BuildArgs a;
+    a.reorder_data = segment_data;
+    a.knn_graph = knn_graph;
+    a.map = nullptr;
+    a.segment_starts = nullptr;
+    a.segment_lengths = nullptr;
+    a.start_points = nullptr;
+    a.graph = graph;
+    a.counters = counters;
+    a.first_point = 0;
+    a.point_count = num;
+    a.segment_num = 0;
+    a.graph_degree = graph_degree;
+    a.boundary_start = kInvalid;
+    a.boundary_start_point = start_point;
+    a.relaxant = relaxant;
+    a.p = BeamParams{beam, knn_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
+    return launch_build(a, as_stream(stream));
+}
+
+int glide_hip_refine_segment(const float* segment_data, uint32_t num, uint32_t dim, const uint32_t* graph_in, uint32_t* graph_out,
+                             uint32_t graph_degree, uint32_t start_point, uint32_t beam, uint32_t max_iterations, uint32_t min_iterations,
+                             uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant, int metric, unsigned long long* counters,
+                             void* stream) {
+    if (!segment_data || !graph_in || !graph_out || graph_in == graph_out) return GLIDE_ERR_BAD_ARGUMENT;
+    if (max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    int rc = check_beam_sizes(graph_degree, graph_degree, beam, dim, hash_bit, metric);
+    if (rc != GLIDE_OK) return rc;
+    if (num == 0) return GLIDE_OK;
+    if (start_point >= num) return GLIDE_ERR_BAD_ARGUMENT;
+    RefineArgs a;
+    a.data = segment_data;
+    a.graph_in = graph_in;
+    a.graph_out = graph_out;
+    a.centroids = nullptr;
+    a.start_points = nullptr;
+    a.counters = counters;
+    a.num = num;
+    a.centroid_num = 0;
+    a.max_centroid = 32;
+    a.segment_start_point = start_point;
+    a.relaxant = relaxant;
+    a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
+    const uint32_t max_cand = graph_degree <= 64 ? 64 : 128;
+    refine_fn fn = max_cand == 64 ? pick_refine_beam<64>(beam, dim) : pick_refine_beam<128>(beam, dim);
+    const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) + prune_lds_bytes(beam) +
+                             (size_t{1} << hash_bit) * sizeof(uint32_t);
+    hipLaunchKernelGGL(fn, dim3(num), dim3(64), lds_bytes, as_stream(stream), a);
+    return launch_status();
+}
+
 size_t glide_hip_reverse_edges_workspace_bytes(uint32_t num, uint32_t graph_degree) {
     const size_t n = num, words = ceil_div(graph_degree, 32);
     // miss bits + offsets + fill (u32 each), cursor (u64, 256-byte slot), pool of (column, source) keys
@@ -426,6 +501,7 @@ int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32
     a.num = num;
     a.centroid_num = centroid_num;
     a.max_centroid = centroid_num <= 32 ? 32 : (graph_degree <= 64 ? 64 : (graph_degree <= 128 ? 128 : 256));
+    a.segment_start_point = 0;
     a.relaxant = relaxant;
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
     const uint32_t max_cand = graph_degree <= 64 ? 64 : 128;

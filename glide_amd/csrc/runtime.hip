@@ -79,6 +79,18 @@ int glide_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream)
     GLIDE_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
     return GLIDE_OK;
 }
+int glide_hip_memcpy_h2d_async(void* dst, const void* src, size_t bytes, void* stream) {
+    GLIDE_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    return GLIDE_OK;
+}
+int glide_hip_memcpy_d2h_async(void* dst, const void* src, size_t bytes, void* stream) {
+    GLIDE_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    return GLIDE_OK;
+}
+int glide_hip_stream_wait_event(void* stream, void* event) {
+    GLIDE_HIP_TRY(hipStreamWaitEvent(as_stream(stream), static_cast<hipEvent_t>(event), 0));
+    return GLIDE_OK;
+}
 int glide_hip_fill_u32(uint32_t* ptr, uint32_t value, size_t count, void* stream) {
     if (!ptr) return GLIDE_ERR_BAD_ARGUMENT;
     if (count == 0) return GLIDE_OK;

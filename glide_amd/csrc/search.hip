@@ -57,7 +57,185 @@ __global__ __launch_bounds__(64) void search_kernel(SearchArgs a) {
     b.flush_counters(a.counters);
 }
 
+// ---- large path: one staged partition at a time ---------------------------------------------------------------
+// select_segment_kernel (search_kernel.cuh:546-607): rank the centroids for each query; keep those within
+// boundary_factor of the nearest, topped up to min_segment_num.  Unlike the reference, which resets only the first
+// output row and leaves the rest uninitialised, every row starts as 0xffffffff.
+struct SelectArgs {
+    const float* queries;
+    const float* centroids;
+    uint32_t* segment_ids;
+    uint32_t query_num, dim, centroid_num, min_segment_num;
+    float boundary_factor;
+    int metric;
+};
+
+template <int MAX_CENTROID>
+__global__ __launch_bounds__(64) void select_segments_kernel(SelectArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* cent_dist = reinterpret_cast<float*>(smem);
+    uint32_t* cent_id = reinterpret_cast<uint32_t*>(cent_dist + round_up32(a.centroid_num));
+    const uint32_t q = blockIdx.x;
+    if (q >= a.query_num) return;
+    const int lane = lane_id();
+    const int half = lane >> 5, t = lane & 31;
+    const float* query = a.queries + static_cast<size_t>(q) * a.dim;
+    for (uint32_t c0 = 0; c0 < a.centroid_num; c0 += 2) {
+        const uint32_t c = c0 + half < a.centroid_num ? c0 + half : c0;
+        float acc = 0.f;
+        for (uint32_t d0 = t * 4; d0 < a.dim; d0 += 128) {
+            RowRegs<1> x, y;
+            x.v[0] = *reinterpret_cast<const float4*>(query + d0);
+            y.v[0] = *reinterpret_cast<const float4*>(a.centroids + static_cast<size_t>(c) * a.dim + d0);
+            acc += partial_sqdist<1>(x, y);
+        }
+        const float d = finish_distance(half_wave_sum(acc), a.metric);
+        if (t == 0 && c0 + half < a.centroid_num) cent_dist[c0 + half] = d;
+    }
+    wave_sync();
+    constexpr int NR = WaveNet<MAX_CENTROID>::NR;
+    constexpr int N32 = MAX_CENTROID / 32;
+    float k[NR];
+    uint32_t v[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        const uint32_t j = (e / N32) + 32 * (e % N32);
+        const bool ok = (MAX_CENTROID >= 64 || lane < 32) && j < a.centroid_num;
+        k[r] = ok ? cent_dist[j] : FLT_MAX;
+        v[r] = ok ? j : kInvalid;
+    }
+    WaveNet<MAX_CENTROID>::sort(k, v, lane);
+    wave_sync();
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        if ((MAX_CENTROID >= 64 || lane < 32) && e < a.centroid_num) {
+            cent_dist[e] = k[r];
+            cent_id[e] = v[r];
+        }
+    }
+    wave_sync();
+    uint32_t* out = a.segment_ids + static_cast<size_t>(q) * a.centroid_num;
+    const float d0 = cent_dist[0];
+    uint32_t allow_num = 0;
+    for (uint32_t base = 0; base < a.centroid_num; base += 64) {
+        const uint32_t i = base + lane;
+        const bool allow = i < a.centroid_num && (cent_dist[i] / d0 <= a.boundary_factor);
+        if (i < a.centroid_num) out[i] = allow ? cent_id[i] : kInvalid;
+        allow_num += __popcll(ballot(allow));
+    }
+    if (allow_num < a.min_segment_num) {
+        const uint32_t need = a.min_segment_num - allow_num;
+        for (uint32_t i = lane; i < need && allow_num + i < a.centroid_num; i += 64) out[allow_num + i] = cent_id[allow_num + i];
+    }
+}
+
+struct SubArgs {
+    const float* data;          // the staged partition
+    const uint32_t* graph;      // partition-local ids
+    const uint32_t* map;        // local id -> original id
+    const float* queries;
+    const uint32_t* segment_ids;
+    uint32_t* final_ids;
+    float* final_dists;
+    unsigned long long* counters;
+    uint32_t query_num, centroid_num, segment_id, start_point, top_k, max_topk;
+    BeamParams p;
+};
+
+// result_merge (search_kernel.cuh:609-651): best top_k of (running result, this partition's beam head)
+template <int MAX_TOPK, int MAX_BEAM>
+__device__ __forceinline__ void merge_result(const float* beam_dist, const uint32_t* beam_id, const uint32_t* map, float* final_dists,
+                                             uint32_t* final_ids, uint32_t top_k, int lane) {
+    constexpr int NR = WaveNet<MAX_TOPK>::NR;
+    const bool live = MAX_TOPK >= 64 || lane < 32;
+    float k[NR];
+    uint32_t v[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        k[r] = (live && e < top_k) ? final_dists[e] : FLT_MAX;
+        v[r] = (live && e < top_k) ? final_ids[e] : kInvalid;
+        const uint32_t kk = MAX_TOPK - 1 - e;
+        if (live && kk < top_k) {
+            const float rk = beam_dist[kk];
+            if (k[r] > rk) {
+                k[r] = rk;
+                v[r] = map[beam_id[kk] & kClean];
+            }
+        }
+    }
+    WaveNet<MAX_TOPK>::merge(k, v, lane);
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        if (live && e < top_k) {
+            final_dists[e] = k[r];
+            final_ids[e] = v[r];
+        }
+    }
+}
+
+// search_on_sub_kernel (search_kernel.cuh:653-765)
+template <int MAX_CAND, int MAX_BEAM, int DIMV>
+__global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    auto* lds = reinterpret_cast<BeamLds<MAX_CAND>*>(smem);
+    float* head_dist = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>));   // beam head staged for the merge (128 pairs)
+    uint32_t* head_id = reinterpret_cast<uint32_t*>(head_dist + 128);
+    uint32_t* hash = head_id + 128;
+    const uint32_t qid = blockIdx.x;
+    if (qid >= a.query_num) return;
+    bool is_search = false;   // wave-uniform scan of this query's partition list
+    for (uint32_t i = 0; i < a.centroid_num; i++) {
+        const uint32_t s = a.segment_ids[static_cast<size_t>(qid) * a.centroid_num + i];
+        if (s == a.segment_id) { is_search = true; break; }
+        if (s == kInvalid) break;
+    }
+    if (!is_search) return;
+
+    Beam<MAX_CAND, MAX_BEAM, DIMV> b;
+    b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
+    b.expand(a.start_point, a.graph, a.data, kInvalid, kInvalid);   // get_init with point_id = 0xffffffff
+    b.run(a.graph, a.data, kInvalid);
+
+    constexpr int NB = MAX_BEAM / 64;
+#pragma unroll
+    for (int r = 0; r < NB; r++) {
+        const uint32_t e = NB * b.lane + r;
+        if (e < 128) {
+            head_dist[e] = b.bk[r];
+            head_id[e] = b.bv[r];
+        }
+    }
+    wave_sync();
+    float* fd = a.final_dists + static_cast<size_t>(qid) * a.top_k;
+    uint32_t* fi = a.final_ids + static_cast<size_t>(qid) * a.top_k;
+    switch (a.max_topk) {   // kernel_config.cuh:312-323
+        case 32: merge_result<32, MAX_BEAM>(head_dist, head_id, a.map, fd, fi, a.top_k, b.lane); break;
+        case 64: merge_result<64, MAX_BEAM>(head_dist, head_id, a.map, fd, fi, a.top_k, b.lane); break;
+        default: merge_result<128, MAX_BEAM>(head_dist, head_id, a.map, fd, fi, a.top_k, b.lane); break;
+    }
+    b.flush_counters(a.counters);
+}
+
 using search_fn = void (*)(SearchArgs);
+using sub_fn = void (*)(SubArgs);
+
+template <int MAX_CAND, int MAX_BEAM>
+sub_fn pick_sub_dim(uint32_t dim) {
+    if (dim <= 128) return search_sub_kernel<MAX_CAND, MAX_BEAM, 1>;
+    if (dim <= 256) return search_sub_kernel<MAX_CAND, MAX_BEAM, 2>;
+    if (dim <= 512) return search_sub_kernel<MAX_CAND, MAX_BEAM, 4>;
+    return search_sub_kernel<MAX_CAND, MAX_BEAM, 8>;
+}
+template <int MAX_CAND>
+sub_fn pick_sub_beam(uint32_t beam, uint32_t dim) {
+    if (beam <= 64) return pick_sub_dim<MAX_CAND, 64>(dim);
+    if (beam <= 128) return pick_sub_dim<MAX_CAND, 128>(dim);
+    return pick_sub_dim<MAX_CAND, 256>(dim);
+}
 
 template <int MAX_CAND, int MAX_BEAM>
 search_fn pick_dim(uint32_t dim) {
@@ -122,6 +300,56 @@ extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, c
     search_fn fn = max_cand == 64 ? pick_beam<64>(beam, dim) : pick_beam<128>(beam, dim);
     const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) +
                              round_up32(centroid_num) * sizeof(float) + (size_t{1} << hash_bit) * sizeof(uint32_t);
+    hipLaunchKernelGGL(fn, dim3(query_num), dim3(64), lds_bytes, as_stream(stream), a);
+    return launch_status();
+}
+
+extern "C" int glide_hip_select_segments(const float* queries, uint32_t query_num, uint32_t dim, const float* centroids, uint32_t centroid_num,
+                                         uint32_t min_segment_num, float boundary_factor, int metric, uint32_t* segment_ids, void* stream) {
+    if (!queries || !centroids || !segment_ids || dim == 0 || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
+    if (centroid_num > 256 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // kernel_config.cuh:290-304
+    if (query_num == 0) return GLIDE_OK;
+    SelectArgs a{queries, centroids, segment_ids, query_num, dim, centroid_num, min_segment_num, boundary_factor, metric};
+    const size_t lds = round_up32(centroid_num) * 8;
+    hipStream_t s = as_stream(stream);
+    if (centroid_num <= 32) hipLaunchKernelGGL(select_segments_kernel<32>, dim3(query_num), dim3(64), lds, s, a);
+    else if (centroid_num <= 64) hipLaunchKernelGGL(select_segments_kernel<64>, dim3(query_num), dim3(64), lds, s, a);
+    else if (centroid_num <= 128) hipLaunchKernelGGL(select_segments_kernel<128>, dim3(query_num), dim3(64), lds, s, a);
+    else hipLaunchKernelGGL(select_segments_kernel<256>, dim3(query_num), dim3(64), lds, s, a);
+    return launch_status();
+}
+
+extern "C" int glide_hip_search_sub(const float* segment_data, uint32_t dim, const uint32_t* segment_graph, uint32_t graph_degree,
+                                    const uint32_t* segment_map, const float* queries, uint32_t query_num, const uint32_t* segment_ids,
+                                    uint32_t centroid_num, uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam,
+                                    uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
+                                    int metric, uint32_t* final_ids, float* final_dists, unsigned long long* counters, void* stream) {
+    if (!segment_data || !segment_graph || !segment_map || !queries || !segment_ids || !final_ids || !final_dists) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim == 0 || graph_degree == 0 || centroid_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
+    if (query_num == 0) return GLIDE_OK;
+    if (graph_degree > 128 || beam > 256 || dim % 4 != 0 || dim > 1024 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
+        return GLIDE_ERR_UNSUPPORTED;   // top_k buckets: kernel_config.cuh:312-323
+    SubArgs a;
+    a.data = segment_data;
+    a.graph = segment_graph;
+    a.map = segment_map;
+    a.queries = queries;
+    a.segment_ids = segment_ids;
+    a.final_ids = final_ids;
+    a.final_dists = final_dists;
+    a.counters = counters;
+    a.query_num = query_num;
+    a.centroid_num = centroid_num;
+    a.segment_id = segment_id;
+    a.start_point = start_point;
+    a.top_k = top_k;
+    a.max_topk = top_k <= 32 ? 32 : (top_k <= 64 ? 64 : 128);
+    a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
+    const uint32_t max_cand = graph_degree <= 64 ? 64 : 128;
+    sub_fn fn = max_cand == 64 ? pick_sub_beam<64>(beam, dim) : pick_sub_beam<128>(beam, dim);
+    const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t);
     hipLaunchKernelGGL(fn, dim3(query_num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }

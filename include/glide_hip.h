@@ -169,6 +169,47 @@ int glide_hip_refine(const float *data, uint32_t num, uint32_t dim, const uint32
                      uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant,
                      int metric, unsigned long long *counters, void *stream);
 
+/* ---- large path: one staged partition at a time (GLIDE_large, glide_large_impl.cuh) ---------------------------
+ * The partition's rows, kNN graph / graph and map are device arrays holding only that partition (ids are
+ * partition-local); the caller stages them (the reference copies each partition from host memory,
+ * glide_large_impl.cuh:109-166).  Data type: float (the reference's large executables instantiate uint8). */
+
+/* Replaces build_for_large_kernel (graph_kernel.cuh:675-728; launch glide_large_impl.cuh:140): sub-graph of one
+ * partition, rows written with partition-local ids. */
+int glide_hip_build_segment(const float *segment_data, uint32_t num, uint32_t dim, const uint32_t *knn_graph,
+                            uint32_t knn_degree, uint32_t start_point, uint32_t graph_degree, uint32_t beam,
+                            uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                            uint32_t hash_reset_interval, float relaxant, int metric, uint32_t *graph,
+                            unsigned long long *counters, void *stream);
+/* Replaces refine_for_large_kernel (graph_kernel.cuh:730-821; launch glide_large_impl.cuh:303): as
+ * glide_hip_refine, searching from the partition's start point. */
+int glide_hip_refine_segment(const float *segment_data, uint32_t num, uint32_t dim, const uint32_t *graph_in,
+                             uint32_t *graph_out, uint32_t graph_degree, uint32_t start_point, uint32_t beam,
+                             uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                             uint32_t hash_reset_interval, float relaxant, int metric,
+                             unsigned long long *counters, void *stream);
+/* Replaces select_segment_kernel (search_kernel.cuh:546-607; launch glide_large_impl.cuh:408): segment_ids is
+ * query_num x centroid_num; row q lists the partitions query q visits (nearest first: those whose centroid
+ * distance is within boundary_factor of the nearest, topped up to min_segment_num), then 0xffffffff. */
+int glide_hip_select_segments(const float *queries, uint32_t query_num, uint32_t dim, const float *centroids,
+                              uint32_t centroid_num, uint32_t min_segment_num, float boundary_factor, int metric,
+                              uint32_t *segment_ids, void *stream);
+/* Replaces search_on_sub_kernel + result_merge (search_kernel.cuh:609-765; launch glide_large_impl.cuh:468): queries
+ * that list `segment_id` search the staged partition and merge its best top_k (mapped to original ids through
+ * segment_map) into final_ids / final_dists (query_num x top_k, initialised by the caller to 0xffffffff /
+ * FLT_MAX before the first partition).  Limits as glide_hip_search, top_k <= 128. */
+int glide_hip_search_sub(const float *segment_data, uint32_t dim, const uint32_t *segment_graph,
+                         uint32_t graph_degree, const uint32_t *segment_map, const float *queries,
+                         uint32_t query_num, const uint32_t *segment_ids, uint32_t centroid_num,
+                         uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam,
+                         uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                         uint32_t hash_reset_interval, int metric, uint32_t *final_ids, float *final_dists,
+                         unsigned long long *counters, void *stream);
+/* asynchronous copies for staging (the caller orders them with streams / events; host memory should be pinned) */
+int glide_hip_memcpy_h2d_async(void *dst, const void *src, size_t bytes, void *stream);
+int glide_hip_memcpy_d2h_async(void *dst, const void *src, size_t bytes, void *stream);
+int glide_hip_stream_wait_event(void *stream, void *event);
+
 /* ---- test hooks for the device primitives (subsystems 5, 6 and the hash set) ------------------------------ */
 /* A plain copy kernel (bytes % 16 == 0, 16-byte aligned): no counterpart in the reference; it is the transfer
  * of known size against which hardware byte counters (FETCH_SIZE / WRITE_SIZE) are calibrated. */

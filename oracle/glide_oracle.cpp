@@ -817,6 +817,167 @@ int go_refine(const float *data, uint32_t num, uint32_t dim, uint32_t *graph, ui
     return 0;
 }
 
+// ----------------------------------------------------------------------------- large path
+// select_segment_kernel search_kernel.cuh:546-607.  The reference resets only the first row of the output and leaves
+// the others uninitialised; every row starts at 0xffffffff here (what the consumer search_kernel.cuh:676-686 expects).
+int go_select_segments(const float *queries, uint32_t query_num, uint32_t dim, const float *centroids,
+                       uint32_t centroid_num, uint32_t min_segment_num, float boundary_factor, int metric,
+                       uint32_t *segment_ids) {
+    const uint32_t maxc = go_max_centroid_partition(centroid_num);   // kernel_config.cuh:290-304
+    if (maxc == 0) return -1;
+    std::vector<uint32_t> ids(centroid_num);
+    std::vector<float> dists(centroid_num);
+    for (uint32_t q = 0; q < query_num; q++) {
+        uint32_t *out = segment_ids + static_cast<size_t>(q) * centroid_num;
+        for (uint32_t i = 0; i < centroid_num; i++) {
+            out[i] = kInvalid;
+            ids[i] = i;
+            dists[i] = dist32(queries + static_cast<size_t>(q) * dim, centroids + static_cast<size_t>(i) * dim, dim, metric);
+        }
+        sort_with_key_value(maxc, centroid_num, ids.data(), dists.data());
+        uint32_t allow_num = 0;
+        for (uint32_t i = 0; i < centroid_num; i++) {
+            if (dists[i] / dists[0] <= boundary_factor) {
+                out[i] = ids[i];
+                allow_num++;
+            }
+        }
+        if (allow_num < min_segment_num) {
+            uint32_t need = min_segment_num - allow_num;
+            for (uint32_t i = 0; i < need && allow_num + i < centroid_num; i++) out[allow_num + i] = ids[allow_num + i];
+        }
+    }
+    return 0;
+}
+
+// search_on_sub_kernel + result_merge search_kernel.cuh:609-765 for one segment; final_* are updated in place
+int go_search_sub(const float *seg_data, uint32_t dim, const uint32_t *seg_graph, uint32_t graph_degree, const uint32_t *seg_map,
+                  const float *queries, uint32_t query_num, const uint32_t *segment_ids, uint32_t centroid_num,
+                  uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam, uint32_t max_iterations,
+                  uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, int metric,
+                  uint32_t *final_ids, float *final_dists, go_stats *stats, int threads) {
+    SearchCfg c;
+    if (!make_cfg(c, beam, graph_degree, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric)) return -1;
+    const uint32_t max_topk = top_k <= 32 ? 32 : top_k <= 64 ? 64 : top_k <= 128 ? 128 : 0;   // kernel_config.cuh:312-323
+    if (max_topk == 0 || top_k > beam) return -1;
+    if (stats) *stats = go_stats{0, 0, 0};
+    threads = set_threads(threads);
+#pragma omp parallel num_threads(threads)
+    {
+        Scratch s;
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t q = 0; q < static_cast<int64_t>(query_num); q++) {
+            bool is_search = false;
+            for (uint32_t i = 0; i < centroid_num; i++) {
+                uint32_t v = segment_ids[static_cast<size_t>(q) * centroid_num + i];
+                if (v == segment_id) { is_search = true; break; }
+                if (v == kInvalid) break;
+            }
+            if (!is_search) continue;
+            const float *query = queries + static_cast<size_t>(q) * dim;
+            s.prepare(c, graph_degree, 0);
+            hash_init(s.hash.data(), c.hash_bit);
+            expand(c, s, query, seg_data, dim, seg_graph, start_point, kInvalid, kInvalid);   // get_init with point_id = max
+            beam_loop(c, s, query, seg_data, dim, seg_graph, kInvalid);
+            // result_merge: half-cleaner against the reversed beam head, then the final merge network
+            const uint32_t N = max_topk / 32;
+            float k[128];
+            uint32_t v[128];
+            float *fd = final_dists + static_cast<size_t>(q) * top_k;
+            uint32_t *fi = final_ids + static_cast<size_t>(q) * top_k;
+            for (uint32_t j = 0; j < max_topk; j++) {
+                k[j] = j < top_k ? fd[j] : FLT_MAX;
+                v[j] = j < top_k ? fi[j] : kInvalid;
+            }
+            for (uint32_t j = 0; j < max_topk; j++) {
+                uint32_t kk = max_topk - 1 - j;
+                if (kk >= top_k) continue;
+                float rk = s.dists[swz(kk)];
+                if (k[j] > rk) {
+                    k[j] = rk;
+                    v[j] = seg_map[s.ids[swz(kk)] & kClean];
+                }
+            }
+            warp_merge(k, v, N, 32);
+            for (uint32_t j = 0; j < top_k; j++) {
+                fd[j] = k[j];
+                fi[j] = v[j];
+            }
+        }
+        add_stats(stats, s.st);
+    }
+    return 0;
+}
+
+// build_for_large_kernel graph_kernel.cuh:675-728: one staged segment, local ids in and out
+int go_build_segment(const float *seg_data, uint32_t num, uint32_t dim, const uint32_t *knn_graph, uint32_t knn_degree,
+                     uint32_t start_point, uint32_t graph_degree, uint32_t beam, uint32_t max_iterations,
+                     uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant, int metric,
+                     uint32_t *graph, go_stats *stats, int threads) {
+    SearchCfg c;
+    if (!make_cfg(c, beam, knn_degree, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric)) return -1;
+    if (stats) *stats = go_stats{0, 0, 0};
+    threads = set_threads(threads);
+#pragma omp parallel num_threads(threads)
+    {
+        Scratch s;
+#pragma omp for schedule(dynamic, 64)
+        for (int64_t pp = 0; pp < static_cast<int64_t>(num); pp++) {
+            uint32_t p = static_cast<uint32_t>(pp);
+            const float *point = seg_data + static_cast<size_t>(p) * dim;
+            s.prepare(c, graph_degree, 0);
+            hash_init(s.hash.data(), c.hash_bit);
+            expand(c, s, point, seg_data, dim, knn_graph, start_point, kInvalid, p);
+            beam_loop(c, s, point, seg_data, dim, knn_graph, p);
+            uint32_t pool = clean_and_compact(c, s);
+            std::fill(s.neighbor.begin(), s.neighbor.end(), kInvalid);
+            sync_prune(seg_data, dim, 0, s.ids.data(), s.dists.data(), pool, graph_degree, relaxant, metric, s.neighbor.data(), &s.st);
+            for (uint32_t i = 0; i < graph_degree; i++) graph[static_cast<size_t>(p) * graph_degree + i] = s.neighbor[i];   // map_to_graph :145-150
+        }
+        add_stats(stats, s.st);
+    }
+    return 0;
+}
+
+// refine_for_large_kernel graph_kernel.cuh:730-821 (entry = the segment's start point), snapshot semantics as go_refine
+int go_refine_segment(const float *seg_data, uint32_t num, uint32_t dim, uint32_t *graph, uint32_t graph_degree,
+                      uint32_t start_point, uint32_t beam, uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                      uint32_t hash_reset_interval, float relaxant, int metric, go_stats *stats, int threads) {
+    SearchCfg c;
+    if (!make_cfg(c, beam, graph_degree, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric)) return -1;
+    if (stats) *stats = go_stats{0, 0, 0};
+    threads = set_threads(threads);
+    std::vector<uint32_t> snap(graph, graph + static_cast<size_t>(num) * graph_degree);
+#pragma omp parallel num_threads(threads)
+    {
+        Scratch s;
+#pragma omp for schedule(dynamic, 64)
+        for (int64_t pp = 0; pp < static_cast<int64_t>(num); pp++) {
+            uint32_t p = static_cast<uint32_t>(pp);
+            const uint32_t *srow = snap.data() + static_cast<size_t>(p) * graph_degree;
+            uint32_t need = 0;
+            for (uint32_t i = 0; i < graph_degree; i++) need += srow[i] == kInvalid;
+            if (need == 0) continue;
+            const float *point = seg_data + static_cast<size_t>(p) * dim;
+            s.prepare(c, graph_degree, 0);
+            for (uint32_t i = 0; i < graph_degree; i++) s.s_graph[i] = srow[i];
+            hash_init(s.hash.data(), c.hash_bit);
+            expand(c, s, point, seg_data, dim, snap.data(), start_point, kInvalid, p);
+            beam_loop(c, s, point, seg_data, dim, snap.data(), p);
+            uint32_t pool = clean_and_compact(c, s);
+            std::fill(s.neighbor.begin(), s.neighbor.end(), kInvalid);
+            sync_prune_refine(seg_data, dim, p, s.ids.data(), s.dists.data(), pool, graph_degree, need, s.s_graph.data(), relaxant,
+                              metric, s.neighbor.data(), &s.st);
+            uint32_t t = 0;
+            uint32_t *row = graph + static_cast<size_t>(p) * graph_degree;
+            for (uint32_t i = 0; i < graph_degree; i++)
+                if (srow[i] == kInvalid) row[i] = s.neighbor[t++];
+        }
+        add_stats(stats, s.st);
+    }
+    return 0;
+}
+
 // ----------------------------------------------------------------------------- brute force + kmeans
 void go_bruteforce_knn(const float *data, uint32_t num, uint32_t dim, const float *queries, uint32_t query_num,
                        uint32_t k, int metric, int exclude_self, uint32_t *ids, float *dists, int threads) {

@@ -113,6 +113,27 @@ int go_refine(const float *data, uint32_t num, uint32_t dim, uint32_t *graph, ui
               uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
               float relaxant, int metric, go_stats *stats, int threads);
 
+/* large path: select_segment_kernel search_kernel.cuh:546-607 (every output row initialised to 0xffffffff) */
+int go_select_segments(const float *queries, uint32_t query_num, uint32_t dim, const float *centroids,
+                       uint32_t centroid_num, uint32_t min_segment_num, float boundary_factor, int metric,
+                       uint32_t *segment_ids);
+/* search_on_sub_kernel + result_merge search_kernel.cuh:609-765 for one segment (final_* updated in place) */
+int go_search_sub(const float *seg_data, uint32_t dim, const uint32_t *seg_graph, uint32_t graph_degree,
+                  const uint32_t *seg_map, const float *queries, uint32_t query_num, const uint32_t *segment_ids,
+                  uint32_t centroid_num, uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam,
+                  uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
+                  int metric, uint32_t *final_ids, float *final_dists, go_stats *stats, int threads);
+/* build_for_large_kernel graph_kernel.cuh:675-728 */
+int go_build_segment(const float *seg_data, uint32_t num, uint32_t dim, const uint32_t *knn_graph, uint32_t knn_degree,
+                     uint32_t start_point, uint32_t graph_degree, uint32_t beam, uint32_t max_iterations,
+                     uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant,
+                     int metric, uint32_t *graph, go_stats *stats, int threads);
+/* refine_for_large_kernel graph_kernel.cuh:730-821 */
+int go_refine_segment(const float *seg_data, uint32_t num, uint32_t dim, uint32_t *graph, uint32_t graph_degree,
+                      uint32_t start_point, uint32_t beam, uint32_t max_iterations, uint32_t min_iterations,
+                      uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant, int metric, go_stats *stats,
+                      int threads);
+
 /* nn_descent.cuh:668-1467 (intended algorithm; per-partition local ids), K-wide rows out */
 int go_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
                  const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,

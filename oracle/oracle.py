@@ -255,6 +255,58 @@ def refine(data, graph, centroids, start_points, sp, relaxant, metric=EUCLIDEAN,
     return g, st.as_dict()
 
 
+def select_segments(queries, centroids, min_segment_num, boundary_factor, metric=EUCLIDEAN):
+    queries, centroids = _f32(queries), _f32(centroids)
+    out = np.empty((queries.shape[0], centroids.shape[0]), dtype=np.uint32)
+    rc = lib().go_select_segments(_p(queries), u32(queries.shape[0]), u32(queries.shape[1]), _p(centroids),
+                                  u32(centroids.shape[0]), u32(min_segment_num), f32(boundary_factor), C.c_int(metric), _p(out))
+    if rc != 0:
+        raise ValueError("oracle select_segments: unsupported parameters")
+    return out
+
+
+def search_sub(seg_data, seg_graph, seg_map, queries, segment_ids, segment_id, start_point, top_k, sp, final_ids, final_dists,
+               metric=EUCLIDEAN, threads=0):
+    seg_data, seg_graph, seg_map, queries = _f32(seg_data), _u32(seg_graph), _u32(seg_map), _f32(queries)
+    segment_ids = _u32(segment_ids)
+    assert final_ids.dtype == np.uint32 and final_dists.dtype == np.float32
+    st = Stats()
+    rc = lib().go_search_sub(_p(seg_data), u32(seg_data.shape[1]), _p(seg_graph), u32(seg_graph.shape[1]), _p(seg_map), _p(queries),
+                             u32(queries.shape[0]), _p(segment_ids), u32(segment_ids.shape[1]), u32(segment_id), u32(start_point),
+                             u32(top_k), u32(sp["beam"]), u32(sp["max_iterations"]), u32(sp["min_iterations"]), u32(sp["hash_bit"]),
+                             u32(sp["hash_reset_interval"]), C.c_int(metric), _p(final_ids), _p(final_dists), C.byref(st),
+                             C.c_int(threads))
+    if rc != 0:
+        raise ValueError("oracle search_sub: unsupported parameters")
+    return st.as_dict()
+
+
+def build_segment(seg_data, knn_graph, start_point, graph_degree, sp, relaxant, metric=EUCLIDEAN, threads=0):
+    seg_data, knn_graph = _f32(seg_data), _u32(knn_graph)
+    graph = np.empty((seg_data.shape[0], graph_degree), dtype=np.uint32)
+    st = Stats()
+    rc = lib().go_build_segment(_p(seg_data), u32(seg_data.shape[0]), u32(seg_data.shape[1]), _p(knn_graph), u32(knn_graph.shape[1]),
+                                u32(start_point), u32(graph_degree), u32(sp["beam"]), u32(sp["max_iterations"]),
+                                u32(sp["min_iterations"]), u32(sp["hash_bit"]), u32(sp["hash_reset_interval"]), f32(relaxant),
+                                C.c_int(metric), _p(graph), C.byref(st), C.c_int(threads))
+    if rc != 0:
+        raise ValueError("oracle build_segment: unsupported parameters")
+    return graph, st.as_dict()
+
+
+def refine_segment(seg_data, graph, start_point, sp, relaxant, metric=EUCLIDEAN, threads=0):
+    seg_data = _f32(seg_data)
+    g = _u32(graph).copy()
+    st = Stats()
+    rc = lib().go_refine_segment(_p(seg_data), u32(seg_data.shape[0]), u32(seg_data.shape[1]), _p(g), u32(g.shape[1]),
+                                 u32(start_point), u32(sp["beam"]), u32(sp["max_iterations"]), u32(sp["min_iterations"]),
+                                 u32(sp["hash_bit"]), u32(sp["hash_reset_interval"]), f32(relaxant), C.c_int(metric), C.byref(st),
+                                 C.c_int(threads))
+    if rc != 0:
+        raise ValueError("oracle refine_segment: unsupported parameters")
+    return g, st.as_dict()
+
+
 def nnd_build(reorder_data, seg_start, seg_len, knn_degree, iterations, seed=0, threads=0):
     reorder_data, seg_start, seg_len = _f32(reorder_data), _u32(seg_start), _u32(seg_len)
     out = np.empty((reorder_data.shape[0], knn_degree), dtype=np.int32)

@@ -1,0 +1,100 @@
+"""Large-path kernels (one staged partition at a time) against the CPU oracle."""
+import numpy as np
+import pytest
+
+from conftest import lowdim_data
+
+pytestmark = pytest.mark.gpu
+INV = 0xFFFFFFFF
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from glide_amd import capi
+    capi.set_device(0)
+    return capi
+
+
+@pytest.fixture(scope="module")
+def large_index():
+    """Three partitions without a boundary list, built by the oracle's large-path functions."""
+    from oracle import oracle as O
+    data = lowdim_data(7000, 128, seed=41)
+    queries = lowdim_data(250, 128, seed=42)
+    cent = O.kmeans(data[::3], 3, iterations=8)
+    idx, lens, _ = O.partition_assign(data, cent, 0.0)             # factor 0: nobody is a boundary point
+    assert lens[3] == 0
+    starts = O.segment_starts(lens)
+    rdata, mp = O.reorder(data, idx, starts, 7000)
+    knn = O.nnd_build(rdata, starts[:3], lens[:3], 32, 6).astype(np.uint32)
+    sp_b, sp_r = O.search_params(64, 32), O.search_params(128, 32)
+    rng = np.random.default_rng(0)
+    start_points = np.array([rng.integers(0, l) for l in lens[:3]], np.uint32)
+    segs = []
+    for s in range(3):
+        a, l = int(starts[s]), int(lens[s])
+        g0, st0 = O.build_segment(rdata[a:a + l], knn[a:a + l], int(start_points[s]), 32, sp_b, 1.05)
+        g1 = O.reverse_edges(g0)
+        g2, st2 = O.refine_segment(rdata[a:a + l], g1, int(start_points[s]), sp_r, 1.05)
+        segs.append(dict(data=rdata[a:a + l], knn=knn[a:a + l], map=mp[a:a + l], built=g0, st_built=st0, rev=g1, graph=g2, st_ref=st2))
+    return dict(data=data, queries=queries, cent=cent, segs=segs, start_points=start_points, sp_b=sp_b, sp_r=sp_r)
+
+
+def test_build_and_refine_segment_bit_exact(hip, large_index):
+    L = large_index
+    for s, seg in enumerate(L["segs"]):
+        n = seg["data"].shape[0]
+        d_data, d_knn = hip.DeviceArray.from_numpy(seg["data"]), hip.DeviceArray.from_numpy(seg["knn"])
+        g = hip.DeviceArray.full((n, 32), 0xDEADBEEF)
+        cnt = hip.DeviceArray.from_numpy(np.zeros(3, np.uint64))
+        p = L["sp_b"]
+        hip.build_segment(d_data, n, 128, d_knn, 32, int(L["start_points"][s]), 32, p["beam"], p["max_iterations"], p["min_iterations"],
+                          p["hash_bit"], p["hash_reset_interval"], 1.05, 0, g, cnt)
+        hip.synchronize()
+        assert np.array_equal(g.numpy(), seg["built"])
+        st = seg["st_built"]
+        assert cnt.numpy().tolist() == [st["iterations"], st["rows_scored"], st["graph_rows"]]
+        g_in, g_out = hip.DeviceArray.from_numpy(seg["rev"]), hip.DeviceArray.full((n, 32), 0xDEADBEEF)
+        p = L["sp_r"]
+        hip.refine_segment(d_data, n, 128, g_in, g_out, 32, int(L["start_points"][s]), p["beam"], p["max_iterations"], p["min_iterations"],
+                           p["hash_bit"], p["hash_reset_interval"], 1.05, 0)
+        hip.synchronize()
+        assert np.array_equal(g_out.numpy(), seg["graph"])
+
+
+@pytest.mark.parametrize("c,min_seg,bf", [(3, 1, 1.2), (3, 2, 1.0), (40, 3, 1.1), (200, 5, 1.05), (7, 7, 1.0)])
+def test_select_segments_bit_exact(hip, c, min_seg, bf):
+    from oracle import oracle as O
+    data = lowdim_data(3000, 128, seed=c)
+    queries = np.rint(lowdim_data(200, 128, seed=c + 1))
+    cent = np.rint(data[np.random.default_rng(c).permutation(3000)[:c]])        # integer centroids: exact distances
+    want = O.select_segments(queries, cent, min_seg, bf)
+    d_q, d_c = hip.DeviceArray.from_numpy(queries), hip.DeviceArray.from_numpy(cent)
+    out = hip.DeviceArray.full((200, c), 0x12345678)
+    hip.select_segments(d_q, 200, 128, d_c, c, min_seg, bf, 0, out)
+    hip.synchronize()
+    assert np.array_equal(out.numpy(), want)
+    assert ((want != INV).sum(1) >= min(min_seg, c)).all()
+
+
+@pytest.mark.parametrize("top_k,beam", [(10, 64), (40, 128), (100, 256)])
+def test_search_over_partitions_bit_exact(hip, large_index, top_k, beam):
+    from glide_amd.datasets import recall
+    from oracle import oracle as O
+    L = large_index
+    nq = L["queries"].shape[0]
+    sp = O.search_params(beam, 32)
+    seg_ids = O.select_segments(L["queries"], L["cent"], 2, 1.1)
+    e_ids, e_d = np.full((nq, top_k), INV, np.uint32), np.full((nq, top_k), np.finfo(np.float32).max, np.float32)
+    d_q, d_seg = hip.DeviceArray.from_numpy(L["queries"]), hip.DeviceArray.from_numpy(seg_ids)
+    g_ids, g_d = hip.DeviceArray.from_numpy(e_ids), hip.DeviceArray.from_numpy(e_d)
+    for s, seg in enumerate(L["segs"]):
+        O.search_sub(seg["data"], seg["graph"], seg["map"], L["queries"], seg_ids, s, int(L["start_points"][s]), top_k, sp, e_ids, e_d)
+        d_data, d_graph, d_map = hip.DeviceArray.from_numpy(seg["data"]), hip.DeviceArray.from_numpy(seg["graph"]), hip.DeviceArray.from_numpy(seg["map"])
+        hip.search_sub(d_data, 128, d_graph, 32, d_map, d_q, nq, d_seg, 3, s, int(L["start_points"][s]), top_k, sp["beam"],
+                       sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 0, g_ids, g_d)
+        hip.synchronize()
+        assert np.array_equal(g_ids.numpy(), e_ids), s
+        assert np.array_equal(g_d.numpy(), e_d), s
+    gt, _ = O.bruteforce_knn(L["data"], L["queries"], 10)
+    assert recall(e_ids[:, :10], gt, 10) >= 0.9          # two partitions per query
