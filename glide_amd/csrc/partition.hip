@@ -252,7 +252,8 @@ __global__ __launch_bounds__(kTilePoints) void slot_kernel(uint32_t* segment_ind
 
 // reorder_kernel (partition_kernel.cuh:68-100): one wavefront per point
 __global__ __launch_bounds__(256) void reorder_kernel(const float* data, float* reorder_data, const uint32_t* segment_indexes,
-                                                      uint32_t* map, const uint32_t* segment_starts, uint32_t num, uint32_t dim) {
+                                                      uint32_t* map, const uint32_t* segment_starts, uint32_t num, uint32_t dim,
+                                                      uint32_t point_id_offset) {
     const int lane = lane_id();
     const uint32_t p = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (p >= num) return;
@@ -269,8 +270,8 @@ __global__ __launch_bounds__(256) void reorder_kernel(const float* data, float* 
         if (bdst) *reinterpret_cast<float4*>(bdst + d0) = v;
     }
     if (lane == 0) {
-        map[rid] = p;
-        if (bdst) map[num + bslot] = p;
+        map[rid] = p + point_id_offset;
+        if (bdst) map[num + bslot] = p + point_id_offset;
     }
 }
 
@@ -373,14 +374,19 @@ int glide_hip_partition_assign(const float* data, uint32_t num, uint32_t dim, co
     return launch_status();
 }
 
-int glide_hip_reorder(const float* data, uint32_t num, uint32_t dim, const uint32_t* segment_indexes, const uint32_t* segment_starts,
-                      float* reorder_data, uint32_t* map, void* stream) {
+int glide_hip_reorder_batch(const float* data, uint32_t num, uint32_t dim, const uint32_t* segment_indexes, const uint32_t* segment_starts,
+                            uint32_t point_id_offset, float* reorder_data, uint32_t* map, void* stream) {
     if (!data || !segment_indexes || !segment_starts || !reorder_data || !map || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
     if (num == 0) return GLIDE_OK;
     hipLaunchKernelGGL(reorder_kernel, dim3(ceil_div(num, 4)), dim3(256), 0, as_stream(stream), data, reorder_data, segment_indexes, map,
-                       segment_starts, num, dim);
+                       segment_starts, num, dim, point_id_offset);
     return launch_status();
+}
+
+int glide_hip_reorder(const float* data, uint32_t num, uint32_t dim, const uint32_t* segment_indexes, const uint32_t* segment_starts,
+                      float* reorder_data, uint32_t* map, void* stream) {
+    return glide_hip_reorder_batch(data, num, dim, segment_indexes, segment_starts, 0u, reorder_data, map, stream);
 }
 
 int glide_hip_sample_rows(const float* data, uint32_t dim, const uint32_t* sample_ids, uint32_t sample_num, float* sample, void* stream) {

@@ -1,0 +1,196 @@
+// class GLIDE_large: data, graph and map live in pinned host memory; one partition at a time is staged through the
+// GPU.  Reference: glide_large.cuh:14-212, glide_large_impl.cuh:14-507 (instantiated there for uint8 rows; float here).
+// Partitions are independent on this path (no boundary list, no cross-partition merge), so build -> reverse edges ->
+// refine run back to back on a staged partition instead of in three passes over the host arrays, and the copy of
+// the next partition overlaps the kernels of the current one.
+#pragma once
+#include <cfloat>
+#include <fstream>
+#include <iostream>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "load.hpp"
+#include "mdarray.hpp"
+#include "params.hpp"
+#include "pinned.hpp"
+
+namespace glide {
+
+template <typename Data_t, typename Index_t>
+class GLIDE_large {
+    static_assert(sizeof(Data_t) == 4, "float rows");
+
+public:
+    // glide_large_impl.cuh:14-28: an index to be built
+    GLIDE_large(device_resources& handle, uint32_t graph_degree, Metric metric, std::string& reorder_file, std::string& map_file,
+                std::string& centroid_file, std::string& segment_file)
+        : handle(handle), metric(metric), h_data(load_matrix_pinned<Data_t>(reorder_file)), h_map(load_vector_data(map_file)),
+          h_centroids(load_matrix_data<float, uint32_t>(centroid_file)), h_segment_start(load_segment_start(segment_file)),
+          h_segment_length(load_segment_length(segment_file)), h_start_point(h_segment_start.size()), h_graph(h_data.extent(0), graph_degree) {}
+    // glide_large_impl.cuh:29-43: a finished index
+    GLIDE_large(device_resources& handle, Metric metric, std::string& reorder_file, std::string& map_file, std::string& centroid_file,
+                std::string& segment_file, std::string& start_point_file, std::string& graph_file)
+        : handle(handle), metric(metric), h_data(load_matrix_pinned<Data_t>(reorder_file)), h_map(load_vector_data(map_file)),
+          h_centroids(load_matrix_data<float, uint32_t>(centroid_file)), h_segment_start(load_segment_start(segment_file)),
+          h_segment_length(load_segment_length(segment_file)), h_start_point(load_vector_data(start_point_file)),
+          h_graph(load_matrix_pinned<uint32_t>(graph_file)) {}
+
+    uint32_t dim() const { return h_data.extent(1); }
+    Index_t num() const { return h_data.extent(0); }
+    uint32_t graph_degree() const { return h_graph.extent(1); }
+    uint32_t segment_num() const { return h_segment_start.size(); }
+    uint32_t centroids_num() const { return h_centroids.extent(0); }
+    const pinned_matrix<uint32_t>& graph_view() const { return h_graph; }
+    host_vector_view<const uint32_t> start_point_view() const { return h_start_point.view(); }
+
+    // glide_large_impl.cuh:328-345
+    void build(IndexParameter& build_param, SearchParameter& search_param_knn, SearchParameter& search_param_refine,
+               const pinned_matrix<uint32_t>& h_knn_graph, std::string& result_file) {
+        std::mt19937 generator(build_param.seed);   // start_point_select (glide_large_impl.cuh:55-76)
+        for (uint32_t i = 0; i < segment_num(); i++) {
+            const uint32_t len = h_segment_length(i);
+            h_start_point(i) = len ? std::uniform_int_distribution<uint32_t>(0, len - 1)(generator) : 0;
+        }
+        const uint32_t knn_degree = h_knn_graph.extent(1), deg = graph_degree();
+        uint32_t max_len = 0;
+        for (uint32_t s = 0; s < segment_num(); s++) max_len = std::max(max_len, h_segment_length(s));
+        device_matrix<float> d_data[2] = {device_matrix<float>(max_len, dim()), device_matrix<float>(max_len, dim())};
+        device_matrix<uint32_t> d_knn[2] = {device_matrix<uint32_t>(max_len, knn_degree), device_matrix<uint32_t>(max_len, knn_degree)};
+        device_matrix<uint32_t> d_graph(max_len, deg), d_rev(max_len, deg);
+        device_vector<uint32_t> d_rev_count(max_len);
+        const size_t wb = glide_hip_reverse_edges_workspace_bytes(max_len, deg);
+        device_buffer ws(wb);
+        const int mc = metric_code(metric);
+        stager st;
+        auto stage = [&](uint32_t s) {
+            const int b = s & 1;
+            const size_t start = h_segment_start(s), len = h_segment_length(s);
+            st.before_copy(b);
+            hip_try(glide_hip_memcpy_h2d_async(d_data[b].data_handle(), h_data.row(start), len * dim() * sizeof(float), st.copy_stream()), "h2d data");
+            hip_try(glide_hip_memcpy_h2d_async(d_knn[b].data_handle(), h_knn_graph.row(start), len * knn_degree * sizeof(uint32_t), st.copy_stream()), "h2d knn");
+            st.after_copy(b);
+        };
+        void* t0 = nullptr;
+        void* t1 = nullptr;
+        hip_try(glide_hip_event_create(&t0), "glide_hip_event_create");
+        hip_try(glide_hip_event_create(&t1), "glide_hip_event_create");
+        void* cs = st.compute_stream();
+        hip_try(glide_hip_event_record(t0, cs), "glide_hip_event_record");
+        if (segment_num()) stage(0);
+        for (uint32_t s = 0; s < segment_num(); s++) {
+            const int b = s & 1;
+            const uint32_t len = h_segment_length(s);
+            if (s + 1 < segment_num()) stage(s + 1);
+            st.before_compute(b);
+            SearchParameter& p = search_param_knn;
+            hip_try(glide_hip_build_segment(d_data[b].data_handle(), len, dim(), d_knn[b].data_handle(), knn_degree, h_start_point(s), deg, p.beam,
+                                            p.max_iterations, p.min_iterations, p.hash_bit, p.hash_reset_interval, build_param.relaxant_factor, mc,
+                                            d_graph.data_handle(), nullptr, cs),
+                    "glide_hip_build_segment");
+            hip_try(glide_hip_reverse_edges(d_graph.data_handle(), len, deg, d_rev.data_handle(), d_rev_count.data_handle(), ws.get(), wb, cs),
+                    "glide_hip_reverse_edges");
+            hip_try(glide_hip_insert_reverse(d_graph.data_handle(), d_rev.data_handle(), d_rev_count.data_handle(), len, deg, cs),
+                    "glide_hip_insert_reverse");
+            const uint32_t* result = d_graph.data_handle();
+            if (search_param_refine.beam != 0) {
+                SearchParameter& r = search_param_refine;
+                hip_try(glide_hip_refine_segment(d_data[b].data_handle(), len, dim(), d_graph.data_handle(), d_rev.data_handle(), deg, h_start_point(s),
+                                                 r.beam, r.max_iterations, r.min_iterations, r.hash_bit, r.hash_reset_interval,
+                                                 build_param.relaxant_factor, mc, nullptr, cs),
+                        "glide_hip_refine_segment");
+                result = d_rev.data_handle();
+            }
+            hip_try(glide_hip_memcpy_d2h_async(h_graph.row(h_segment_start(s)), result, static_cast<size_t>(len) * deg * sizeof(uint32_t), cs), "d2h graph");
+            st.after_compute(b);
+        }
+        hip_try(glide_hip_event_record(t1, cs), "glide_hip_event_record");
+        st.sync();
+        float ms = 0.f;
+        hip_try(glide_hip_event_elapsed_ms(t0, t1, &ms), "glide_hip_event_elapsed_ms");
+        glide_hip_event_destroy(t0);
+        glide_hip_event_destroy(t1);
+        const float build_time = ms / 1000.0f;
+        std::cout << "index build time: " << build_time << " s" << std::endl;
+        std::ofstream result_out(result_file, std::ios::app);
+        result_out << build_time << ",";
+    }
+
+    // glide_large_impl.cuh:347-507
+    void search(SearchParameter& param, uint32_t min_segment_num, float boundary_factor, device_matrix_view<Data_t> d_query_view,
+                host_matrix_view<uint32_t> h_result_ids_view, host_matrix_view<float> h_result_distances_view, std::string& result_file) {
+        const uint32_t query_number = d_query_view.extent(0), top_k = param.top_k, deg = graph_degree(), c = centroids_num();
+        device_matrix<uint32_t> d_final_ids(query_number, top_k), d_segment_ids(query_number, c);
+        device_matrix<float> d_final_dists(query_number, top_k), d_centroids(c, dim());
+        copy_to_device(d_centroids.data_handle(), h_centroids.data_handle(), h_centroids.size());
+        uint32_t max_len = 0;
+        for (uint32_t s = 0; s < segment_num(); s++) max_len = std::max(max_len, h_segment_length(s));
+        device_matrix<float> d_data[2] = {device_matrix<float>(max_len, dim()), device_matrix<float>(max_len, dim())};
+        device_matrix<uint32_t> d_graph[2] = {device_matrix<uint32_t>(max_len, deg), device_matrix<uint32_t>(max_len, deg)};
+        device_vector<uint32_t> d_map[2] = {device_vector<uint32_t>(max_len), device_vector<uint32_t>(max_len)};
+        const int mc = metric_code(metric);
+        stager st;
+        void* cs = st.compute_stream();
+        auto stage = [&](uint32_t s) {
+            const int b = s & 1;
+            const size_t start = h_segment_start(s), len = h_segment_length(s);
+            st.before_copy(b);
+            hip_try(glide_hip_memcpy_h2d_async(d_data[b].data_handle(), h_data.row(start), len * dim() * sizeof(float), st.copy_stream()), "h2d data");
+            hip_try(glide_hip_memcpy_h2d_async(d_graph[b].data_handle(), h_graph.row(start), len * deg * sizeof(uint32_t), st.copy_stream()), "h2d graph");
+            hip_try(glide_hip_memcpy_h2d_async(d_map[b].data_handle(), h_map.data_handle() + start, len * sizeof(uint32_t), st.copy_stream()), "h2d map");
+            st.after_copy(b);
+        };
+        void* t0 = nullptr;
+        void* t1 = nullptr;
+        hip_try(glide_hip_event_create(&t0), "glide_hip_event_create");
+        hip_try(glide_hip_event_create(&t1), "glide_hip_event_create");
+        hip_try(glide_hip_fill_u32(d_final_ids.data_handle(), 0xffffffffu, d_final_ids.size(), cs), "glide_hip_fill_u32");
+        const float fmax = FLT_MAX;
+        uint32_t fmax_bits;
+        std::memcpy(&fmax_bits, &fmax, 4);
+        hip_try(glide_hip_fill_u32(reinterpret_cast<uint32_t*>(d_final_dists.data_handle()), fmax_bits, d_final_dists.size(), cs), "glide_hip_fill_u32");
+        hip_try(glide_hip_event_record(t0, cs), "glide_hip_event_record");
+        hip_try(glide_hip_select_segments(d_query_view.data_handle(), query_number, dim(), d_centroids.data_handle(), c, min_segment_num,
+                                          boundary_factor, mc, d_segment_ids.data_handle(), cs),
+                "glide_hip_select_segments");
+        if (segment_num()) stage(0);
+        for (uint32_t s = 0; s < segment_num(); s++) {
+            const int b = s & 1;
+            if (s + 1 < segment_num()) stage(s + 1);
+            st.before_compute(b);
+            hip_try(glide_hip_search_sub(d_data[b].data_handle(), dim(), d_graph[b].data_handle(), deg, d_map[b].data_handle(),
+                                         d_query_view.data_handle(), query_number, d_segment_ids.data_handle(), c, s, h_start_point(s), top_k,
+                                         param.beam, param.max_iterations, param.min_iterations, param.hash_bit, param.hash_reset_interval, mc,
+                                         d_final_ids.data_handle(), d_final_dists.data_handle(), nullptr, cs),
+                    "glide_hip_search_sub");
+            st.after_compute(b);
+        }
+        hip_try(glide_hip_event_record(t1, cs), "glide_hip_event_record");
+        st.sync();
+        float ms = 0.f;
+        hip_try(glide_hip_event_elapsed_ms(t0, t1, &ms), "glide_hip_event_elapsed_ms");
+        glide_hip_event_destroy(t0);
+        glide_hip_event_destroy(t1);
+        const float search_time = ms / 1000.0f;   // staging included: this is what a caller of the host-resident index sees
+        std::cout << "query time: " << search_time << " s" << "   " << "QPS: " << static_cast<float>(query_number) / search_time << std::endl;
+        std::ofstream result;
+        result.setf(std::ios::fixed);
+        result.open(result_file, std::ios::app);
+        result << search_time << "," << static_cast<float>(query_number) / search_time << ",";
+        result.close();
+        copy_to_host(h_result_ids_view.data_handle(), d_final_ids.data_handle(), d_final_ids.size());
+        copy_to_host(h_result_distances_view.data_handle(), d_final_dists.data_handle(), d_final_dists.size());
+    }
+
+private:
+    device_resources& handle;
+    Metric metric;
+    pinned_matrix<Data_t> h_data;
+    host_vector<uint32_t> h_map;
+    host_matrix<float> h_centroids;
+    host_vector<uint32_t> h_segment_start, h_segment_length, h_start_point;
+    pinned_matrix<uint32_t> h_graph;
+};
+
+}  // namespace glide

@@ -1,0 +1,46 @@
+// large_preprocess data_file preprocess_file result_file centroid_num sample_factor metric
+// Reference: large_preprocess.cu:21-80 (same argv and output files; float rows here, uint8 there).
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+#include <string>
+
+#include "load.hpp"
+#include "partition_large.hpp"
+
+using namespace glide;
+
+int main(int argc, char** argv) {
+    if (argc != 7) {
+        std::cout << argv[0] << " data_file preprocess_file result_file centroid_num sample_factor metric" << std::endl;
+        exit(-1);
+    }
+    device_resources handle(std::getenv("GLIDE_DEVICE") ? std::atoi(std::getenv("GLIDE_DEVICE")) : 0);
+    std::string data_file(argv[1]), preprocess_file(argv[2]), result_file(argv[3]);
+    PartitionParameter param;
+    param.centroid_num = std::stoi(argv[4]);
+    param.sample_factor = std::stof(argv[5]);
+    std::string metric(argv[6]);
+    param.metric = metric == "Cosine" ? Metric::Cosine : Metric::Euclidean;
+    const uint32_t batch_num = 10;   // large_preprocess.cu:66
+
+    std::ifstream probe(result_file);
+    if (!probe.good()) {
+        std::ofstream result_out(result_file, std::ios::app);
+        result_out << "pre_time,knn_time,degree,index_time,beam,search_time,QPS,recall" << std::endl;
+    }
+    auto h_data = load_matrix_pinned<float>(data_file);
+    const size_t num = h_data.extent(0), dim = h_data.extent(1);
+    pinned_matrix<float> h_reorder(num, dim);
+    host_vector<uint32_t> h_map(num), h_segment_start(param.centroid_num), h_segment_length(param.centroid_num);
+    device_matrix<float> d_centroids(param.centroid_num, dim);
+    preprocess_for_large<float>(handle, param, h_data, h_reorder, h_map.view(), h_segment_start.view(), h_segment_length.view(), d_centroids.view(),
+                                batch_num, result_file);
+    host_matrix<float> h_centroids(param.centroid_num, dim);
+    copy_to_host(h_centroids.data_handle(), d_centroids.data_handle(), h_centroids.size());
+    save_matrix_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view());
+    save_segment(preprocess_file + ".segment", std::as_const(h_segment_start).view(), std::as_const(h_segment_length).view());
+    save_vector_data(preprocess_file + ".map", std::as_const(h_map).view());
+    save_matrix_pinned(preprocess_file + ".reorder", h_reorder);
+    return 0;
+}

@@ -89,6 +89,13 @@ int glide_hip_partition_assign(const float *data, uint32_t num, uint32_t dim, co
 int glide_hip_reorder(const float *data, uint32_t num, uint32_t dim, const uint32_t *segment_indexes,
                       const uint32_t *segment_starts, float *reorder_data, uint32_t *map, void *stream);
 
+/* Batched form for data sets staged through the GPU in pieces (replaces reorder_for_large_kernel,
+ * partition_kernel.cuh:164-193; partition.cuh:339-415): `data` holds `num` rows of one batch, segment_starts the
+ * offsets of the segments inside this batch's output buffer, and map receives point_id_offset + row. */
+int glide_hip_reorder_batch(const float *data, uint32_t num, uint32_t dim, const uint32_t *segment_indexes,
+                            const uint32_t *segment_starts, uint32_t point_id_offset, float *reorder_data,
+                            uint32_t *map, void *stream);
+
 /* Replaces sample_kernel (partition_kernel.cuh:7-20; partition.cuh:31-45): sample[i] = data[sample_ids[i]]. */
 int glide_hip_sample_rows(const float *data, uint32_t dim, const uint32_t *sample_ids, uint32_t sample_num,
                           float *sample, void *stream);

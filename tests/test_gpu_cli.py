@@ -81,3 +81,60 @@ def test_small_pipeline_cli(tmp_path):
 def test_cli_usage_error():
     r = subprocess.run([os.path.join(BIN, "small_search")], capture_output=True, text=True)
     assert r.returncode != 0 and "data_file" in r.stdout      # exit(-1) on a bad argument count, like the reference
+
+
+def test_large_pipeline_cli(tmp_path):
+    """large_* executables: host-resident data staged partition by partition; every stage checked against the oracle."""
+    from glide_amd import datasets as D
+    from oracle import oracle as O
+    n, dim, nq, c = 9003, 128, 200, 5          # not a multiple of the 10 preprocessing batches
+    data, queries = lowdim_data(n, dim, seed=51), lowdim_data(nq, dim, seed=52)
+    truth, _ = O.bruteforce_knn(data, queries, 100)
+    f = lambda name: str(tmp_path / name)
+    D.write_fbin(f("base.fbin"), data)
+    D.write_fbin(f("query.fbin"), queries)
+    D.write_fbin(f("truth"), truth.astype(np.uint32))
+    pre, knn_file, graph_base, result = f("pre"), f("knn"), f("graph"), f("result.csv")
+
+    run(os.path.join(BIN, "large_preprocess"), f("base.fbin"), pre, result, c, 0.05, "Euclidean")
+    centroids = D.read_fbin(pre + ".centroid")
+    starts, lengths = D.read_segment(pre + ".segment")
+    mp = D.read_vector(pre + ".map")
+    rdata = D.read_fbin(pre + ".reorder")
+    assert starts.size == c and lengths.sum() == n and rdata.shape == (n, dim)      # no boundary list on this path
+    e_idx, e_len, near = O.partition_assign(data, centroids, 0.0)
+    if (np.abs(near[:, 1] / near[:, 0] - 1) > 1e-4).all():
+        assert np.array_equal(e_len[:c], lengths)
+        e_rdata, e_map = O.reorder(data, e_idx, O.segment_starts(e_len), n)
+        assert np.array_equal(e_map, mp) and np.array_equal(e_rdata, rdata)       # rows keep input order inside a partition
+    assert np.array_equal(rdata, data[mp])
+
+    run(os.path.join(BIN, "large_knn"), pre, knn_file, result, 32)
+    knn = D.read_fbin(knn_file, np.uint32)
+    assert knn.shape == (n, 32)
+    for s, l in zip(starts.tolist(), lengths.tolist()):
+        assert (knn[s:s + l] < l).all()
+    s, l = int(starts[1]), int(lengths[1])
+    gt, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + 200], 32, exclude_self=True)
+    assert D.recall(knn[s:s + 200], gt, 32) >= 0.95
+
+    run(os.path.join(BIN, "large_build"), pre, knn_file, graph_base, result, "Euclidean", 32, 32, 1.05, 64, 128)
+    graph = D.read_fbin(graph_base + ".graph", np.uint32)
+    sp = D.read_vector(graph_base + ".sp")
+    assert graph.shape == (n, 32) and sp.size == c
+    sp_b, sp_r = O.search_params(64, 32), O.search_params(128, 32)
+    for i, (s, l) in enumerate(zip(starts.tolist(), lengths.tolist())):            # bit-exact per partition
+        g0, _ = O.build_segment(rdata[s:s + l], knn[s:s + l], int(sp[i]), 32, sp_b, 1.05)
+        g2, _ = O.refine_segment(rdata[s:s + l], O.reverse_edges(g0), int(sp[i]), sp_r, 1.05)
+        assert np.array_equal(graph[s:s + l], g2), i
+
+    out = run(os.path.join(BIN, "large_search"), pre, f("query.fbin"), f("truth"), graph_base, result, "Euclidean", 10, 50, 2, 1.1)
+    recall = float(out.split("total_recall:")[1].split()[0])
+    seg_ids = O.select_segments(queries, centroids, 2, 1.1)
+    e_ids, e_d = np.full((nq, 10), 0xFFFFFFFF, np.uint32), np.full((nq, 10), np.finfo(np.float32).max, np.float32)
+    spp = O.search_params(50, 32)
+    for i, (s, l) in enumerate(zip(starts.tolist(), lengths.tolist())):
+        O.search_sub(rdata[s:s + l], graph[s:s + l], mp[s:s + l], queries, seg_ids, i, int(sp[i]), 10, spp, e_ids, e_d)
+    assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= 0.9
+    row = open(result).read().strip().splitlines()[1].split(",")
+    assert len(row) == 8
