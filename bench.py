@@ -147,10 +147,10 @@ def run_workload(args, workload, torch, want_cpu):
     sweep = []
     for beam in (32, 64, 128, 256):
         sp = G.make_search_parameter(beam, degree, top_k)
-        cnt = capi.DeviceArray.from_numpy(np.zeros(3, np.uint64))
+        cnt = capi.new_counters()
         index.search(sp, d_q, counters=cnt, out=(d_ids, d_dists))
         capi.synchronize()
-        c = cnt.numpy()
+        c = capi.read_counters(cnt)
         r = {}
         index.search(sp, d_q, result=r, out=(d_ids, d_dists))
         rec = D.recall(d_ids.numpy(), gt, top_k)

@@ -9,7 +9,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libglide_hip.so")
+LIB_PATH = os.environ.get("GLIDE_HIP_LIB", os.path.join(_HERE, "libglide_hip.so"))   # override: an alternative build of the library
 _lib = None
 
 EUCLIDEAN, COSINE = 0, 1
@@ -108,6 +108,19 @@ class DeviceArray:
             self.free()
         except Exception:
             pass
+
+
+COUNTER_STRIPES = 256
+
+
+def new_counters():
+    """Zeroed device counters for the beam kernels (COUNTER_STRIPES x 3 u64)."""
+    return DeviceArray.from_numpy(np.zeros((COUNTER_STRIPES, 3), np.uint64))
+
+
+def read_counters(counters):
+    """[beam iterations, data rows scored, graph rows read] summed over the stripes."""
+    return counters.numpy().sum(0).tolist()
 
 
 def _ptr(x):

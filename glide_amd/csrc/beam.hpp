@@ -18,6 +18,8 @@ struct BeamParams {
     int metric;
 };
 
+constexpr uint32_t kCounterStripes = 256;
+
 struct BeamCounters {  // wave-uniform tallies for traffic accounting
     uint32_t iterations = 0, rows_scored = 0, graph_rows = 0;
 };
@@ -224,11 +226,14 @@ struct Beam {
         }
     }
 
+    // `counters` holds kCounterStripes x 3 u64 (striped by workgroup: a single shared address would serialise the
+    // whole launch); the host adds the stripes up
     __device__ __forceinline__ void flush_counters(unsigned long long* counters) {
         if (counters != nullptr && lane == 0) {
-            atomicAdd(&counters[0], static_cast<unsigned long long>(cnt.iterations));
-            atomicAdd(&counters[1], static_cast<unsigned long long>(cnt.rows_scored));
-            atomicAdd(&counters[2], static_cast<unsigned long long>(cnt.graph_rows));
+            unsigned long long* slot = counters + 3 * (blockIdx.x % kCounterStripes);
+            atomicAdd(&slot[0], static_cast<unsigned long long>(cnt.iterations));
+            atomicAdd(&slot[1], static_cast<unsigned long long>(cnt.rows_scored));
+            atomicAdd(&slot[2], static_cast<unsigned long long>(cnt.graph_rows));
         }
     }
 };

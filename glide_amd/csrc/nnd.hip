@@ -148,10 +148,15 @@ struct JoinArgs {
     Segments segs;
 };
 
-struct JoinLds {
+struct JoinRows {
     _Float16 xn[kBi][kRowHalfs];
     _Float16 xo[kBi][kRowHalfs];
-    float dist[kBi][kDStride];
+};
+struct JoinLds {
+    union {               // the distance tile is written only after the last matrix-core pass has read the rows
+        JoinRows rows;
+        float dist[kBi][kDStride];
+    };
     uint32_t new_ids[kBi], old_ids[kBi];
     float new_norms[kBi], old_norms[kBi];
     uint32_t hash_new[128], hash_old[128];
@@ -192,41 +197,70 @@ __device__ __forceinline__ void mfma_chunk(float16v& acc, const _Float16 (*A)[kR
     }
 }
 
+// Nearest partner of one row (BY_ROW) or one column of the distance tile (get_min_item, nn_descent.cuh:581-623):
+// four adjacent lanes scan 16 entries each, then combine (smaller distance, then smaller index).
+// Thread t handles line t/4; `skip(idx)` excludes entries (the line's own id).
+template <bool BY_ROW, class SkipFn>
+__device__ __forceinline__ void line_argmin(const float (*dist)[kDStride], uint32_t line, uint32_t part, uint32_t count, SkipFn skip,
+                                            float& best, uint32_t& best_idx) {
+    best = FLT_MAX;
+    best_idx = kInvalid;
+    const uint32_t first = part * 16;
+#pragma unroll 4
+    for (uint32_t k = 0; k < 16; k++) {
+        const uint32_t idx = first + k;
+        if (idx < count) {
+            const float d = BY_ROW ? dist[line][idx] : dist[idx][line];
+            if (d < best && !skip(idx)) {
+                best = d;
+                best_idx = idx;
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 1; m <= 2; m <<= 1) {
+        const float od = m == 1 ? lane_xor<1>(best) : lane_xor<2>(best);
+        const uint32_t oi = m == 1 ? lane_xor<1>(best_idx) : lane_xor<2>(best_idx);
+        if (od < best || (od == best && oi < best_idx)) {
+            best = od;
+            best_idx = oi;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     JoinLds& L = *reinterpret_cast<JoinLds*>(smem);
     const uint32_t node = blockIdx.x;
     if (node >= a.num) return;
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
-    uint32_t seg_start, seg_len;
-    locate(a.segs, node, seg_start, seg_len);
 
-    const uint32_t c_fn = a.counts[static_cast<size_t>(node) * 4 + 0], c_fo = a.counts[static_cast<size_t>(node) * 4 + 1];
-    uint32_t c_rn = a.counts[static_cast<size_t>(node) * 4 + 2], c_ro = a.counts[static_cast<size_t>(node) * 4 + 3];
-    c_rn = c_rn < kSamples ? c_rn : kSamples;
-    c_ro = c_ro < kSamples ? c_ro : kSamples;
-    if (c_fn + c_rn == 0) return;
-
+    // sample ids are fetched before the counts are known (one memory round trip instead of two)
+    uint32_t my_id = kInvalid;
     if (tid < 128) {
+        const bool is_old = tid >= 64;
+        const uint32_t k = tid & 63;
+        const uint32_t* src = k < kSamples ? (is_old ? a.fwd_old : a.fwd_new) : (is_old ? a.rev_old : a.rev_new);
+        my_id = src[static_cast<size_t>(node) * kSamples + (k & (kSamples - 1))];
         L.hash_new[tid] = kInvalid;
         L.hash_old[tid] = kInvalid;
     }
-    if (tid == 0) {
-        L.n_new = 0;
-        L.n_old = 0;
-    }
+    const uint4 c4 = *reinterpret_cast<const uint4*>(a.counts + static_cast<size_t>(node) * 4);
+    uint32_t seg_start, seg_len;
+    locate(a.segs, node, seg_start, seg_len);
+    const uint32_t c_fn = c4.x, c_fo = c4.y;
+    const uint32_t c_rn = c4.z < kSamples ? c4.z : kSamples, c_ro = c4.w < kSamples ? c4.w : kSamples;
+    if (c_fn + c_rn == 0) return;
     __syncthreads();
     // forward then reverse samples, duplicates removed with an LDS hash set (reference: sort + binary search, :625-666)
     if (tid < 128) {
         const bool is_old = tid >= 64;
         const uint32_t k = tid & 63;
         const uint32_t cf = is_old ? c_fo : c_fn, cr = is_old ? c_ro : c_rn;
-        uint32_t id = kInvalid;
-        if (k < cf) id = (is_old ? a.fwd_old : a.fwd_new)[static_cast<size_t>(node) * kSamples + k];
-        else if (k >= kSamples && k - kSamples < cr) id = (is_old ? a.rev_old : a.rev_new)[static_cast<size_t>(node) * kSamples + (k - kSamples)];
-        bool keep = id != kInvalid && id < seg_len && lds_set_insert(is_old ? L.hash_old : L.hash_new, id);
-        // forward entries first: rank within the wave keeps that order (wave 0 = new, wave 1 = old)
-        const uint64_t m = ballot(keep);
+        const bool present = k < kSamples ? k < cf : (k - kSamples) < cr;
+        const uint32_t id = present ? my_id : kInvalid;
+        const bool keep = id != kInvalid && id < seg_len && lds_set_insert(is_old ? L.hash_old : L.hash_new, id);
+        const uint64_t m = ballot(keep);   // wave 0 = new, wave 1 = old; forward entries keep the lower ranks
         if (keep) {
             const uint32_t pos = prefix_count(m);
             (is_old ? L.old_ids : L.new_ids)[pos] = id;
@@ -251,6 +285,7 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
     for (uint32_t k0 = 0; k0 < a.dim_pad; k0 += 128) {
         if (k0) __syncthreads();
         // gather: 16 lanes x 16 B per 128-dim chunk row, 16 rows per pass, new rows then old rows
+#pragma unroll
         for (uint32_t r0 = 0; r0 < 128; r0 += 16) {
             const uint32_t r = r0 + (tid >> 4), q = tid & 15;
             const bool is_old = r >= 64;
@@ -262,16 +297,17 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
                 const uint32_t id = (is_old ? L.old_ids : L.new_ids)[rr];
                 v = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
             }
-            *reinterpret_cast<float4*>(&(is_old ? L.xo : L.xn)[rr][q * 8]) = v;
+            *reinterpret_cast<float4*>(&(is_old ? L.rows.xo : L.rows.xn)[rr][q * 8]) = v;
         }
         __syncthreads();
-        if (need_nn) mfma_chunk(acc_nn, L.xn, L.xn, rb, cb, lane);
-        if (need_no) mfma_chunk(acc_no, L.xn, L.xo, rb, cb, lane);
+        if (need_nn) mfma_chunk(acc_nn, L.rows.xn, L.rows.xn, rb, cb, lane);
+        if (need_no) mfma_chunk(acc_no, L.rows.xn, L.rows.xo, rb, cb, lane);
     }
 
     const int t = lane & 31, kh = lane >> 5;
+    const uint32_t line = tid >> 2, part = tid & 3;
     // ---- phase 1: new x new
-    __syncthreads();
+    __syncthreads();   // every wave is done with the rows: the tile may overwrite them
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
@@ -280,18 +316,11 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
         L.dist[i][j] = d;
     }
     __syncthreads();
-    if (tid < 64 && static_cast<uint32_t>(tid) < n_new) {   // get_min_item (:581-623): nearest partner with a different id
-        const uint32_t me = L.new_ids[tid];
-        float best = FLT_MAX;
-        uint32_t bid = kInvalid;
-        for (uint32_t j = 0; j < n_new; j++) {
-            const float d = L.dist[tid][j];
-            if (j != static_cast<uint32_t>(tid) && d < best) {
-                best = d;
-                bid = L.new_ids[j];
-            }
-        }
-        emit_offer(a, seg_start, seg_len, me, bid, best);
+    {
+        float best;
+        uint32_t bj;
+        line_argmin<true>(L.dist, line, part, n_new, [line](uint32_t j) { return j == line; }, best, bj);
+        if (part == 0 && line < n_new && bj != kInvalid) emit_offer(a, seg_start, seg_len, L.new_ids[line], L.new_ids[bj], best);
     }
     if (n_old == 0) return;
     // ---- phase 2: new x old (rows: new, columns: old)
@@ -304,35 +333,21 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
         L.dist[i][j] = d;
     }
     __syncthreads();
-    if (tid < 64) {
-        if (static_cast<uint32_t>(tid) < n_new) {
-            const uint32_t me = L.new_ids[tid];
-            float best = FLT_MAX;
-            uint32_t bid = kInvalid;
-            for (uint32_t j = 0; j < n_old; j++) {
-                const float d = L.dist[tid][j];
-                if (L.old_ids[j] != me && d < best) {
-                    best = d;
-                    bid = L.old_ids[j];
-                }
-            }
-            emit_offer(a, seg_start, seg_len, me, bid, best);
-        }
-    } else if (tid < 128) {
-        const uint32_t c = tid - 64;
-        if (c < n_old) {
-            const uint32_t me = L.old_ids[c];
-            float best = FLT_MAX;
-            uint32_t bid = kInvalid;
-            for (uint32_t i = 0; i < n_new; i++) {
-                const float d = L.dist[i][c];
-                if (L.new_ids[i] != me && d < best) {
-                    best = d;
-                    bid = L.new_ids[i];
-                }
-            }
-            emit_offer(a, seg_start, seg_len, me, bid, best);
-        }
+    {
+        float best;
+        uint32_t bj;
+        const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
+        const uint32_t* old_ids = L.old_ids;
+        line_argmin<true>(L.dist, line, part, n_old, [old_ids, me](uint32_t j) { return old_ids[j] == me; }, best, bj);
+        if (part == 0 && line < n_new && bj != kInvalid) emit_offer(a, seg_start, seg_len, me, L.old_ids[bj], best);
+    }
+    {
+        float best;
+        uint32_t bi;
+        const uint32_t me = line < n_old ? L.old_ids[line] : kInvalid;
+        const uint32_t* new_ids = L.new_ids;
+        line_argmin<false>(L.dist, line, part, n_new, [new_ids, me](uint32_t i) { return new_ids[i] == me; }, best, bi);
+        if (part == 0 && line < n_old && bi != kInvalid) emit_offer(a, seg_start, seg_len, me, L.new_ids[bi], best);
     }
 }
 
@@ -541,9 +556,10 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
         counts[static_cast<size_t>(node) * 4 + 1] = total_old < kSamples ? total_old : kSamples;
         counts[static_cast<size_t>(node) * 4 + 2] = 0;
         counts[static_cast<size_t>(node) * 4 + 3] = 0;
-        if (stats) {
-            atomicAdd(&stats[0], static_cast<unsigned long long>(raw));
-            if (raw > inbox_cap) atomicAdd(&stats[1], static_cast<unsigned long long>(raw - inbox_cap));
+        if (stats) {   // striped over 1024 slots: one shared address would serialise every wavefront of the launch
+            unsigned long long* slot = stats + 2 * (blockIdx.x & 1023u);
+            atomicAdd(&slot[0], static_cast<unsigned long long>(raw));
+            if (raw > inbox_cap) atomicAdd(&slot[1], static_cast<unsigned long long>(raw - inbox_cap));
         }
     }
 }
@@ -554,6 +570,24 @@ __host__ __device__ inline uint32_t xorshift32(uint32_t u) {   // reference util
     u ^= u << 27;
     u ^= u >> 5;
     return u * 0x9E3779B9u;
+}
+
+__global__ __launch_bounds__(1024) void nnd_stats_reduce_kernel(const unsigned long long* striped, unsigned long long* out) {
+    __shared__ unsigned long long part[2][1024];
+    part[0][threadIdx.x] = striped[2 * threadIdx.x];
+    part[1][threadIdx.x] = striped[2 * threadIdx.x + 1];
+    __syncthreads();
+    for (int off = 512; off > 0; off >>= 1) {
+        if (static_cast<int>(threadIdx.x) < off) {
+            part[0][threadIdx.x] += part[0][threadIdx.x + off];
+            part[1][threadIdx.x] += part[1][threadIdx.x + off];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        out[0] = part[0][0];
+        out[1] = part[1][0];
+    }
 }
 
 __global__ __launch_bounds__(256) void nnd_finalize_kernel(const uint32_t* list_ids, uint32_t num, uint32_t width, uint32_t degree, Segments segs,
@@ -602,7 +636,7 @@ NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
     l.inbox_counts = take(n * 4);
     l.inbox = take(n * l.cap * 8);
     l.bloom = take(n * l.bloom_sets * 64);
-    l.stats = take(64);
+    l.stats = take(1024 * 16);
     l.total = off;
     return l;
 }
@@ -643,7 +677,7 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
     const uint32_t n = reorder_num;
 
     if (stats) {
-        int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(stats), 0u, 4, stream);
+        int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(stats), 0u, 1024 * 4, stream);
         if (rc != GLIDE_OK) return rc;
     }
     hipLaunchKernelGGL(nnd_prepare_kernel, dim3(ceil_div(n, 4)), dim3(256), 0, s, reorder_data, n, dim, l.dim_pad, half_rows, norms);
@@ -670,7 +704,7 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
         }
     }
     hipLaunchKernelGGL(nnd_finalize_kernel, dim3(ceil_div(n * knn_degree, 256)), dim3(256), 0, s, list_ids, n, l.width, knn_degree, segs, knn_graph);
-    if (stats_out) GLIDE_HIP_TRY(hipMemcpyAsync(stats_out, stats, 16, hipMemcpyDeviceToDevice, s));
+    if (stats_out) hipLaunchKernelGGL(nnd_stats_reduce_kernel, dim3(1), dim3(1024), 0, s, stats, stats_out);
     return launch_status();
 }
 

@@ -263,7 +263,7 @@ class GLIDE:
         d_ss = capi.DeviceArray.from_numpy(np.ascontiguousarray(h_segment_start, dtype=np.uint32))
         d_sl = capi.DeviceArray.from_numpy(np.ascontiguousarray(h_segment_length, dtype=np.uint32))
         d_rsp = capi.DeviceArray.from_numpy(reorder_sp)
-        cnt = capi.DeviceArray.from_numpy(np.zeros(3, np.uint64)) if counters else None
+        cnt = capi.new_counters() if counters else None
         times = {}
         p = search_param_knn
         with _Timer() as t:
@@ -279,7 +279,7 @@ class GLIDE:
         times["boundary"] = t.seconds
         if counters and result is not None:
             capi.synchronize()
-            result["build_counters"] = cnt.numpy().tolist()
+            result["build_counters"] = capi.read_counters(cnt)
         for consumed in (d_knn_graph, d_map, d_reorder_data):
             capi.synchronize()
             consumed.free()
@@ -299,7 +299,7 @@ class GLIDE:
         times["refine"] = 0.0
         if search_param_refine.beam != 0:
             p = search_param_refine
-            cnt2 = capi.DeviceArray.from_numpy(np.zeros(3, np.uint64)) if counters else None
+            cnt2 = capi.new_counters() if counters else None
             with _Timer() as t:
                 capi.refine(self.d_data, num, dim, self.d_graph, d_rev, deg, self.d_centroids, self.centroid_num(),
                             self.d_start_points, p.beam, p.max_iterations, p.min_iterations, p.hash_bit, p.hash_reset_interval,
@@ -307,7 +307,7 @@ class GLIDE:
             times["refine"] = t.seconds
             self.d_graph, d_rev = d_rev, self.d_graph
             if counters and result is not None:
-                result["refine_counters"] = cnt2.numpy().tolist()
+                result["refine_counters"] = capi.read_counters(cnt2)
         d_rev.free()
         if result is not None:
             result["index_time"] = times["subgraph"] + times["boundary"] + times["reverse"]

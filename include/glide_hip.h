@@ -29,6 +29,7 @@ extern "C" {
 #define GLIDE_METRIC_COSINE 1
 
 #define GLIDE_INVALID_ID 0xffffffffu
+#define GLIDE_COUNTER_STRIPES 256
 
 /* ---- library / device ------------------------------------------------------------------------------------ */
 const char *glide_hip_version(void);
@@ -58,8 +59,9 @@ int glide_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* synchroni
 /* ---- beam search (subsystem 4) ----------------------------------------------------------------------------
  * Replaces search_kernel<MAX_CANDIDATE,MAX_BEAM,MAX_CENTROID> (search_kernel.cuh:393-490) as launched by
  * GLIDE::search (glide_impl.cuh:370-454).  One query per wavefront.  result_ids/result_dists are
- * query_num x top_k.  `counters` (nullable) receives three u64 sums: beam iterations, data rows scored, graph
- * rows read -- the algorithmic-traffic tallies.
+ * query_num x top_k.  `counters` (nullable) points at GLIDE_COUNTER_STRIPES x 3 u64 that the caller zeroed; the
+ * kernel adds {beam iterations, data rows scored, graph rows read} into the stripe of each workgroup (one shared
+ * address would serialise the launch); the sums over the stripes are the algorithmic-traffic tallies.
  * Limits: graph_degree <= 128, beam <= 256, centroid_num <= 256, dim % 4 == 0, dim <= 1024, top_k <= beam. */
 int glide_hip_search(const float *data, uint32_t num, uint32_t dim, const uint32_t *graph, uint32_t graph_degree,
                      const float *centroids, uint32_t centroid_num, const uint32_t *start_points,

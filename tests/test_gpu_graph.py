@@ -41,7 +41,7 @@ def gpu_build_sub(hip, idx, sp, D=32, relaxant=1.05, metric=0):
     d = dev(hip, idx)
     n, dim = idx["data"].shape
     graph = hip.DeviceArray.full((n, D), INV)
-    cnt = hip.DeviceArray.from_numpy(np.zeros(3, np.uint64))
+    cnt = hip.new_counters()
     hip.build_subgraph(d["rdata"], n, dim, d["knn"], idx["knn"].shape[1], d["map"], d["ss"], d["sl"], idx["seg_start"].size, d["lsp"],
                        D, sp["beam"], sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"],
                        relaxant, metric, graph, cnt)
@@ -53,7 +53,7 @@ def test_build_subgraph_bit_exact(hip, small_index, stages):
     _, graph, cnt = gpu_build_sub(hip, small_index, stages["sp"])
     assert np.array_equal(graph.numpy(), stages["sub"])
     st = stages["st_sub"]
-    assert cnt.numpy().tolist() == [st["iterations"], st["rows_scored"], st["graph_rows"]]
+    assert hip.read_counters(cnt) == [st["iterations"], st["rows_scored"], st["graph_rows"]]
 
 
 def test_build_boundary_bit_exact(hip, small_index, stages):
@@ -120,14 +120,14 @@ def test_refine_bit_exact(hip, small_index, stages):
     data = hip.DeviceArray.from_numpy(idx["data"], np.float32)
     cent = hip.DeviceArray.from_numpy(idx["centroids"], np.float32)
     spd = hip.DeviceArray.from_numpy(idx["start_points"], np.uint32)
-    cntd = hip.DeviceArray.from_numpy(np.zeros(3, np.uint64))
+    cntd = hip.new_counters()
     assert (stages["rev"] == INV).any(), "fixture must leave holes for refinement"
     hip.refine(data, n, dim, g_in, g_out, 32, cent, idx["centroids"].shape[0], spd, sp["beam"], sp["max_iterations"],
                sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 1.05, 0, cntd)
     hip.synchronize()
     assert np.array_equal(g_out.numpy(), stages["ref"])
     st = stages["st_ref"]
-    assert cntd.numpy().tolist() == [st["iterations"], st["rows_scored"], st["graph_rows"]]
+    assert hip.read_counters(cntd) == [st["iterations"], st["rows_scored"], st["graph_rows"]]
     assert np.array_equal(g_in.numpy(), stages["rev"])      # input untouched
 
 

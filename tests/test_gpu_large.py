@@ -46,14 +46,14 @@ def test_build_and_refine_segment_bit_exact(hip, large_index):
         n = seg["data"].shape[0]
         d_data, d_knn = hip.DeviceArray.from_numpy(seg["data"]), hip.DeviceArray.from_numpy(seg["knn"])
         g = hip.DeviceArray.full((n, 32), 0xDEADBEEF)
-        cnt = hip.DeviceArray.from_numpy(np.zeros(3, np.uint64))
+        cnt = hip.new_counters()
         p = L["sp_b"]
         hip.build_segment(d_data, n, 128, d_knn, 32, int(L["start_points"][s]), 32, p["beam"], p["max_iterations"], p["min_iterations"],
                           p["hash_bit"], p["hash_reset_interval"], 1.05, 0, g, cnt)
         hip.synchronize()
         assert np.array_equal(g.numpy(), seg["built"])
         st = seg["st_built"]
-        assert cnt.numpy().tolist() == [st["iterations"], st["rows_scored"], st["graph_rows"]]
+        assert hip.read_counters(cnt) == [st["iterations"], st["rows_scored"], st["graph_rows"]]
         g_in, g_out = hip.DeviceArray.from_numpy(seg["rev"]), hip.DeviceArray.full((n, 32), 0xDEADBEEF)
         p = L["sp_r"]
         hip.refine_segment(d_data, n, 128, g_in, g_out, 32, int(L["start_points"][s]), p["beam"], p["max_iterations"], p["min_iterations"],

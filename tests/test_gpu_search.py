@@ -18,12 +18,12 @@ def run_gpu_search(hip, data, graph, centroids, start_points, queries, top_k, sp
              q=hip.DeviceArray.from_numpy(queries, np.float32))
     nq = queries.shape[0]
     ids, dists = hip.DeviceArray((nq, top_k), np.uint32), hip.DeviceArray((nq, top_k), np.float32)
-    cnt = hip.DeviceArray.from_numpy(np.zeros(3, np.uint64)) if counters else None
+    cnt = hip.new_counters() if counters else None
     hip.search(d["data"], data.shape[0], data.shape[1], d["graph"], graph.shape[1], d["cent"], centroids.shape[0], d["sp"],
                d["q"], nq, top_k, sp["beam"], sp["max_iterations"], sp["min_iterations"], sp["hash_bit"],
                sp["hash_reset_interval"], metric, ids, dists, cnt)
     hip.synchronize()
-    return ids.numpy(), dists.numpy(), (cnt.numpy() if counters else None)
+    return ids.numpy(), dists.numpy(), (hip.read_counters(cnt) if counters else None)
 
 
 @pytest.mark.parametrize("beam,top_k", [(32, 10), (64, 10), (96, 32), (128, 10), (256, 100)])
@@ -36,7 +36,7 @@ def test_search_bit_exact_on_integer_data(hip, small_index, beam, top_k):
                                         idx["queries"], top_k, sp, counters=True)
     assert np.array_equal(gids, eids)
     assert np.array_equal(gdists, edists)
-    assert gcnt.tolist() == [est["iterations"], est["rows_scored"], est["graph_rows"]]
+    assert gcnt == [est["iterations"], est["rows_scored"], est["graph_rows"]]
 
 
 def test_search_recall_against_brute_force(hip, small_index):
