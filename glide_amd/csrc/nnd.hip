@@ -16,7 +16,7 @@
 
 namespace glide {
 
-typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kSamples = 32;     // NUM_SAMPLES (nn_descent.cuh:391)
@@ -37,6 +37,23 @@ __device__ __forceinline__ void locate(const Segments& s, uint32_t node, uint32_
         if (node < s.starts[i] + s.lengths[i]) break;
     start = s.starts[i];
     len = s.lengths[i];
+}
+
+// Same result for a node every lane of the wavefront shares: the lanes test one segment each, so the lookup costs
+// one memory round trip instead of one per segment.  Every lane of the wavefront must call it.
+__device__ __forceinline__ void locate_uniform(const Segments& s, uint32_t node, uint32_t& start, uint32_t& len) {
+    uint32_t found = s.count - 1;
+    for (uint32_t base = 0; base + 1 < s.count; base += 64) {
+        const uint32_t i = base + lane_id();
+        const bool hit = i + 1 < s.count && node < s.starts[i] + s.lengths[i];
+        const uint64_t m = ballot(hit);
+        if (m) {
+            found = base + static_cast<uint32_t>(__ffsll(static_cast<long long>(m))) - 1;
+            break;
+        }
+    }
+    start = s.starts[found];
+    len = s.lengths[found];
 }
 
 // ---- prepare: fp32 rows -> fp16 rows (stride dim_pad, zero padded) + squared norms of the fp32 input
@@ -88,7 +105,7 @@ __global__ __launch_bounds__(256) void nnd_sample_kernel(uint32_t* list_ids, uin
     const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (node >= num) return;
     uint32_t start, len;
-    locate(segs, node, start, len);
+    locate_uniform(segs, node, start, len);
     uint32_t nn = 0, no = 0;
     for (uint32_t base = 0; base < width; base += 64) {
         const uint32_t j = base + lane;
@@ -122,7 +139,7 @@ __global__ __launch_bounds__(256) void nnd_reverse_kernel(const uint32_t* fwd_ne
     const uint32_t node = idx / 64, j = idx % 64;
     if (node >= num) return;
     uint32_t start, len;
-    locate(segs, node, start, len);
+    locate_uniform(segs, node, start, len);
     const uint32_t which = j / kSamples, k = j % kSamples;   // 0: new, 1: old
     if (k >= counts[static_cast<size_t>(node) * 4 + which]) return;
     const uint32_t v = (which ? fwd_old : fwd_new)[static_cast<size_t>(node) * kSamples + k];
@@ -174,26 +191,18 @@ __device__ __forceinline__ bool lds_set_insert(uint32_t* table, uint32_t key) { 
     return false;
 }
 
-__device__ __forceinline__ void emit_offer(const JoinArgs& a, uint32_t seg_start, uint32_t seg_len, uint32_t target, uint32_t cand, float d) {
-    if (cand == kInvalid || cand == target || cand >= seg_len || !(d < FLT_MAX)) return;
-    // No filtering against the target's current list: the reference also explores offers that do not enter the
-    // list (they are the "new" samples of the next round, nn_descent.cuh:973-1001).
-    const uint32_t g = seg_start + target;
-    const uint32_t pos = atomicAdd(&a.inbox_counts[g], 1u);
-    if (pos < a.inbox_cap) {
-        a.inbox[static_cast<size_t>(g) * a.inbox_cap + pos] = make_uint2(__float_as_uint(d), cand);
-    }
-}
+// No filtering of offers against the target's current list: the reference also explores offers that do not enter
+// the list (they are the "new" samples of the next round, nn_descent.cuh:973-1001).
 
 // A (rows) x B (rows) dot products of a 128-dim chunk for this wave's 32 x 32 quadrant.
-// v_mfma_f32_32x32x8_f16: lane supplies A[i = lane%32][k = 4*(lane/32) .. +3] and B[k = same][j = lane%32].
+// v_mfma_f32_32x32x16_f16 (gfx950): lane supplies A[i = lane%32][k = 8*(lane/32) .. +7] and B[k = same][j = lane%32].
 __device__ __forceinline__ void mfma_chunk(float16v& acc, const _Float16 (*A)[kRowHalfs], const _Float16 (*B)[kRowHalfs], int rb, int cb, int lane) {
     const int t = lane & 31, kh = lane >> 5;
 #pragma unroll
-    for (int kk = 0; kk < 128; kk += 8) {
-        const half4v av = *reinterpret_cast<const half4v*>(&A[rb * 32 + t][kk + 4 * kh]);
-        const half4v bv = *reinterpret_cast<const half4v*>(&B[cb * 32 + t][kk + 4 * kh]);
-        acc = __builtin_amdgcn_mfma_f32_32x32x8f16(av, bv, acc, 0, 0, 0);
+    for (int kk = 0; kk < 128; kk += 16) {
+        const half8v av = *reinterpret_cast<const half8v*>(&A[rb * 32 + t][kk + 8 * kh]);
+        const half8v bv = *reinterpret_cast<const half8v*>(&B[cb * 32 + t][kk + 8 * kh]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, acc, 0, 0, 0);
     }
 }
 
@@ -247,7 +256,7 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
     }
     const uint4 c4 = *reinterpret_cast<const uint4*>(a.counts + static_cast<size_t>(node) * 4);
     uint32_t seg_start, seg_len;
-    locate(a.segs, node, seg_start, seg_len);
+    locate_uniform(a.segs, node, seg_start, seg_len);
     const uint32_t c_fn = c4.x, c_fo = c4.y;
     const uint32_t c_rn = c4.z < kSamples ? c4.z : kSamples, c_ro = c4.w < kSamples ? c4.w : kSamples;
     if (c_fn + c_rn == 0) return;
@@ -264,7 +273,6 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
         if (keep) {
             const uint32_t pos = prefix_count(m);
             (is_old ? L.old_ids : L.new_ids)[pos] = id;
-            (is_old ? L.old_norms : L.new_norms)[pos] = a.norms[seg_start + id];
         }
         if (lane == 0) (is_old ? L.n_old : L.n_new) = __popcll(m);
     }
@@ -293,9 +301,10 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
             const uint32_t n = is_old ? n_old : n_new;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             const uint32_t d0 = k0 + q * 8;
-            if (rr < n && d0 < a.dim_pad) {
+            if (rr < n) {
                 const uint32_t id = (is_old ? L.old_ids : L.new_ids)[rr];
-                v = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
+                if (d0 < a.dim_pad) v = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
+                if (k0 == 0 && q == 0) (is_old ? L.old_norms : L.new_norms)[rr] = a.norms[seg_start + id];   // same round trip as the row
             }
             *reinterpret_cast<float4*>(&(is_old ? L.rows.xo : L.rows.xn)[rr][q * 8]) = v;
         }
@@ -316,38 +325,66 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
         L.dist[i][j] = d;
     }
     __syncthreads();
+    // offers are collected first and sent at the end, so their atomics overlap instead of costing a round trip each
+    uint32_t off_target[3] = {kInvalid, kInvalid, kInvalid}, off_cand[3] = {kInvalid, kInvalid, kInvalid};
+    float off_dist[3] = {FLT_MAX, FLT_MAX, FLT_MAX};
     {
         float best;
         uint32_t bj;
         line_argmin<true>(L.dist, line, part, n_new, [line](uint32_t j) { return j == line; }, best, bj);
-        if (part == 0 && line < n_new && bj != kInvalid) emit_offer(a, seg_start, seg_len, L.new_ids[line], L.new_ids[bj], best);
+        if (part == 0 && line < n_new && bj != kInvalid) {
+            off_target[0] = L.new_ids[line];
+            off_cand[0] = L.new_ids[bj];
+            off_dist[0] = best;
+        }
     }
-    if (n_old == 0) return;
-    // ---- phase 2: new x old (rows: new, columns: old)
-    __syncthreads();
+    if (n_old != 0) {
+        // ---- phase 2: new x old (rows: new, columns: old)
+        __syncthreads();
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
-        float d = FLT_MAX;
-        if (i < n_new && j < n_old) d = fmaxf((L.new_norms[i] + L.old_norms[j]) - 2.f * acc_no[r], 0.f);
-        L.dist[i][j] = d;
+        for (int r = 0; r < 16; r++) {
+            const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
+            float d = FLT_MAX;
+            if (i < n_new && j < n_old) d = fmaxf((L.new_norms[i] + L.old_norms[j]) - 2.f * acc_no[r], 0.f);
+            L.dist[i][j] = d;
+        }
+        __syncthreads();
+        {
+            float best;
+            uint32_t bj;
+            const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
+            const uint32_t* old_ids = L.old_ids;
+            line_argmin<true>(L.dist, line, part, n_old, [old_ids, me](uint32_t j) { return old_ids[j] == me; }, best, bj);
+            if (part == 0 && line < n_new && bj != kInvalid) {
+                off_target[1] = me;
+                off_cand[1] = L.old_ids[bj];
+                off_dist[1] = best;
+            }
+        }
+        {
+            float best;
+            uint32_t bi;
+            const uint32_t me = line < n_old ? L.old_ids[line] : kInvalid;
+            const uint32_t* new_ids = L.new_ids;
+            line_argmin<false>(L.dist, line, part, n_new, [new_ids, me](uint32_t i) { return new_ids[i] == me; }, best, bi);
+            if (part == 0 && line < n_old && bi != kInvalid) {
+                off_target[2] = me;
+                off_cand[2] = L.new_ids[bi];
+                off_dist[2] = best;
+            }
+        }
     }
-    __syncthreads();
-    {
-        float best;
-        uint32_t bj;
-        const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
-        const uint32_t* old_ids = L.old_ids;
-        line_argmin<true>(L.dist, line, part, n_old, [old_ids, me](uint32_t j) { return old_ids[j] == me; }, best, bj);
-        if (part == 0 && line < n_new && bj != kInvalid) emit_offer(a, seg_start, seg_len, me, L.old_ids[bj], best);
+    uint32_t pos[3];
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        const bool ok = off_cand[k] != kInvalid && off_cand[k] != off_target[k] && off_cand[k] < seg_len && off_dist[k] < FLT_MAX;
+        if (!ok) off_target[k] = kInvalid;
+        pos[k] = ok ? atomicAdd(&a.inbox_counts[seg_start + off_target[k]], 1u) : kInvalid;
     }
-    {
-        float best;
-        uint32_t bi;
-        const uint32_t me = line < n_old ? L.old_ids[line] : kInvalid;
-        const uint32_t* new_ids = L.new_ids;
-        line_argmin<false>(L.dist, line, part, n_new, [new_ids, me](uint32_t i) { return new_ids[i] == me; }, best, bi);
-        if (part == 0 && line < n_old && bi != kInvalid) emit_offer(a, seg_start, seg_len, me, L.new_ids[bi], best);
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        if (off_target[k] != kInvalid && pos[k] < a.inbox_cap)
+            a.inbox[static_cast<size_t>(seg_start + off_target[k]) * a.inbox_cap + pos[k]] = make_uint2(__float_as_uint(off_dist[k]), off_cand[k]);
     }
 }
 
