@@ -23,6 +23,14 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes one launch of the timed kernel moves, measured with two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch) and scaled by what the same counters report for copy_kernel moving exactly 1 GiB
+# (--copy-calibration: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Keyed by (workload, beam); other combinations report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg1", 256): 6_320_900 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
+    ("cfg1-navigable", 32): 2_434_500 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -189,7 +197,8 @@ def run_workload(args, workload, torch, want_cpu):
         partition_sizes=[int(x) for x in h_len], empty_slots_fraction=holes,
         sweep=sweep, beam=chosen["beam"], recall_at_10=chosen["recall_at_10"], recall_target_met=bool(ok),
         qps=nq * args.steps / (wall_ms * 1e-3), ms_per_step=ms_per_step, kernel_ms=kernel_ms,
-        roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS, traffic=None,
+        roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
+                      traffic=MEASURED_TRAFFIC_BYTES.get((workload, chosen["beam"])),
                       kernel="search_kernel<64,%d,1>" % (64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256),
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )

@@ -1,0 +1,120 @@
+"""Whole small-build pipeline on the GPU against the CPU oracle's pipeline, on reduced copies of the benchmark
+configurations (clipped mixture L2 with k=64, normalised mixture cosine with 96 dims, 960 dims with degree 64).
+
+The two pipelines share the centroids and the entry points, so the partitioning is the same; the kNN graphs come
+from two different NN-descent runs, so the comparison is statistical:
+  * kNN-graph recall@k against exact neighbours inside each partition: GPU >= CPU - 0.005,
+  * search recall@10 at equal beam: GPU >= CPU - 0.015 (1 000 queries: one standard error is ~0.004).
+With the GPU's kNN graph as input, the later stages are deterministic and the finished graph must be bit-identical.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from glide_amd import capi
+    capi.set_device(0)
+    return capi
+
+
+def _exact_knn_in_partitions(O, rdata, seg_start, seg_len, k, metric, rows_per_partition=200):
+    out = []
+    for s, l in zip(seg_start.tolist(), seg_len.tolist()):
+        if l <= 2 * k:
+            continue
+        m = min(rows_per_partition, l)
+        ids, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + m], k + 1, metric)
+        # drop the row itself (first by distance, or anywhere on ties)
+        rows = []
+        for i in range(m):
+            r = [x for x in ids[i].tolist() if x != i][:k]
+            rows.append(r)
+        out.append((s, m, np.array(rows, dtype=np.uint32)))
+    return out
+
+
+def _graph_recall(D, knn, truth, k):
+    vals = [D.recall(knn[s:s + m, :k], gt, k) for s, m, gt in truth]
+    return float(np.mean(vals))
+
+
+CASES = [
+    # name, generator, num, dim, partitions, graph degree, knn degree, NN-descent iterations, metric, queries
+    ("clipped-mixture-k64", "gmm_clipped", 20_000, 128, 4, 32, 64, 8, 0, 1000),
+    ("normalised-mixture-cosine", "gmm_normalized", 20_000, 96, 4, 32, 32, 10, 1, 1000),
+    ("beta-960-degree64", "beta_scaled", 6_000, 960, 3, 64, 64, 8, 0, 300),
+]
+
+
+@pytest.mark.parametrize("name,gen,num,dim,parts,degree,knn_degree,iters,metric,nq", CASES, ids=[c[0] for c in CASES])
+def test_pipeline_matches_cpu_pipeline(hip, name, gen, num, dim, parts, degree, knn_degree, iters, metric, nq):
+    from glide_amd import datasets as D, index as G
+    from oracle import oracle as O
+    data = getattr(D, gen)(num, dim, seed=1234)
+    queries = getattr(D, gen)(nq, dim, seed=4321)
+    print("case", name, data.shape, flush=True)
+
+    # ---- GPU pipeline
+    d_data = hip.DeviceArray.from_numpy(data)
+    pp = G.PartitionParameter(centroid_num=parts, boundary_factor=1.04, sample_factor=0.05, metric=metric)
+    d_re, d_map, h_start, h_len, d_cent = G.preprocess(pp, d_data)
+    centroids = d_cent.numpy()
+    rdata, h_map = d_re.numpy(), d_map.numpy()
+    d_knn = G.build_nnd(G.NNDescentParameter(graph_degree=knn_degree, max_iterations=iters), d_re, h_start, h_len)
+    knn_gpu = d_knn.numpy()
+    index = G.GLIDE(degree, d_data, d_cent, metric)
+    bp = G.IndexParameter(graph_degree=degree, knn_degree=knn_degree, relaxant_factor=1.05)
+    sp_b, sp_r = G.make_search_parameter(64, knn_degree), G.make_search_parameter(128, knn_degree)
+    local_sp, start_points = index.start_point_select(h_start, h_len, h_map, bp.seed)
+    index.build(bp, sp_b, sp_r, d_knn, h_start, h_len, d_map, d_re)
+    graph_gpu = index.d_graph.numpy()
+    assert np.array_equal(index.d_start_points.numpy(), start_points)
+
+    # ---- CPU pipeline from the same centroids and entry points
+    seg_idx, seg_len, _ = O.partition_assign(data, centroids, 1.04, metric)
+    assert np.array_equal(seg_len, h_len), "partition sizes differ"
+    seg_start = O.segment_starts(seg_len)
+    rdata_cpu, map_cpu = O.reorder(data, seg_idx, seg_start, num + int(seg_len[parts]))
+    assert np.array_equal(map_cpu, h_map) and np.array_equal(rdata_cpu, rdata)
+    knn_cpu = O.nnd_build(rdata, seg_start, seg_len, knn_degree, iters, 0).astype(np.uint32)
+
+    def finish(knn):
+        ps = O.search_params(64, knn_degree)
+        g, _ = O.build_subgraph(rdata, num, knn, h_map, seg_start, seg_len, local_sp, degree, ps, 1.05, metric)
+        if rdata.shape[0] > num:
+            g, _ = O.build_boundary(rdata, num, knn, h_map, int(local_sp[parts]), g, ps, 1.05, metric)
+        g = O.reverse_edges(g)
+        g, _ = O.refine(data, g, centroids, start_points, O.search_params(128, knn_degree), 1.05, metric)
+        return g
+
+    # the stages after NN-descent are deterministic: same kNN graph in, same graph out
+    float_data = gen != "gmm_clipped"
+    graph_from_gpu_knn = finish(knn_gpu)
+    same_rows = (graph_from_gpu_knn == graph_gpu).all(axis=1).mean()
+    if float_data:
+        assert same_rows >= 0.98, same_rows     # float distances: a reassociated sum can flip a near-tie
+    else:
+        assert same_rows == 1.0, same_rows
+    graph_cpu = finish(knn_cpu)
+
+    # ---- kNN-graph recall inside partitions
+    k_eval = min(32, knn_degree)
+    truth = _exact_knn_in_partitions(O, rdata, seg_start, seg_len, k_eval, metric)
+    r_gpu, r_cpu = _graph_recall(D, knn_gpu, truth, k_eval), _graph_recall(D, knn_cpu, truth, k_eval)
+    print("graph recall@%d gpu %.4f cpu %.4f" % (k_eval, r_gpu, r_cpu), flush=True)
+    assert r_gpu >= r_cpu - 0.005
+
+    # ---- search recall@10 at equal beam, each pipeline on its own graph
+    gt, _ = O.bruteforce_knn(data, queries, 10, metric)
+    d_q = hip.DeviceArray.from_numpy(queries)
+    for beam in (32, 64, 128):
+        sp = G.make_search_parameter(beam, degree, 10)
+        ids_gpu, _ = index.search(sp, d_q)
+        ids_cpu, _, _ = O.search(data, graph_cpu, centroids, start_points, queries, 10, sp.beam, sp.max_iterations, sp.min_iterations,
+                                 sp.hash_bit, sp.hash_reset_interval, metric)
+        a, b = D.recall(ids_gpu, gt, 10), D.recall(ids_cpu, gt, 10)
+        print("beam %d recall@10 gpu %.4f cpu %.4f" % (beam, a, b), flush=True)
+        assert a >= b - 0.015
