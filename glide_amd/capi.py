@@ -290,6 +290,50 @@ def nnd_build(reorder_data, reorder_num, dim, segment_starts, segment_lengths, s
                                     _ptr(stats), vp(stream)), "glide_hip_nnd_build")
 
 
+class NndLayout(C.Structure):
+    """glide_nnd_layout: byte offsets of the NN-descent arrays inside the workspace."""
+    _fields_ = [(n, C.c_uint64) for n in ("half_rows", "norms", "list_ids", "list_dists", "fwd_new", "fwd_old", "rev_new", "rev_old",
+                                          "counts", "inbox_counts", "inbox", "bloom", "total")] + \
+               [(n, C.c_uint32) for n in ("width", "inbox_cap", "row_halfs", "bloom_sets")]
+
+
+def nnd_layout(reorder_num, dim, knn_degree):
+    out = NndLayout()
+    check(lib().glide_hip_nnd_layout(u32(reorder_num), u32(dim), u32(knn_degree), C.byref(out)), "glide_hip_nnd_layout")
+    return out
+
+
+def _nnd_stage(name, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream):
+    check(getattr(lib(), name)(u32(reorder_num), u32(dim), _ptr(segment_starts), _ptr(segment_lengths), u32(segment_num),
+                               u32(knn_degree), _ptr(workspace), C.c_size_t(workspace_bytes), vp(stream)), name)
+
+
+def nnd_prepare(reorder_data, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, seed, workspace,
+                workspace_bytes, stream=None):
+    check(lib().glide_hip_nnd_prepare(_ptr(reorder_data), u32(reorder_num), u32(dim), _ptr(segment_starts), _ptr(segment_lengths),
+                                      u32(segment_num), u32(knn_degree), u32(seed), _ptr(workspace), C.c_size_t(workspace_bytes),
+                                      vp(stream)), "glide_hip_nnd_prepare")
+
+
+def nnd_reverse_sample(*args, stream=None):
+    _nnd_stage("glide_hip_nnd_reverse_sample", *args, stream)
+
+
+def nnd_local_join(*args, stream=None):
+    _nnd_stage("glide_hip_nnd_local_join", *args, stream)
+
+
+def nnd_merge(*args, stream=None):
+    _nnd_stage("glide_hip_nnd_merge", *args, stream)
+
+
+def nnd_finalize(reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, knn_graph, stats, workspace,
+                 workspace_bytes, stream=None):
+    check(lib().glide_hip_nnd_finalize(u32(reorder_num), u32(dim), _ptr(segment_starts), _ptr(segment_lengths), u32(segment_num),
+                                       u32(knn_degree), _ptr(knn_graph), _ptr(stats), _ptr(workspace), C.c_size_t(workspace_bytes),
+                                       vp(stream)), "glide_hip_nnd_finalize")
+
+
 def copy_bytes(dst, src, nbytes, stream=None):
     check(lib().glide_hip_copy_bytes(_ptr(dst), _ptr(src), C.c_size_t(nbytes), vp(stream)), "glide_hip_copy_bytes")
 

@@ -11,6 +11,7 @@
 // (one atomic counter per node, no locks, no cross-workgroup read-after-write inside a kernel) and a merge kernel
 // folds each inbox into the node's sorted list with a wave-wide bitonic sort; sampling uses the new/old flag kept
 // in the list instead of a host-side Bloom filter.  All ids are partition-local.
+#include <cstdlib>
 #include "common.hpp"
 #include "host_util.hpp"
 
@@ -86,12 +87,19 @@ __global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t* list_ids, float
     uint32_t start, len;
     locate(segs, node, start, len);
     const uint32_t local = node - start;
-    // pseudo-random partition-local neighbour, never the node itself; a repeated id in a row is harmless (the
-    // join and the merge both drop repeats)
+    // width distinct pseudo-random partition-local neighbours, never the node itself: the partition is cut into
+    // width + 1 strata (rotated by a per-node offset), entry j draws from stratum j, and the entry that would hit the
+    // node itself draws from the spare stratum instead.  Partitions with fewer than width + 2 points list every other point.
     uint32_t id = kInvalid;
-    if (len > 1) {
-        id = mix32(mix32(node + seed * 0x9E3779B9u) ^ (j * 0x85EBCA6Bu + 1u)) % len;
-        if (id == local) id = (id + 1) % len;
+    const uint32_t stride = len / (width + 1);
+    if (stride >= 1) {
+        const uint32_t h = mix32(node + seed * 0x9E3779B9u);
+        const uint32_t rot = h % len;
+        auto draw = [&](uint32_t stratum) { return (rot + stratum * stride + mix32(h ^ (stratum * 0x85EBCA6Bu + 1u)) % stride) % len; };
+        id = draw(j);
+        if (id == local) id = draw(width);
+    } else if (j + 1 < len) {
+        id = (local + 1 + j) % len;
     }
     list_ids[static_cast<size_t>(node) * width + j] = id;   // new (flag clear)
     list_dists[static_cast<size_t>(node) * width + j] = FLT_MAX;
@@ -457,11 +465,14 @@ __device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane
     return incl - value;
 }
 
-// Merge + resample.  The list and this round's offers are sorted together by (distance, id); repeats of an id are
-// dropped; the first `width` survive as the new list.  Samples for the next join:
-//   new = the best <= 32 offers of this round (what the reference's 32-wide device list would hold) that the
-//         Bloom filter has not seen (sample_graph_new :973-1001); those that made the list are flagged old;
-//   old = the first <= 32 list entries that were already flagged old (sample_segment_graph :1073-1104).
+// Merge + resample, one wavefront per node.  The reference keeps, per node and round, a 32-wide sorted "device" list of
+// the offers (insert_to_global_graph :509-579), merges it into the host list (update_graph :1106-1126) and draws the
+// samples of the next join from both (sample_graph_new :973-1001, sample_segment_graph :1073-1104).  Here:
+//   old samples = the first <= 32 entries of the incoming list that are flagged old (the reference samples them before
+//                 this round's results are merged);
+//   the list and this round's offers are sorted together by (distance, id); of the distinct offered ids only the
+//   best 32 count (the rest are dropped, as the 32-wide device list drops them); those not yet in the list enter it;
+//   new samples = those of the best 32 that the Bloom filter has not seen; the ones entering the list are flagged old.
 template <int M>
 __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t num,
                                                         uint32_t width, uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new,
@@ -479,6 +490,7 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
     const uint32_t n_in = raw < inbox_cap ? raw : inbox_cap;
     unsigned long long k[NR];
     uint32_t v[NR];
+    uint32_t old_count = 0;
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         const uint32_t e = NR * lane + r;
@@ -490,6 +502,7 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
             if (id != kInvalid) {
                 k[r] = (static_cast<unsigned long long>(__float_as_uint(d)) << 32) | (static_cast<unsigned long long>(id & ~kOld) << 1);
                 v[r] = id & kOld;
+                old_count += (id & kOld) != 0;
             }
         } else if (e - width < n_in) {
             const uint2 o = inbox[static_cast<size_t>(node) * inbox_cap + (e - width)];
@@ -497,31 +510,46 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
             v[r] = 0;   // offers enter as new
         }
     }
+    // old samples from the incoming list (element order = list order)
+    uint32_t total_old;
+    {
+        uint32_t rank = wave_exclusive_scan(old_count, lane, total_old);
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            if (k[r] != ~0ull && !(k[r] & 1ull) && (v[r] & kOld)) {
+                if (rank < kSamples) fwd_old[static_cast<size_t>(node) * kSamples + rank] = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+                rank++;
+            }
+        }
+    }
     Net64<M>::sort(k, v, lane);
-    // drop repeats of an id (equal id => equal distance => adjacent after the sort; the list's own copy sorts first)
-    uint32_t keep_count = 0, offer_count = 0, old_count = 0;
-    bool keep[NR], offer[NR];
+    // Equal id => equal distance => adjacent after the sort, the list's own copy first.  An id's first offered copy
+    // represents the offer; it is "known" when the list already holds the id.
+    bool from_list[NR], first_offer[NR], known[NR];
+    uint32_t offer_count = 0;
     const unsigned long long last_of_prev = __shfl_up(k[NR - 1], 1);
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         const unsigned long long prev = r == 0 ? last_of_prev : k[r - 1];
-        const bool first = (r == 0 && lane == 0);
-        keep[r] = k[r] != ~0ull && (first || (prev >> 1) != (k[r] >> 1));
-        offer[r] = keep[r] && (k[r] & 1ull);
-        keep_count += keep[r];
-        offer_count += offer[r];
+        const bool head = (r == 0 && lane == 0);
+        const bool valid = k[r] != ~0ull;
+        const bool same_id = !head && (prev >> 1) == (k[r] >> 1);
+        from_list[r] = valid && !(k[r] & 1ull) && !same_id;   // a repeated id inside the list (random start) is dropped
+        first_offer[r] = valid && (k[r] & 1ull) && (!same_id || !(prev & 1ull));
+        known[r] = first_offer[r] && same_id;
+        offer_count += first_offer[r];
     }
-    uint32_t total_keep, total_offer, total_new, total_old;
-    uint32_t pos = wave_exclusive_scan(keep_count, lane, total_keep);
+    uint32_t total_offer, total_keep, total_new;
     uint32_t orank = wave_exclusive_scan(offer_count, lane, total_offer);
-    // Bloom check of the best 32 offers against the filter as it was before this round
-    bool fresh[NR];
-    uint32_t fresh_count = 0;
+    bool keep[NR], fresh[NR];
+    uint32_t keep_count = 0, fresh_count = 0;
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         fresh[r] = false;
-        if (offer[r]) {
+        keep[r] = from_list[r];
+        if (first_offer[r]) {
             if (orank < kSamples) {
+                keep[r] = !known[r];
                 const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
                 const uint32_t base = (id % bloom_sets) * 512;
                 uint32_t h = bloom_h0(id);
@@ -535,43 +563,30 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
             }
             orank++;
         }
+        keep_count += keep[r];
         fresh_count += fresh[r];
     }
+    uint32_t pos = wave_exclusive_scan(keep_count, lane, total_keep);
     uint32_t nrank = wave_exclusive_scan(fresh_count, lane, total_new);
-    // old samples: list entries (final position < width) that were flagged old before this round
-    uint32_t p2 = pos;
-    bool oldf[NR];
-#pragma unroll
-    for (int r = 0; r < NR; r++) {
-        oldf[r] = keep[r] && p2 < width && (v[r] & kOld) != 0;
-        old_count += oldf[r];
-        p2 += keep[r];
-    }
-    uint32_t orank_old = wave_exclusive_scan(old_count, lane, total_old);
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
         uint32_t flag = v[r];
-        if (fresh[r]) {
-            if (nrank < kSamples) {
-                fwd_new[static_cast<size_t>(node) * kSamples + nrank] = id;
-                flag = kOld;
-                const uint32_t base = (id % bloom_sets) * 512;
-                uint32_t h = bloom_h0(id);
-                const uint32_t b0 = base + h % 512;
-                h += bloom_h1(id);
-                const uint32_t b1 = base + h % 512;
-                h += bloom_h1(id);
-                const uint32_t b2 = base + h % 512;
-                atomicOr(&filter[b0 >> 5], 1u << (b0 & 31));
-                atomicOr(&filter[b1 >> 5], 1u << (b1 & 31));
-                atomicOr(&filter[b2 >> 5], 1u << (b2 & 31));
-            }
+        if (fresh[r]) {   // at most 32 of them: all become samples
+            fwd_new[static_cast<size_t>(node) * kSamples + nrank] = id;
             nrank++;
-        }
-        if (oldf[r]) {
-            if (orank_old < kSamples) fwd_old[static_cast<size_t>(node) * kSamples + orank_old] = id;
-            orank_old++;
+            flag = kOld;
+            const uint32_t base = (id % bloom_sets) * 512;
+            uint32_t h = bloom_h0(id);
+            const uint32_t b0 = base + h % 512;
+            h += bloom_h1(id);
+            const uint32_t b1 = base + h % 512;
+            h += bloom_h1(id);
+            const uint32_t b2 = base + h % 512;
+            atomicOr(&filter[b0 >> 5], 1u << (b0 & 31));
+            atomicOr(&filter[b1 >> 5], 1u << (b1 & 31));
+            atomicOr(&filter[b2 >> 5], 1u << (b2 & 31));
         }
         if (keep[r]) {
             if (pos < width) {
@@ -589,7 +604,7 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
     if (static_cast<uint32_t>(lane) < bloom_words) bloom[static_cast<size_t>(node) * bloom_words + lane] = filter[lane];
     if (lane == 0) {
         inbox_counts[node] = 0;
-        counts[static_cast<size_t>(node) * 4 + 0] = total_new < kSamples ? total_new : kSamples;
+        counts[static_cast<size_t>(node) * 4 + 0] = total_new;
         counts[static_cast<size_t>(node) * 4 + 1] = total_old < kSamples ? total_old : kSamples;
         counts[static_cast<size_t>(node) * 4 + 2] = 0;
         counts[static_cast<size_t>(node) * 4 + 3] = 0;
@@ -645,7 +660,7 @@ using namespace glide;
 
 namespace {
 uint32_t nnd_width(uint32_t degree) { return round_up32(static_cast<uint32_t>(degree * (degree <= 32 ? 1.0 : 1.3))); }  // nn_descent.cuh:1427-1428
-uint32_t nnd_inbox_cap(uint32_t width) { return 256 - width; }   // list + inbox fill one 256-element sort
+uint32_t nnd_inbox_cap(uint32_t width) { return (getenv("GLIDE_EXP_CAP512") ? 512 : 256) - width; }   // list + inbox fill one 256-element sort
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
 struct NndLayout {
@@ -685,64 +700,164 @@ size_t glide_hip_nnd_workspace_bytes(uint32_t reorder_num, uint32_t dim, uint32_
     return nnd_layout(reorder_num, dim, knn_degree).total;
 }
 
+namespace {
+struct NndCtx {
+    NndLayout l;
+    _Float16* half_rows;
+    float* norms;
+    uint32_t* list_ids;
+    float* list_dists;
+    uint32_t *fwd_new, *fwd_old, *rev_new, *rev_old, *counts, *inbox_counts;
+    uint2* inbox;
+    uint32_t* bloom;
+    unsigned long long* stats;
+    Segments segs;
+    uint32_t n;
+    hipStream_t s;
+};
+
+int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
+                uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!segment_starts || !segment_lengths || !workspace) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim == 0 || segment_num == 0 || knn_degree == 0 || reorder_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // also keeps the Bloom filter within 64 words
+    c.l = nnd_layout(reorder_num, dim, knn_degree);
+    if (c.l.bloom_sets > 4) return GLIDE_ERR_UNSUPPORTED;
+    if (workspace_bytes < c.l.total || reinterpret_cast<uintptr_t>(workspace) % 16) return GLIDE_ERR_BAD_ARGUMENT;
+    unsigned char* w = static_cast<unsigned char*>(workspace);
+    c.half_rows = reinterpret_cast<_Float16*>(w + c.l.half_rows);
+    c.norms = reinterpret_cast<float*>(w + c.l.norms);
+    c.list_ids = reinterpret_cast<uint32_t*>(w + c.l.list_ids);
+    c.list_dists = reinterpret_cast<float*>(w + c.l.list_dists);
+    c.fwd_new = reinterpret_cast<uint32_t*>(w + c.l.fwd_new);
+    c.fwd_old = reinterpret_cast<uint32_t*>(w + c.l.fwd_old);
+    c.rev_new = reinterpret_cast<uint32_t*>(w + c.l.rev_new);
+    c.rev_old = reinterpret_cast<uint32_t*>(w + c.l.rev_old);
+    c.counts = reinterpret_cast<uint32_t*>(w + c.l.counts);
+    c.inbox_counts = reinterpret_cast<uint32_t*>(w + c.l.inbox_counts);
+    c.inbox = reinterpret_cast<uint2*>(w + c.l.inbox);
+    c.bloom = reinterpret_cast<uint32_t*>(w + c.l.bloom);
+    c.stats = reinterpret_cast<unsigned long long*>(w + c.l.stats);
+    c.segs = Segments{segment_starts, segment_lengths, segment_num};
+    c.n = reorder_num;
+    c.s = as_stream(stream);
+    return GLIDE_OK;
+}
+
+int nnd_prepare(const NndCtx& c, const float* data, uint32_t dim, uint32_t seed) {
+    int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(c.stats), 0u, 1024 * 4, c.s);
+    if (rc != GLIDE_OK) return rc;
+    rc = glide_hip_fill_u32(c.bloom, 0u, static_cast<size_t>(c.n) * c.l.bloom_sets * 16, c.s);
+    if (rc != GLIDE_OK) return rc;
+    hipLaunchKernelGGL(nnd_prepare_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, data, c.n, dim, c.l.dim_pad, c.half_rows, c.norms);
+    hipLaunchKernelGGL(nnd_init_kernel, dim3(ceil_div(c.n * c.l.width, 256)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.n,
+                       c.l.width, c.segs, seed);
+    // first samples come from the random lists (sample_graph(true), nn_descent.cuh:1266); later ones from the merge
+    hipLaunchKernelGGL(nnd_sample_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.n, c.l.width, c.segs, c.fwd_new, c.fwd_old, c.counts);
+    return launch_status();
+}
+
+int nnd_reverse(const NndCtx& c) {
+    hipLaunchKernelGGL(nnd_reverse_kernel, dim3(ceil_div(c.n * 64, 256)), dim3(256), 0, c.s, c.fwd_new, c.fwd_old, c.counts, c.rev_new, c.rev_old, c.n,
+                       c.segs);
+    return launch_status();
+}
+
+int nnd_join(const NndCtx& c) {
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(sizeof(JoinLds))));
+    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.counts, c.list_dists, c.inbox_counts, c.inbox, c.stats,
+                c.n, c.l.dim_pad, c.l.width, c.l.cap, c.segs};
+    hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja);
+    return launch_status();
+}
+
+int nnd_merge(const NndCtx& c, bool with_stats) {
+    unsigned long long* stats = with_stats ? c.stats : nullptr;
+    const uint32_t m = c.l.width + c.l.cap;
+    if (m <= 128) {
+        hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
+                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats);
+    } else {
+        hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
+                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats);
+    }
+    return launch_status();
+}
+
+int nnd_finalize(const NndCtx& c, uint32_t knn_degree, uint32_t* knn_graph, unsigned long long* stats_out) {
+    hipLaunchKernelGGL(nnd_finalize_kernel, dim3(ceil_div(c.n * knn_degree, 256)), dim3(256), 0, c.s, c.list_ids, c.n, c.l.width, knn_degree, c.segs,
+                       knn_graph);
+    if (stats_out) hipLaunchKernelGGL(nnd_stats_reduce_kernel, dim3(1), dim3(1024), 0, c.s, c.stats, stats_out);
+    return launch_status();
+}
+}  // namespace
+
 int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts,
                         const uint32_t* segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations, uint32_t seed,
                         uint32_t* knn_graph, void* workspace, size_t workspace_bytes, unsigned long long* stats_out, void* stream) {
-    if (!reorder_data || !segment_starts || !segment_lengths || !knn_graph || !workspace) return GLIDE_ERR_BAD_ARGUMENT;
-    if (dim == 0 || segment_num == 0 || knn_degree == 0) return GLIDE_ERR_BAD_ARGUMENT;
-    if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // also keeps the Bloom filter within 64 words
-    if (reorder_num == 0) return GLIDE_OK;
-    const NndLayout l = nnd_layout(reorder_num, dim, knn_degree);
-    if (l.bloom_sets > 4) return GLIDE_ERR_UNSUPPORTED;
-    if (workspace_bytes < l.total || reinterpret_cast<uintptr_t>(workspace) % 16) return GLIDE_ERR_BAD_ARGUMENT;
-    hipStream_t s = as_stream(stream);
-    unsigned char* w = static_cast<unsigned char*>(workspace);
-    _Float16* half_rows = reinterpret_cast<_Float16*>(w + l.half_rows);
-    float* norms = reinterpret_cast<float*>(w + l.norms);
-    uint32_t* list_ids = reinterpret_cast<uint32_t*>(w + l.list_ids);
-    float* list_dists = reinterpret_cast<float*>(w + l.list_dists);
-    uint32_t* fwd_new = reinterpret_cast<uint32_t*>(w + l.fwd_new);
-    uint32_t* fwd_old = reinterpret_cast<uint32_t*>(w + l.fwd_old);
-    uint32_t* rev_new = reinterpret_cast<uint32_t*>(w + l.rev_new);
-    uint32_t* rev_old = reinterpret_cast<uint32_t*>(w + l.rev_old);
-    uint32_t* counts = reinterpret_cast<uint32_t*>(w + l.counts);
-    uint32_t* inbox_counts = reinterpret_cast<uint32_t*>(w + l.inbox_counts);
-    uint2* inbox = reinterpret_cast<uint2*>(w + l.inbox);
-    uint32_t* bloom = reinterpret_cast<uint32_t*>(w + l.bloom);
-    unsigned long long* stats = stats_out ? reinterpret_cast<unsigned long long*>(w + l.stats) : nullptr;
-    const Segments segs{segment_starts, segment_lengths, segment_num};
-    const uint32_t n = reorder_num;
-
-    if (stats) {
-        int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(stats), 0u, 1024 * 4, stream);
-        if (rc != GLIDE_OK) return rc;
-    }
-    hipLaunchKernelGGL(nnd_prepare_kernel, dim3(ceil_div(n, 4)), dim3(256), 0, s, reorder_data, n, dim, l.dim_pad, half_rows, norms);
-    hipLaunchKernelGGL(nnd_init_kernel, dim3(ceil_div(n * l.width, 256)), dim3(256), 0, s, list_ids, list_dists, inbox_counts, n, l.width, segs, seed);
-    JoinArgs ja{half_rows, norms, fwd_new, fwd_old, rev_new, rev_old, counts, list_dists, inbox_counts, inbox, stats, n, l.dim_pad, l.width, l.cap, segs};
-    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      static_cast<int>(sizeof(JoinLds))));
-    {
-        int rc = glide_hip_fill_u32(bloom, 0u, static_cast<size_t>(n) * l.bloom_sets * 16, stream);
-        if (rc != GLIDE_OK) return rc;
-    }
-    // first samples come from the random lists (sample_graph(true), nn_descent.cuh:1266); later ones from the merge
-    hipLaunchKernelGGL(nnd_sample_kernel, dim3(ceil_div(n, 4)), dim3(256), 0, s, list_ids, n, l.width, segs, fwd_new, fwd_old, counts);
+    if (!reorder_data || !knn_graph) return GLIDE_ERR_BAD_ARGUMENT;
+    if (reorder_num == 0 && segment_starts && segment_lengths && workspace && dim && segment_num && knn_degree) return GLIDE_OK;
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    if (rc != GLIDE_OK) return rc;
+    if ((rc = nnd_prepare(c, reorder_data, dim, seed)) != GLIDE_OK) return rc;
     for (uint32_t it = 0; it < iterations; it++) {
-        hipLaunchKernelGGL(nnd_reverse_kernel, dim3(ceil_div(n * 64, 256)), dim3(256), 0, s, fwd_new, fwd_old, counts, rev_new, rev_old, n, segs);
-        hipLaunchKernelGGL(nnd_join_kernel, dim3(n), dim3(256), sizeof(JoinLds), s, ja);
-        const uint32_t m = l.width + l.cap;
-        if (m <= 128) {
-            hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(n, 4)), dim3(256), 0, s, list_ids, list_dists, inbox_counts, inbox, n, l.width, l.cap,
-                               bloom, l.bloom_sets, fwd_new, fwd_old, counts, stats);
-        } else {
-            hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(n, 4)), dim3(256), 0, s, list_ids, list_dists, inbox_counts, inbox, n, l.width, l.cap,
-                               bloom, l.bloom_sets, fwd_new, fwd_old, counts, stats);
-        }
+        if ((rc = nnd_reverse(c)) != GLIDE_OK) return rc;
+        if ((rc = nnd_join(c)) != GLIDE_OK) return rc;
+        if ((rc = nnd_merge(c, stats_out != nullptr)) != GLIDE_OK) return rc;
     }
-    hipLaunchKernelGGL(nnd_finalize_kernel, dim3(ceil_div(n * knn_degree, 256)), dim3(256), 0, s, list_ids, n, l.width, knn_degree, segs, knn_graph);
-    if (stats_out) hipLaunchKernelGGL(nnd_stats_reduce_kernel, dim3(1), dim3(1024), 0, s, stats, stats_out);
-    return launch_status();
+    return nnd_finalize(c, knn_degree, knn_graph, stats_out);
+}
+
+int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree, glide_nnd_layout* out) {
+    if (!out || dim == 0 || knn_degree == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    const NndLayout l = nnd_layout(reorder_num, dim, knn_degree);
+    out->half_rows = l.half_rows; out->norms = l.norms; out->list_ids = l.list_ids; out->list_dists = l.list_dists;
+    out->fwd_new = l.fwd_new; out->fwd_old = l.fwd_old; out->rev_new = l.rev_new; out->rev_old = l.rev_old;
+    out->counts = l.counts; out->inbox_counts = l.inbox_counts; out->inbox = l.inbox; out->bloom = l.bloom; out->total = l.total;
+    out->width = l.width; out->inbox_cap = l.cap; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
+    return GLIDE_OK;
+}
+
+int glide_hip_nnd_prepare(const float* reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts,
+                          const uint32_t* segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t seed, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+    if (!reorder_data) return GLIDE_ERR_BAD_ARGUMENT;
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    return rc != GLIDE_OK ? rc : nnd_prepare(c, reorder_data, dim, seed);
+}
+
+int glide_hip_nnd_reverse_sample(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
+                                 uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    return rc != GLIDE_OK ? rc : nnd_reverse(c);
+}
+
+int glide_hip_nnd_local_join(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
+                             uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    return rc != GLIDE_OK ? rc : nnd_join(c);
+}
+
+int glide_hip_nnd_merge(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
+                        uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    return rc != GLIDE_OK ? rc : nnd_merge(c, true);
+}
+
+int glide_hip_nnd_finalize(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
+                           uint32_t segment_num, uint32_t knn_degree, uint32_t* knn_graph, unsigned long long* stats_out, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    if (!knn_graph) return GLIDE_ERR_BAD_ARGUMENT;
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    return rc != GLIDE_OK ? rc : nnd_finalize(c, knn_degree, knn_graph, stats_out);
 }
 
 }  // extern "C"

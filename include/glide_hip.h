@@ -125,6 +125,44 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
                         uint32_t knn_degree, uint32_t iterations, uint32_t seed, uint32_t *knn_graph,
                         void *workspace, size_t workspace_bytes, unsigned long long *stats_out, void *stream);
 
+/* The same build one stage per call, on the same workspace (the stages of GNND::build's loop, nn_descent.cuh:1289-1368):
+ *   prepare         preprocess_data_kernel :445 (fp16 rows + fp32 squared norms), init_random_graph :1003,
+ *                   Bloom filter cleared, first samples (sample_graph(true) :1040-1071)
+ *   reverse_sample  add_rev_edges_kernel :490-507
+ *   local_join      local_join_kernel :668-914; offers go to the per-node inbox instead of a spin-locked list
+ *   merge           update_graph :1106-1126 + sample_graph_new :973-1001 + sample_segment_graph :1073-1104
+ *   finalize        the shrink step :1376-1402
+ * glide_hip_nnd_build = prepare, `iterations` x (reverse_sample, local_join, merge), finalize.
+ * glide_hip_nnd_layout reports where each array lives in the workspace (byte offsets), so a caller or a test can
+ * inspect or replace any of them between stages:
+ *   list_ids   num x width u32: partition-local id | 0x80000000 ("already sampled"), 0xffffffff = empty; nearest first
+ *   list_dists num x width f32 (squared L2 of the fp16 rows, FLT_MAX for the random start entries)
+ *   fwd_new / fwd_old / rev_new / rev_old  num x 32 u32 sample lists; counts num x 4 u32 = their lengths
+ *                   (reverse lengths count every arrival and may exceed 32; 32 are stored)
+ *   inbox      num x inbox_cap x (u32 distance bits, u32 id); inbox_counts num u32 (arrivals, may exceed inbox_cap)
+ *   bloom      num x bloom_sets x 512 bits */
+typedef struct {
+    uint64_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, counts, inbox_counts, inbox, bloom, total;
+    uint32_t width, inbox_cap, row_halfs, bloom_sets;
+} glide_nnd_layout;
+int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree, glide_nnd_layout *out);
+int glide_hip_nnd_prepare(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                          const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t seed,
+                          void *workspace, size_t workspace_bytes, void *stream);
+int glide_hip_nnd_reverse_sample(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                                 const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+int glide_hip_nnd_local_join(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                             const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
+                             void *workspace, size_t workspace_bytes, void *stream);
+int glide_hip_nnd_merge(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                        const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
+                        void *workspace, size_t workspace_bytes, void *stream);
+int glide_hip_nnd_finalize(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                           const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
+                           uint32_t *knn_graph, unsigned long long *stats_out, void *workspace, size_t workspace_bytes,
+                           void *stream);
+
 /* ---- graph construction (subsystem 3) ----------------------------------------------------------------------
  * All kernels give one point to one wavefront.  Limits as for glide_hip_search (knn_degree, graph_degree <= 128,
  * beam <= 256, dim % 4 == 0, dim <= 1024).  `counters` as in glide_hip_search (prune distances count as rows). */
