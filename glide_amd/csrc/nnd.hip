@@ -73,9 +73,34 @@ __global__ __launch_bounds__(256) void nnd_prepare_kernel(const float* data, uin
     if (lane == 0) norms[i] = acc;
 }
 
-// ---- random initial lists (reference init_random_graph :1003-1038 uses shuffled sequences on the host)
+// ---- random initial lists.  The reference (init_random_graph :1003-1038) shuffles one sequence of len / num_sub values
+// per sub-list on the host and hands out consecutive runs of it: entry j of sub-list `sub` of node i is
+// seq_sub[(i * width + 32 * sub + j) % m] * num_sub + sub.  Every id therefore starts with the same in-degree and
+// neighbouring nodes start with disjoint lists, which shapes the first rounds; the same construction is used here,
+// with a keyed bijection (a cycle-walking Feistel network) in place of the host-side shuffle.
 __device__ __forceinline__ uint32_t mix32(uint32_t x) {
     x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    return x;
+}
+
+// A permutation of [0, m): four Feistel rounds on the smallest even number of bits covering m, re-applied until the
+// value falls below m (at most 4 m values in the domain, so a few rounds on average; every walk ends because the
+// network is a bijection of the domain).
+__device__ __forceinline__ uint32_t permute(uint32_t x, uint32_t m, uint32_t key) {
+    if (m <= 1) return 0;
+    uint32_t bits = 32 - __clz(m - 1);
+    bits = bits < 2 ? 2 : (bits + 1) & ~1u;
+    const uint32_t half = bits / 2, mask = (1u << half) - 1;
+    do {
+        uint32_t l = x >> half, r = x & mask;
+#pragma unroll
+        for (uint32_t round = 0; round < 4; round++) {
+            const uint32_t t = l ^ (mix32(r ^ (key + round * 0x9E3779B9u)) & mask);
+            l = r;
+            r = t;
+        }
+        x = (l << half) | r;
+    } while (x >= m);
     return x;
 }
 
@@ -87,22 +112,17 @@ __global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t* list_ids, float
     uint32_t start, len;
     locate(segs, node, start, len);
     const uint32_t local = node - start;
-    // width distinct pseudo-random partition-local neighbours, never the node itself: the partition is cut into
-    // width + 1 strata (rotated by a per-node offset), entry j draws from stratum j, and the entry that would hit the
-    // node itself draws from the spare stratum instead.  Partitions with fewer than width + 2 points list every other point.
-    uint32_t id = kInvalid;
-    const uint32_t stride = len / (width + 1);
-    if (stride >= 1) {
-        const uint32_t h = mix32(node + seed * 0x9E3779B9u);
-        const uint32_t rot = h % len;
-        auto draw = [&](uint32_t stratum) { return (rot + stratum * stride + mix32(h ^ (stratum * 0x85EBCA6Bu + 1u)) % stride) % len; };
-        id = draw(j);
-        if (id == local) id = draw(width);
-    } else if (j + 1 < len) {
-        id = (local + 1 + j) % len;
-    }
-    list_ids[static_cast<size_t>(node) * width + j] = id;   // new (flag clear)
-    list_dists[static_cast<size_t>(node) * width + j] = FLT_MAX;
+    const uint32_t num_sub = width / kSamples, sub = j / kSamples;
+    const uint32_t m = len / num_sub > 1 ? len / num_sub : 1;
+    const uint32_t key = mix32(seed * 7919u + sub + 0x5bd1e995u * start);
+    const uint32_t at = local * width + j;
+    uint32_t id = permute(at % m, m, key) * num_sub + sub;
+    if (id == local) id = permute((at + kSamples) % m, m, key) * num_sub + sub;
+    if (id >= len || id == local) id = kInvalid;   // partitions too small to fill a list
+    // stored column-major over the sub-lists, the order in which the first samples are taken (:1052-1068)
+    const uint32_t slot = (j % kSamples) * num_sub + sub;
+    list_ids[static_cast<size_t>(node) * width + slot] = id;   // new (flag clear)
+    list_dists[static_cast<size_t>(node) * width + slot] = FLT_MAX;
     if (j == 0) inbox_counts[node] = 0;
 }
 
