@@ -74,6 +74,7 @@ struct Beam {
     BeamParams p;
     BeamCounters cnt;
     int lane;
+    uint32_t last_scored;   // rows scored by the latest expansion (wave-uniform)
 
     __device__ __forceinline__ void init(BeamLds<MAX_CAND>* lds_, uint32_t* hash_, const BeamParams& p_, const float* query) {
         lds = lds_;
@@ -108,6 +109,7 @@ struct Beam {
         }
         wave_sync();
         cnt.rows_scored += nv;
+        last_scored = nv;
         BeamLds<MAX_CAND>* l = lds;
         score_list<DIMV>(q, data, p.dim, p.metric, 0, nv, lane,
                          [l](uint32_t idx) { return l->cand_id[l->vlist[idx]]; },
@@ -117,6 +119,9 @@ struct Beam {
 
     // reference update_result_buffer: sort the candidates, then fold them into the beam
     __device__ __forceinline__ void absorb(bool first) {
+        // No row scored: every candidate distance is FLT_MAX, the sort would not move anything (equal keys are never
+        // exchanged) and no candidate can displace a beam entry, so the beam stays as it is.
+        if (!first && last_scored == 0) return;
         float ck[NC];
         uint32_t cv[NC];
 #pragma unroll
@@ -145,6 +150,7 @@ struct Beam {
                 bv[r] = take ? lds->cand_id[e] : kInvalid;
             }
         } else {
+            bool replaced = false;
 #pragma unroll
             for (int r = 0; r < NB; r++) {
                 const uint32_t e = NB * lane + r;
@@ -154,16 +160,21 @@ struct Beam {
                     if (bk[r] > c) {
                         bk[r] = c;
                         bv[r] = lds->cand_id[k];
+                        replaced = true;
                     }
                 }
             }
-            WaveNet<MAX_BEAM>::merge(bk, bv, lane);
+            // Nothing replaced: the beam is still the ascending sequence the previous merge left, and the merge
+            // network (strict comparisons) is the identity on it.
+            if (ballot(replaced) != 0) {
+                WaveNet<MAX_BEAM>::merge(bk, bv, lane);
 #pragma unroll
-            for (int r = 0; r < NB; r++) {
-                const uint32_t e = NB * lane + r;
-                if (e >= p.beam) {
-                    bk[r] = FLT_MAX;
-                    bv[r] = kInvalid;
+                for (int r = 0; r < NB; r++) {
+                    const uint32_t e = NB * lane + r;
+                    if (e >= p.beam) {
+                        bk[r] = FLT_MAX;
+                        bv[r] = kInvalid;
+                    }
                 }
             }
         }

@@ -22,15 +22,35 @@ struct WaveNet {
             uint32_t tv = v0; v0 = v1; v1 = tv;
         }
     }
-    // compare-exchange with the lane `lane ^ LM` (bitonic.cuh:36-44); keep_min: this lane keeps the smaller key
+    // Lanes that keep the smaller key in stage (K, J) for register r: bit l set <=> lane l is the lower partner of an
+    // ascending pair or the upper partner of a descending one.  A compile-time constant.
+    template <int K, int J>
+    static constexpr uint64_t keep_min_mask(int r) {
+        constexpr int LM = J / NR;
+        uint64_t m = 0;
+        for (int l = 0; l < 64; l++) {
+            const int e = NR * l + r;
+            const bool asc = (K >= M) ? true : ((e & K) == 0);
+            const bool lower = (l & LM) == 0;
+            if (lower == asc) m |= 1ull << l;
+        }
+        return m;
+    }
+    // compare-exchange with the lane `lane ^ LM` (bitonic.cuh:36-44): a lane that keeps the minimum takes the partner's
+    // pair iff partner < mine, a lane that keeps the maximum iff mine < partner.  Both tests are strict, so equal keys
+    // are never exchanged (the reference's k0 != k1 guard).  The two predicates are combined with the constant
+    // keep-min mask on the scalar unit; for the half-swap (LM = 32) the second predicate is the first with its halves
+    // swapped, which costs no vector instruction.  (The scalar unit is shared by the four SIMDs of a CU, so longer
+    // scalar sequences that would save the second compare for the other distances do not pay.)
     template <int LM>
-    static __device__ __forceinline__ void cmpx_lane(float& k, uint32_t& v, bool keep_min) {
+    static __device__ __forceinline__ void cmpx_lane(float& k, uint32_t& v, uint64_t keep_min) {
         const float ok = lane_xor<LM>(k);
         const uint32_t ov = lane_xor<LM>(v);
-        if ((k != ok) && ((k < ok) != keep_min)) {
-            k = ok;
-            v = ov;
-        }
+        const uint64_t less = __builtin_amdgcn_ballot_w64(ok < k);
+        const uint64_t more = LM == 32 ? mask_xor<32>(less) : __builtin_amdgcn_ballot_w64(k < ok);
+        const uint64_t take = (less & keep_min) | (more & ~keep_min);
+        k = select_by_mask(k, ok, take);
+        v = select_by_mask(v, ov, take);
     }
 
     // one network stage: partner distance J (elements), direction block K (elements); K == M means all ascending
@@ -47,13 +67,8 @@ struct WaveNet {
             }
         } else {
             constexpr int LM = J / NR;
-            const bool lower = (lane & LM) == 0;
 #pragma unroll
-            for (int r = 0; r < NR; r++) {
-                const int e = NR * lane + r;
-                const bool asc = (K >= M) ? true : ((e & K) == 0);
-                cmpx_lane<LM>(k[r], v[r], lower == asc);
-            }
+            for (int r = 0; r < NR; r++) cmpx_lane<LM>(k[r], v[r], keep_min_mask<K, J>(r));
         }
     }
 

@@ -28,21 +28,41 @@ __device__ __forceinline__ int lane_id() { return static_cast<int>(__builtin_amd
 template <int MASK>
 __device__ __forceinline__ int lane_xor_i(int v) {
     static_assert(MASK == 1 || MASK == 2 || MASK == 4 || MASK == 8 || MASK == 16 || MASK == 32, "xor mask");
+    // mov_dpp leaves the destination's previous value undefined for lanes the pattern does not write; every pattern
+    // below writes all 64 lanes, so no register has to be initialised first
     if constexpr (MASK == 1) {
-        return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, false);  // quad_perm:[1,0,3,2]
+        return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xf, 0xf, false);  // quad_perm:[1,0,3,2]
     } else if constexpr (MASK == 2) {
-        return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, false);  // quad_perm:[2,3,0,1]
+        return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xf, 0xf, false);  // quad_perm:[2,3,0,1]
     } else if constexpr (MASK == 4) {
-        int r = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xf, 0x5, false);  // row_shl:4 -> banks 0,2 read lane+4
-        r = __builtin_amdgcn_update_dpp(r, v, 0x114, 0xf, 0xA, false);      // row_shr:4 -> banks 1,3 read lane-4
+        int r = __builtin_amdgcn_mov_dpp(v, 0x104, 0xf, 0x5, false);    // row_shl:4 -> banks 0,2 read lane+4
+        r = __builtin_amdgcn_update_dpp(r, v, 0x114, 0xf, 0xA, false);  // row_shr:4 -> banks 1,3 read lane-4
         return r;
     } else if constexpr (MASK == 8) {
-        return __builtin_amdgcn_update_dpp(v, v, 0x128, 0xf, 0xf, false);  // row_ror:8
+        return __builtin_amdgcn_mov_dpp(v, 0x128, 0xf, 0xf, false);  // row_ror:8
     } else if constexpr (MASK == 16) {
         return __builtin_amdgcn_ds_swizzle(v, 0x401F);  // BITMODE and=0x1f or=0 xor=0x10
     } else {
         return __builtin_amdgcn_ds_bpermute((lane_id() ^ 32) << 2, v);
     }
+}
+// A 64-lane predicate mask with every bit moved to the lane MASK away (the partner's predicate), on the scalar unit.
+template <int MASK>
+__device__ __forceinline__ uint64_t mask_xor(uint64_t m) {
+    constexpr uint64_t low = MASK == 1 ? 0x5555555555555555ull : MASK == 2 ? 0x3333333333333333ull : MASK == 4 ? 0x0F0F0F0F0F0F0F0Full
+                           : MASK == 8 ? 0x00FF00FF00FF00FFull : MASK == 16 ? 0x0000FFFF0000FFFFull : 0x00000000FFFFFFFFull;
+    return ((m & low) << MASK) | ((m >> MASK) & low);
+}
+// per-lane select driven by a scalar 64-bit mask: lane l gets `b` where bit l is set, else `a`
+__device__ __forceinline__ float select_by_mask(float a, float b, uint64_t mask) {
+    float out;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(out) : "v"(a), "v"(b), "s"(mask));
+    return out;
+}
+__device__ __forceinline__ uint32_t select_by_mask(uint32_t a, uint32_t b, uint64_t mask) {
+    uint32_t out;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(out) : "v"(a), "v"(b), "s"(mask));
+    return out;
 }
 template <int MASK>
 __device__ __forceinline__ float lane_xor(float v) { return __builtin_bit_cast(float, lane_xor_i<MASK>(__builtin_bit_cast(int, v))); }

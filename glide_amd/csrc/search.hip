@@ -35,26 +35,27 @@ __global__ __launch_bounds__(64) void search_kernel(SearchArgs a) {
     auto* lds = reinterpret_cast<BeamLds<MAX_CAND>*>(smem);
     float* cent = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>));
     uint32_t* hash = reinterpret_cast<uint32_t*>(cent + round_up32(a.centroid_num));
-    const uint32_t qid = blockIdx.x;
-    if (qid >= a.query_num) return;
+    // a wavefront takes queries blockIdx.x, blockIdx.x + gridDim.x, ... (the host sizes the grid)
+    for (uint32_t qid = blockIdx.x; qid < a.query_num; qid += gridDim.x) {
+        Beam<MAX_CAND, MAX_BEAM, DIMV> b;
+        b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
+        const uint32_t c0 = pick_centroid<DIMV>(a.max_centroid, b.q, a.centroids, a.centroid_num, a.p.dim, a.p.metric, cent, b.lane);
+        const uint32_t entry = a.start_points[c0];
+        b.expand(entry, a.graph, a.data, kInvalid, kInvalid);  // result_init: entry node itself is never scored
+        b.run(a.graph, a.data, kInvalid);
 
-    Beam<MAX_CAND, MAX_BEAM, DIMV> b;
-    b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
-    const uint32_t c0 = pick_centroid<DIMV>(a.max_centroid, b.q, a.centroids, a.centroid_num, a.p.dim, a.p.metric, cent, b.lane);
-    const uint32_t entry = a.start_points[c0];
-    b.expand(entry, a.graph, a.data, kInvalid, kInvalid);  // result_init: entry node itself is never scored
-    b.run(a.graph, a.data, kInvalid);
-
-    constexpr int NB = MAX_BEAM / 64;
+        constexpr int NB = MAX_BEAM / 64;
 #pragma unroll
-    for (int r = 0; r < NB; r++) {
-        const uint32_t e = NB * b.lane + r;
-        if (e < a.top_k) {
-            a.result_ids[static_cast<size_t>(qid) * a.top_k + e] = b.bv[r] & kClean;
-            a.result_dists[static_cast<size_t>(qid) * a.top_k + e] = b.bk[r];
+        for (int r = 0; r < NB; r++) {
+            const uint32_t e = NB * b.lane + r;
+            if (e < a.top_k) {
+                a.result_ids[static_cast<size_t>(qid) * a.top_k + e] = b.bv[r] & kClean;
+                a.result_dists[static_cast<size_t>(qid) * a.top_k + e] = b.bk[r];
+            }
         }
+        b.flush_counters(a.counters);
+        wave_sync();   // the next query reuses the LDS
     }
-    b.flush_counters(a.counters);
 }
 
 // ---- large path: one staged partition at a time ---------------------------------------------------------------
@@ -251,6 +252,23 @@ search_fn pick_beam(uint32_t beam, uint32_t dim) {
     return pick_dim<MAX_CAND, 256>(dim);
 }
 
+// Grid size for the one-query-per-wavefront search kernel.  With small beams the kernel is bound by row gathers; when
+// the batch is a little larger than what the chip holds at once (10 000 queries against 8 192 wavefront slots),
+// hardware dispatch runs one full round and a thin, latency-bound tail.  Equal rounds are faster: the grid is the
+// batch divided by the number of rounds and every wavefront loops over its share.  Larger beams are bound by the
+// sorting networks and keep one workgroup per query.
+uint32_t balanced_grid(uint32_t items, uint32_t beam, size_t lds_bytes) {
+    if (beam > 64) return items;
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return items;
+    const size_t by_lds = lds_bytes ? (160 * 1024) / lds_bytes : 32;
+    const size_t slots = static_cast<size_t>(cus) * (by_lds < 32 ? by_lds : 32);   // 4 SIMDs x 8 wavefronts per CU
+    if (slots == 0 || items <= slots) return items;
+    const size_t rounds = (items + slots - 1) / slots;
+    return static_cast<uint32_t>((items + rounds - 1) / rounds);
+}
+
 }  // namespace glide
 
 using namespace glide;
@@ -300,7 +318,7 @@ extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, c
     search_fn fn = max_cand == 64 ? pick_beam<64>(beam, dim) : pick_beam<128>(beam, dim);
     const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) +
                              round_up32(centroid_num) * sizeof(float) + (size_t{1} << hash_bit) * sizeof(uint32_t);
-    hipLaunchKernelGGL(fn, dim3(query_num), dim3(64), lds_bytes, as_stream(stream), a);
+    hipLaunchKernelGGL(fn, dim3(balanced_grid(query_num, beam, lds_bytes)), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }
 
