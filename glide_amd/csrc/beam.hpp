@@ -7,7 +7,7 @@
 // the id's MSB.  The D candidates of one expansion are produced into LDS by graph-row slot, pulled into
 // registers with the reference's strided->blocked permutation, sorted by the wave network and staged back to
 // LDS so that beam element e can pick candidate MAX_BEAM-1-e (the half-cleaner).  The visited set is an LDS
-// open-addressing table.  Data rows are gathered two at a time (one 32-lane half each, 16 B per lane).
+// open-addressing table.  Data rows are gathered several at a time (one lane group each, 16 B per lane and load).
 #pragma once
 #include "bitonic.hpp"
 
@@ -33,18 +33,19 @@ struct BeamLds {  // per-wave LDS (the hash table follows, 1 << hash_bit words)
 
 __device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
 
-// Distances from `ref` to `count` listed rows, two rows per step (one per 32-lane half), U steps in flight.
-// id_of(idx) -> row id of list entry idx; out(idx, dist) is called by one lane per scored row.
+// Distances from `ref` to `count` listed rows, RowShape<DIMV>::ROWS rows per step (one per lane group), U steps in
+// flight.  id_of(idx) -> row id of list entry idx; out(idx, dist) is called by one lane per scored row.
 template <int DIMV, class IdFn, class OutFn>
 __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float* data, uint32_t dim, int metric,
                                            uint32_t first, uint32_t count, int lane, IdFn id_of, OutFn out) {
-    const int half = lane >> 5, t = lane & 31;
-    constexpr int U = DIMV == 1 ? 4 : (DIMV == 2 ? 2 : 1);
-    for (uint32_t base = first; base < count; base += 2 * U) {
+    using Shape = RowShape<DIMV>;
+    const int g = Shape::row_of_lane(lane), t = Shape::lane_in_row(lane);
+    constexpr int U = DIMV == 1 ? 2 : (DIMV == 2 ? 2 : (DIMV == 4 ? 2 : 1));
+    for (uint32_t base = first; base < count; base += Shape::ROWS * U) {
         RowRegs<DIMV> rows[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const uint32_t idx = base + 2 * u + half;
+            const uint32_t idx = base + Shape::ROWS * u + g;
             if (idx < count) {
                 load_row<DIMV>(rows[u], data + static_cast<size_t>(id_of(idx)) * dim, dim, t);
             } else {
@@ -53,8 +54,8 @@ __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const uint32_t idx = base + 2 * u + half;
-            const float d = finish_distance(half_wave_sum(partial_sqdist<DIMV>(ref, rows[u])), metric);
+            const uint32_t idx = base + Shape::ROWS * u + g;
+            const float d = finish_distance(row_sum<DIMV>(partial_sqdist<DIMV>(ref, rows[u])), metric);
             if (t == 0 && idx < count) out(idx, d);
         }
     }
@@ -81,7 +82,7 @@ struct Beam {
         hash = hash_;
         p = p_;
         lane = lane_id();
-        load_row<DIMV>(q, query, p.dim, lane & 31);
+        load_row<DIMV>(q, query, p.dim, RowShape<DIMV>::lane_in_row(lane));
         hash_clear(hash, p.hash_bit, lane);
         wave_sync();
     }
@@ -254,16 +255,17 @@ struct Beam {
 template <int MAX_CENTROID, int DIMV>
 __device__ __forceinline__ uint32_t nearest_centroid(const RowRegs<DIMV>& q, const float* centroids, uint32_t centroid_num,
                                                      uint32_t dim, int metric, float* cent_dist, int lane) {
-    const int half = lane >> 5, t = lane & 31;
-    for (uint32_t c0 = 0; c0 < centroid_num; c0 += 2) {
-        const uint32_t c = c0 + half;
+    using Shape = RowShape<DIMV>;
+    const int g = Shape::row_of_lane(lane), t = Shape::lane_in_row(lane);
+    for (uint32_t c0 = 0; c0 < centroid_num; c0 += Shape::ROWS) {
+        const uint32_t c = c0 + g;
         RowRegs<DIMV> row;
         if (c < centroid_num) {
             load_row<DIMV>(row, centroids + static_cast<size_t>(c) * dim, dim, t);
         } else {
             row = q;
         }
-        const float d = finish_distance(half_wave_sum(partial_sqdist<DIMV>(q, row)), metric);
+        const float d = finish_distance(row_sum<DIMV>(partial_sqdist<DIMV>(q, row)), metric);
         if (t == 0 && c < centroid_num) cent_dist[c] = d;
     }
     wave_sync();

@@ -114,34 +114,65 @@ __device__ __forceinline__ uint32_t hash_insert(uint32_t* table, uint32_t bitlen
     return 0;
 }
 
-// ---------------------------------------------------------------- row distance with a 32-lane half per row
-// Lane t of a half owns dims [c*128 + 4t, c*128 + 4t + 4) of chunk c.  DIMV = number of 128-dim chunks.
+// ---------------------------------------------------------------- row distance, several rows per wave-wide load
+// A row is read by a group of LPR adjacent lanes, 16 bytes per lane and load, NV loads per lane; lane t of a group
+// owns dims [(c*LPR + t)*4, +4) of load c, so one load instruction touches LPR*16 contiguous bytes of each row.
+// Narrow rows use narrow groups: the cross-lane sum then needs log2(LPR) steps instead of 5 and one instruction
+// serves 64/LPR rows.  DIMV selects the shape by row length (dim <= 128*DIMV):
+//   DIMV 1: 8 lanes x 4 loads (8 rows per wavefront)    DIMV 2: 16 lanes x 4 loads (4 rows)
+//   DIMV 4: 32 lanes x 4 loads (2 rows)                 DIMV 8: 32 lanes x 8 loads (2 rows)
 template <int DIMV>
-struct RowRegs {
-    float4 v[DIMV];
+struct RowShape {
+    static_assert(DIMV == 1 || DIMV == 2 || DIMV == 4 || DIMV == 8, "row shape");
+    static constexpr int LPR = DIMV == 1 ? 8 : (DIMV == 2 ? 16 : 32);
+    static constexpr int NV = DIMV == 8 ? 8 : 4;
+    static constexpr int ROWS = 64 / LPR;
+    static __device__ __forceinline__ int lane_in_row(int lane) { return lane & (LPR - 1); }
+    static __device__ __forceinline__ int row_of_lane(int lane) { return lane / LPR; }
 };
 
 template <int DIMV>
+struct RowRegs {
+    float4 v[RowShape<DIMV>::NV];
+};
+
+// t = RowShape<DIMV>::lane_in_row(lane)
+template <int DIMV>
 __device__ __forceinline__ void load_row(RowRegs<DIMV>& r, const float* row, uint32_t dim, int t) {
 #pragma unroll
-    for (int c = 0; c < DIMV; c++) {
-        const uint32_t d0 = c * 128 + t * 4;
+    for (int c = 0; c < RowShape<DIMV>::NV; c++) {
+        const uint32_t d0 = (c * RowShape<DIMV>::LPR + t) * 4;
         r.v[c] = d0 < dim ? *reinterpret_cast<const float4*>(row + d0) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
+}
+
+__device__ __forceinline__ float sqdist4(const float4& a, const float4& b, float acc) {
+    const float dx = a.x - b.x, dy = a.y - b.y, dz = a.z - b.z, dw = a.w - b.w;
+    acc = fmaf(dx, dx, acc);
+    acc = fmaf(dy, dy, acc);
+    acc = fmaf(dz, dz, acc);
+    acc = fmaf(dw, dw, acc);
+    return acc;
 }
 
 template <int DIMV>
 __device__ __forceinline__ float partial_sqdist(const RowRegs<DIMV>& a, const RowRegs<DIMV>& b) {
     float acc = 0.f;
 #pragma unroll
-    for (int c = 0; c < DIMV; c++) {
-        float dx = a.v[c].x - b.v[c].x, dy = a.v[c].y - b.v[c].y, dz = a.v[c].z - b.v[c].z, dw = a.v[c].w - b.v[c].w;
-        acc = fmaf(dx, dx, acc);
-        acc = fmaf(dy, dy, acc);
-        acc = fmaf(dz, dz, acc);
-        acc = fmaf(dw, dw, acc);
-    }
+    for (int c = 0; c < RowShape<DIMV>::NV; c++) acc = sqdist4(a.v[c], b.v[c], acc);
     return acc;
+}
+
+// Sum over each group of LPR lanes; every lane of a group ends with the group's total.
+template <int DIMV>
+__device__ __forceinline__ float row_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+    if constexpr (RowShape<DIMV>::LPR >= 16)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));  // row_mirror
+    if constexpr (RowShape<DIMV>::LPR >= 32) v += lane_xor<16>(v);
+    return v;
 }
 
 // reference distance.cuh:22-26: Euclidean reports sqrt, Cosine the squared L2 of pre-normalised rows

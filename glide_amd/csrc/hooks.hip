@@ -15,10 +15,7 @@ __global__ __launch_bounds__(64) void distance_batch_kernel(const float* a, cons
         const float* x = a + static_cast<size_t>(i) * dim;
         const float* y = b + static_cast<size_t>(i) * dim;
         for (uint32_t d0 = t * 4; d0 < dim; d0 += 128) {
-            RowRegs<1> rx, ry;
-            rx.v[0] = *reinterpret_cast<const float4*>(x + d0);
-            ry.v[0] = *reinterpret_cast<const float4*>(y + d0);
-            acc += partial_sqdist<1>(rx, ry);
+            acc = sqdist4(*reinterpret_cast<const float4*>(x + d0), *reinterpret_cast<const float4*>(y + d0), acc);
         }
     }
     const float d = finish_distance(half_wave_sum(acc), metric);

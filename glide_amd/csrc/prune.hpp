@@ -84,7 +84,7 @@ __device__ __forceinline__ uint32_t prune_pool(PruneLds<MAX_BEAM>* pl, uint32_t 
         if (lane == 0) pl->neighbor[nsize] = head;
         nsize++;
         RowRegs<DIMV> hrow;
-        load_row<DIMV>(hrow, data + static_cast<size_t>(head) * dim, dim, lane & 31);
+        load_row<DIMV>(hrow, data + static_cast<size_t>(head) * dim, dim, RowShape<DIMV>::lane_in_row(lane));
         rows_scored += pool_size - 1;
         score_list<DIMV>(hrow, data, dim, metric, 1, pool_size, lane,
                          [pl, segment_start](uint32_t idx) { return pl->pool_id[idx] + segment_start; },
@@ -121,7 +121,7 @@ __device__ __forceinline__ uint32_t prune_pool_refine(PruneLds<MAX_BEAM>* pl, ui
         if (lane == 0) pl->neighbor[nsize] = head;
         nsize++;
         RowRegs<DIMV> hrow;
-        load_row<DIMV>(hrow, data + static_cast<size_t>(head) * dim, dim, lane & 31);
+        load_row<DIMV>(hrow, data + static_cast<size_t>(head) * dim, dim, RowShape<DIMV>::lane_in_row(lane));
         rows_scored += pool_size - position;
         score_list<DIMV>(hrow, data, dim, metric, position, pool_size, lane,
                          [pl](uint32_t idx) { return pl->pool_id[idx]; },

@@ -85,10 +85,8 @@ __global__ __launch_bounds__(64) void select_segments_kernel(SelectArgs a) {
         const uint32_t c = c0 + half < a.centroid_num ? c0 + half : c0;
         float acc = 0.f;
         for (uint32_t d0 = t * 4; d0 < a.dim; d0 += 128) {
-            RowRegs<1> x, y;
-            x.v[0] = *reinterpret_cast<const float4*>(query + d0);
-            y.v[0] = *reinterpret_cast<const float4*>(a.centroids + static_cast<size_t>(c) * a.dim + d0);
-            acc += partial_sqdist<1>(x, y);
+            acc = sqdist4(*reinterpret_cast<const float4*>(query + d0),
+                          *reinterpret_cast<const float4*>(a.centroids + static_cast<size_t>(c) * a.dim + d0), acc);
         }
         const float d = finish_distance(half_wave_sum(acc), a.metric);
         if (t == 0 && c0 + half < a.centroid_num) cent_dist[c0 + half] = d;
