@@ -43,6 +43,8 @@ def parse():
     ap.add_argument("--no-navigable", action="store_true", help="skip the extra navigable-data variant")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel on 1 GiB x steps (yardstick for rocprofv3 byte counters) and exit")
+    ap.add_argument("--partition-only", type=int, default=0, metavar="C",
+                    help="only time partition assignment of 1M x 128 rows against C centroids (fp32 matrix-core tile) and exit")
     return ap.parse_args()
 
 
@@ -263,6 +265,30 @@ def main():
         ms = e0.elapsed_ms(e1) / args.steps
         print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes, "ms": ms,
                           "GBps_read_plus_write": 2 * nbytes / ms / 1e6}))
+        return
+
+    if args.partition_only:
+        import numpy as np
+        from glide_amd import datasets as D
+        num, dim, c = 1_000_000, 128, args.partition_only
+        data = D.gmm_clipped(num, dim, seed=1234)
+        d_data = capi.DeviceArray.from_numpy(data)
+        d_cent = capi.DeviceArray.from_numpy(data[np.random.default_rng(7).permutation(num)[:c]].copy())
+        d_idx, d_len = capi.DeviceArray((num, 3), np.uint32), capi.DeviceArray(c + 1, np.uint32)
+        wb = capi.partition_assign_workspace_bytes(num, c)
+        ws = capi.DeviceArray(wb // 4 + 1, np.uint32)
+        run = lambda: capi.partition_assign(d_data, num, dim, d_cent, c, 1.04, 0, d_idx, d_len, None, ws, wb)
+        for _ in range(args.warmup):
+            run()
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record()
+        for _ in range(args.steps):
+            run()
+        e1.record()
+        ms = e0.elapsed_ms(e1) / args.steps
+        print(json.dumps({"stage": "partition assign (assign + scan + slot kernels)", "rows": num, "dim": dim, "centroids": c, "ms": ms,
+                          "algorithmic_GBps": (num * dim * 4 + num * 12) / ms / 1e6, "algorithmic_TFLOPs": 2.0 * num * c * dim / ms / 1e9,
+                          "fp32_mfma_peak_TFLOPs": 157.3}))
         return
 
     main_res = run_workload(args, args.workload, torch, want_cpu=not args.no_cpu)

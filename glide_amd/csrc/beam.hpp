@@ -45,12 +45,9 @@ __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float
         RowRegs<DIMV> rows[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
+            // lane groups past the end re-read the last listed row (same cache lines, no branch); their result is dropped
             const uint32_t idx = base + Shape::ROWS * u + g;
-            if (idx < count) {
-                load_row<DIMV>(rows[u], data + static_cast<size_t>(id_of(idx)) * dim, dim, t);
-            } else {
-                rows[u] = ref;
-            }
+            load_row<DIMV>(rows[u], data + static_cast<size_t>(id_of(idx < count ? idx : count - 1)) * dim, dim, t);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
