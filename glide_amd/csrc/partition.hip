@@ -66,26 +66,37 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[cb][r] = 0.f;
 
-    for (uint32_t k0 = 0; k0 < a.dim; k0 += kChunk) {
-        __syncthreads();
-        // centroid chunk: 8 lanes x float4 per row
-        for (uint32_t idx = threadIdx.x; idx < 32u * CB * 8; idx += 256) {
-            const uint32_t row = idx >> 3, q = idx & 7;
-            const uint32_t d0 = k0 + q * 4;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (row < a.centroid_num && d0 < a.dim) v = *reinterpret_cast<const float4*>(a.centroids + static_cast<size_t>(row) * a.dim + d0);
-            *reinterpret_cast<float4*>(cent_tile + row * kLdsStride + q * 4) = v;
-        }
-        // this wave's 32 points
+    // Chunks of kChunk dims go global -> registers -> LDS; the loads of chunk k+1 are issued before the matrix
+    // instructions of chunk k, so their latency is covered by the MFMA work.
+    float4 cpre[CB], xpre[4];
+    auto prefetch = [&](uint32_t k0) {
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const uint32_t row = it * 8 + (lane >> 3), q = lane & 7;
-            const uint32_t p = wave_base + row, d0 = k0 + q * 4;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (p < a.num && d0 < a.dim) v = *reinterpret_cast<const float4*>(a.data + static_cast<size_t>(p) * a.dim + d0);
-            *reinterpret_cast<float4*>(xw + row * kLdsStride + q * 4) = v;
+        for (int it = 0; it < CB; it++) {   // centroid chunk: 8 lanes x float4 per row, 32*CB rows over 256 threads
+            const uint32_t idx = threadIdx.x + 256 * it;
+            const uint32_t row = idx >> 3, d0 = k0 + (idx & 7) * 4;
+            cpre[it] = (row < a.centroid_num && d0 < a.dim) ? *reinterpret_cast<const float4*>(a.centroids + static_cast<size_t>(row) * a.dim + d0)
+                                                           : make_float4(0.f, 0.f, 0.f, 0.f);
         }
+#pragma unroll
+        for (int it = 0; it < 4; it++) {    // this wave's 32 points
+            const uint32_t row = it * 8 + (lane >> 3);
+            const uint32_t p = wave_base + row, d0 = k0 + (lane & 7) * 4;
+            xpre[it] = (p < a.num && d0 < a.dim) ? *reinterpret_cast<const float4*>(a.data + static_cast<size_t>(p) * a.dim + d0)
+                                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    prefetch(0);
+    for (uint32_t k0 = 0; k0 < a.dim; k0 += kChunk) {
+        __syncthreads();   // every wave is done with the previous chunk
+#pragma unroll
+        for (int it = 0; it < CB; it++) {
+            const uint32_t idx = threadIdx.x + 256 * it;
+            *reinterpret_cast<float4*>(cent_tile + (idx >> 3) * kLdsStride + (idx & 7) * 4) = cpre[it];
+        }
+#pragma unroll
+        for (int it = 0; it < 4; it++) *reinterpret_cast<float4*>(xw + (it * 8 + (lane >> 3)) * kLdsStride + (lane & 7) * 4) = xpre[it];
         __syncthreads();
+        if (k0 + kChunk < a.dim) prefetch(k0 + kChunk);
         // v_mfma_f32_32x32x2_f32: lane supplies A[i = lane%32][k-slot = lane/32] and B[k-slot][j = lane%32].
         // A k-slot pair is fed from one float4 per half (dims kk+4*half .. +3), component by component.
 #pragma unroll
@@ -102,8 +113,9 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
         }
     }
 
-    // ranking epilogue: score = ||c||^2 - 2 x.c (the ||x||^2 term is constant per point); lane i < 32 keeps the
-    // kTop smallest scores of point i
+    // ranking epilogue: score = ||c||^2 - 2 x.c (the ||x||^2 term is constant per point).  Lane (i = lane % 32,
+    // half) keeps the kTop smallest scores of point i over its half of every 32-column block; the halves are merged
+    // afterwards, so both lanes of a point end with the same kTop candidates.
     float best_s[kTop];
     uint32_t best_c[kTop];
 #pragma unroll
@@ -111,6 +123,19 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
         best_s[k] = FLT_MAX;
         best_c[k] = kInvalid;
     }
+    auto offer = [&](float s, uint32_t c) {
+#pragma unroll
+        for (int k = 0; k < kTop; k++) {
+            if (s < best_s[k]) {
+                const float ts = best_s[k];
+                const uint32_t tc = best_c[k];
+                best_s[k] = s;
+                best_c[k] = c;
+                s = ts;
+                c = tc;
+            }
+        }
+    };
 #pragma unroll
     for (int cb = 0; cb < CB; cb++) {
         const uint32_t j = cb * 32 + t;
@@ -121,62 +146,80 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
             sw[i * 33 + t] = j < a.centroid_num ? cn - 2.f * acc[cb][r] : FLT_MAX;
         }
         __syncthreads();
-        if (lane < 32) {
-            for (int jj = 0; jj < 32; jj++) {
-                float s = sw[lane * 33 + jj];
-                uint32_t c = cb * 32 + jj;
-#pragma unroll
-                for (int k = 0; k < kTop; k++) {
-                    if (s < best_s[k]) {
-                        const float ts = best_s[k];
-                        const uint32_t tc = best_c[k];
-                        best_s[k] = s;
-                        best_c[k] = c;
-                        s = ts;
-                        c = tc;
-                    }
-                }
-            }
-        }
+#pragma unroll 4
+        for (int jj = 0; jj < 16; jj++) offer(sw[t * 33 + half * 16 + jj], cb * 32 + half * 16 + jj);
         __syncthreads();
     }
-
-    // exact rescoring of the kept candidates; lanes 0..31 own the points, halves do the row pairs
-    float d0 = FLT_MAX, d1 = FLT_MAX;
-    uint32_t c0 = kInvalid, c1 = kInvalid;
-    for (int i = 0; i < 32; i++) {
-        const uint32_t p = wave_base + i;
-        if (p >= a.num) break;   // wave-uniform
-        const float* x = a.data + static_cast<size_t>(p) * a.dim;
-        float dd[kTop];
-        uint32_t cc[kTop];
-#pragma unroll
-        for (int k = 0; k < kTop; k += 2) {
-            const uint32_t ca = read_lane(best_c[k], i), cb2 = read_lane(best_c[k + 1], i);
-            const uint32_t mine = half ? cb2 : ca;
-            const float sq = exact_distance_half(x, a.centroids + static_cast<size_t>(mine != kInvalid ? mine : 0u) * a.dim, a.dim, t);
-            const float da = read_lane(sq, 0), db = read_lane(sq, 32);
-            dd[k] = ca != kInvalid ? finish_distance(da, a.metric) : FLT_MAX;
-            dd[k + 1] = cb2 != kInvalid ? finish_distance(db, a.metric) : FLT_MAX;
-            cc[k] = ca;
-            cc[k + 1] = cb2;
-        }
-        // smallest two by (distance, centroid id)
-        float m0 = FLT_MAX, m1 = FLT_MAX;
-        uint32_t i0 = kInvalid, i1 = kInvalid;
+    {
+        float os[kTop];
+        uint32_t oc[kTop];
 #pragma unroll
         for (int k = 0; k < kTop; k++) {
-            const bool lt0 = dd[k] < m0 || (dd[k] == m0 && cc[k] < i0);
-            const bool lt1 = dd[k] < m1 || (dd[k] == m1 && cc[k] < i1);
-            if (lt0) {
-                m1 = m0; i1 = i0;
-                m0 = dd[k]; i0 = cc[k];
-            } else if (lt1) {
-                m1 = dd[k]; i1 = cc[k];
+            os[k] = lane_xor<32>(best_s[k]);
+            oc[k] = lane_xor<32>(best_c[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < kTop; k++) offer(os[k], oc[k]);
+    }
+
+    // exact rescoring of the kept candidates: 32 points x kTop pairs per wavefront, one pair per group of 8 lanes,
+    // four steps (32 pairs) in flight.  Candidates and distances are exchanged through this wave's score tile.
+    uint32_t* cand = reinterpret_cast<uint32_t*>(sw);          // [32][kTop]
+    float* exact = sw + 32 * kTop;                             // [32][kTop]
+    if (half == 0) {
+#pragma unroll
+        for (int k = 0; k < kTop; k++) cand[t * kTop + k] = best_c[k];
+    }
+    __syncthreads();
+    {
+        const int g = lane >> 3, t8 = lane & 7;
+        const uint32_t last = a.num - 1;
+        for (int s0 = 0; s0 < 32 * kTop / 8; s0 += 4) {
+            const float* xr[4];
+            const float* cr[4];
+            uint32_t cid[4];
+            float part[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int pair = (s0 + u) * 8 + g;
+                const uint32_t pt = wave_base + (pair / kTop);
+                cid[u] = cand[pair];
+                xr[u] = a.data + static_cast<size_t>(pt < a.num ? pt : last) * a.dim;
+                cr[u] = a.centroids + static_cast<size_t>(cid[u] != kInvalid ? cid[u] : 0u) * a.dim;
+                part[u] = 0.f;
+            }
+            for (uint32_t d0 = t8 * 4; d0 < a.dim; d0 += 32) {
+                float4 xv[4], cv[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    xv[u] = *reinterpret_cast<const float4*>(xr[u] + d0);
+                    cv[u] = *reinterpret_cast<const float4*>(cr[u] + d0);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) part[u] = sqdist4(xv[u], cv[u], part[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const float sq = row_sum<1>(part[u]);   // 8-lane groups
+                if (t8 == 0) exact[(s0 + u) * 8 + g] = cid[u] != kInvalid ? finish_distance(sq, a.metric) : FLT_MAX;
             }
         }
-        if (lane == i) {
-            d0 = m0; d1 = m1; c0 = i0; c1 = i1;
+    }
+    __syncthreads();
+    // smallest two by (distance, centroid id); lane i < 32 owns point i
+    float d0 = FLT_MAX, d1 = FLT_MAX;
+    uint32_t c0 = kInvalid, c1 = kInvalid;
+#pragma unroll
+    for (int k = 0; k < kTop; k++) {
+        const float dk = exact[t * kTop + k];
+        const uint32_t ck = cand[t * kTop + k];
+        const bool lt0 = dk < d0 || (dk == d0 && ck < c0);
+        const bool lt1 = dk < d1 || (dk == d1 && ck < c1);
+        if (lt0) {
+            d1 = d0; c1 = c0;
+            d0 = dk; c0 = ck;
+        } else if (lt1) {
+            d1 = dk; c1 = ck;
         }
     }
     (void) c1;
