@@ -283,17 +283,17 @@ def nnd_workspace_bytes(reorder_num, dim, knn_degree):
 
 
 def nnd_build(reorder_data, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, iterations,
-              seed, knn_graph, workspace, workspace_bytes, stats=None, stream=None):
+              termination_threshold, seed, knn_graph, workspace, workspace_bytes, stats=None, stream=None):
     check(lib().glide_hip_nnd_build(_ptr(reorder_data), u32(reorder_num), u32(dim), _ptr(segment_starts),
                                     _ptr(segment_lengths), u32(segment_num), u32(knn_degree), u32(iterations),
-                                    u32(seed), _ptr(knn_graph), _ptr(workspace), C.c_size_t(workspace_bytes),
-                                    _ptr(stats), vp(stream)), "glide_hip_nnd_build")
+                                    f32(termination_threshold), u32(seed), _ptr(knn_graph), _ptr(workspace),
+                                    C.c_size_t(workspace_bytes), _ptr(stats), vp(stream)), "glide_hip_nnd_build")
 
 
 class NndLayout(C.Structure):
     """glide_nnd_layout: byte offsets of the NN-descent arrays inside the workspace."""
     _fields_ = [(n, C.c_uint64) for n in ("half_rows", "norms", "list_ids", "list_dists", "fwd_new", "fwd_old", "rev_new", "rev_old",
-                                          "counts", "inbox_counts", "inbox", "bloom", "total")] + \
+                                          "counts", "inbox_counts", "inbox", "bloom", "segment_state", "segment_updates", "total")] + \
                [(n, C.c_uint32) for n in ("width", "inbox_cap", "row_halfs", "bloom_sets")]
 
 
@@ -325,6 +325,13 @@ def nnd_local_join(*args, stream=None):
 
 def nnd_merge(*args, stream=None):
     _nnd_stage("glide_hip_nnd_merge", *args, stream)
+
+
+def nnd_converge(reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, termination_threshold, workspace,
+                 workspace_bytes, stream=None):
+    check(lib().glide_hip_nnd_converge(u32(reorder_num), u32(dim), _ptr(segment_starts), _ptr(segment_lengths), u32(segment_num),
+                                       u32(knn_degree), f32(termination_threshold), _ptr(workspace), C.c_size_t(workspace_bytes),
+                                       vp(stream)), "glide_hip_nnd_converge")
 
 
 def nnd_finalize(reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, knn_graph, stats, workspace,

@@ -30,7 +30,12 @@ struct Segments {
     const uint32_t* starts;
     const uint32_t* lengths;
     uint32_t count;
+    uint32_t* state;     // per partition: kActive, kLastRound (one more join, as the reference's overlapped loop does), kDone
+    uint32_t* updates;   // per partition: list insertions seen on every 100th row in the current round
 };
+constexpr uint32_t kActive = 0, kLastRound = 1, kDone = 2;
+constexpr uint32_t kMaxSegments = 2048;
+constexpr uint32_t kCounterInterval = 100;   // counter_interval, nn_descent.cuh:1123
 
 __device__ __forceinline__ void locate(const Segments& s, uint32_t node, uint32_t& start, uint32_t& len) {
     uint32_t i = 0;
@@ -41,8 +46,8 @@ __device__ __forceinline__ void locate(const Segments& s, uint32_t node, uint32_
 }
 
 // Same result for a node every lane of the wavefront shares: the lanes test one segment each, so the lookup costs
-// one memory round trip instead of one per segment.  Every lane of the wavefront must call it.
-__device__ __forceinline__ void locate_uniform(const Segments& s, uint32_t node, uint32_t& start, uint32_t& len) {
+// one memory round trip instead of one per segment.  Every lane of the wavefront must call it.  Returns the index.
+__device__ __forceinline__ uint32_t locate_uniform(const Segments& s, uint32_t node, uint32_t& start, uint32_t& len) {
     uint32_t found = s.count - 1;
     for (uint32_t base = 0; base + 1 < s.count; base += 64) {
         const uint32_t i = base + lane_id();
@@ -55,6 +60,7 @@ __device__ __forceinline__ void locate_uniform(const Segments& s, uint32_t node,
     }
     start = s.starts[found];
     len = s.lengths[found];
+    return found;
 }
 
 // ---- prepare: fp32 rows -> fp16 rows (stride dim_pad, zero padded) + squared norms of the fp32 input
@@ -167,7 +173,8 @@ __global__ __launch_bounds__(256) void nnd_reverse_kernel(const uint32_t* fwd_ne
     const uint32_t node = idx / 64, j = idx % 64;
     if (node >= num) return;
     uint32_t start, len;
-    locate_uniform(segs, node, start, len);
+    const uint32_t seg = locate_uniform(segs, node, start, len);
+    if (segs.state[seg] == kDone) return;
     const uint32_t which = j / kSamples, k = j % kSamples;   // 0: new, 1: old
     if (k >= counts[static_cast<size_t>(node) * 4 + which]) return;
     const uint32_t v = (which ? fwd_old : fwd_new)[static_cast<size_t>(node) * kSamples + k];
@@ -284,7 +291,8 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
     }
     const uint4 c4 = *reinterpret_cast<const uint4*>(a.counts + static_cast<size_t>(node) * 4);
     uint32_t seg_start, seg_len;
-    locate_uniform(a.segs, node, seg_start, seg_len);
+    const uint32_t seg = locate_uniform(a.segs, node, seg_start, seg_len);
+    if (a.segs.state[seg] == kDone) return;
     const uint32_t c_fn = c4.x, c_fo = c4.y;
     const uint32_t c_rn = c4.z < kSamples ? c4.z : kSamples, c_ro = c4.w < kSamples ? c4.w : kSamples;
     if (c_fn + c_rn == 0) return;
@@ -496,13 +504,16 @@ __device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane
 template <int M>
 __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t num,
                                                         uint32_t width, uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new,
-                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats) {
+                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats, Segments segs) {
     constexpr int NR = M / 64;
     __shared__ uint32_t filter_lds[4][64];
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (node >= num) return;
+    uint32_t seg_start, seg_len;
+    const uint32_t seg = locate_uniform(segs, node, seg_start, seg_len);
+    if (segs.state[seg] == kDone) return;
     uint32_t* filter = filter_lds[wave];
     const uint32_t bloom_words = bloom_sets * 16;
     if (static_cast<uint32_t>(lane) < bloom_words) filter[lane] = bloom[static_cast<size_t>(node) * bloom_words + lane];
@@ -589,6 +600,7 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
     uint32_t pos = wave_exclusive_scan(keep_count, lane, total_keep);
     uint32_t nrank = wave_exclusive_scan(fresh_count, lane, total_new);
     __builtin_amdgcn_wave_barrier();
+    uint32_t inserted = 0;
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
@@ -612,9 +624,16 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
             if (pos < width) {
                 list_ids[static_cast<size_t>(node) * width + pos] = id | flag;
                 list_dists[static_cast<size_t>(node) * width + pos] = __uint_as_float(static_cast<uint32_t>(k[r] >> 32));
+                inserted += first_offer[r];
             }
             pos++;
         }
+    }
+    // update_counter (update_graph :1106-1126): insertions on every 100th row, per partition
+    if (node % kCounterInterval == 0) {
+        uint32_t total_inserted;
+        wave_exclusive_scan(inserted, lane, total_inserted);
+        if (lane == 0 && total_inserted) atomicAdd(&segs.updates[seg], total_inserted);
     }
     for (uint32_t e = total_keep + lane; e < width; e += 64) {
         list_ids[static_cast<size_t>(node) * width + e] = kInvalid;
@@ -634,6 +653,21 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
             if (raw > inbox_cap) atomicAdd(&slot[1], static_cast<unsigned long long>(raw - inbox_cap));
         }
     }
+}
+
+// Termination test of GNND::build's update_and_sample (nn_descent.cuh:1270-1284): a partition whose sampled update
+// count falls below termination_threshold * rows * dim / 100 (rows = all rows of the build, as in the reference) runs
+// one more round -- the reference has already started that round's join when the host notices -- and then rests.
+__global__ void nnd_converge_kernel(Segments segs, float limit) {
+    const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
+    if (s >= segs.count) return;
+    const uint32_t state = segs.state[s];
+    if (state == kLastRound) {
+        segs.state[s] = kDone;
+    } else if (state == kActive && static_cast<float>(segs.updates[s]) < limit) {
+        segs.state[s] = kLastRound;
+    }
+    segs.updates[s] = 0;
 }
 
 // ---- finalize (shrink step :1376-1402): first `degree` ids of each list; unfilled slots get a pseudo-random id
@@ -684,7 +718,7 @@ uint32_t nnd_inbox_cap(uint32_t width) { return (getenv("GLIDE_EXP_CAP512") ? 51
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
 struct NndLayout {
-    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, counts, inbox_counts, inbox, bloom, stats, total;
+    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, counts, inbox_counts, inbox, bloom, stats, seg_state, seg_updates, total;
     uint32_t width, cap, dim_pad, bloom_sets;
 };
 NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
@@ -709,6 +743,8 @@ NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
     l.inbox = take(n * l.cap * 8);
     l.bloom = take(n * l.bloom_sets * 64);
     l.stats = take(1024 * 16);
+    l.seg_state = take(kMaxSegments * 4);
+    l.seg_updates = take(kMaxSegments * 4);
     l.total = off;
     return l;
 }
@@ -740,6 +776,7 @@ int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* s
                 uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
     if (!segment_starts || !segment_lengths || !workspace) return GLIDE_ERR_BAD_ARGUMENT;
     if (dim == 0 || segment_num == 0 || knn_degree == 0 || reorder_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (segment_num > kMaxSegments) return GLIDE_ERR_UNSUPPORTED;
     if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // also keeps the Bloom filter within 64 words
     c.l = nnd_layout(reorder_num, dim, knn_degree);
     if (c.l.bloom_sets > 4) return GLIDE_ERR_UNSUPPORTED;
@@ -758,7 +795,8 @@ int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* s
     c.inbox = reinterpret_cast<uint2*>(w + c.l.inbox);
     c.bloom = reinterpret_cast<uint32_t*>(w + c.l.bloom);
     c.stats = reinterpret_cast<unsigned long long*>(w + c.l.stats);
-    c.segs = Segments{segment_starts, segment_lengths, segment_num};
+    c.segs = Segments{segment_starts, segment_lengths, segment_num, reinterpret_cast<uint32_t*>(w + c.l.seg_state),
+                      reinterpret_cast<uint32_t*>(w + c.l.seg_updates)};
     c.n = reorder_num;
     c.s = as_stream(stream);
     return GLIDE_OK;
@@ -768,6 +806,8 @@ int nnd_prepare(const NndCtx& c, const float* data, uint32_t dim, uint32_t seed)
     int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(c.stats), 0u, 1024 * 4, c.s);
     if (rc != GLIDE_OK) return rc;
     rc = glide_hip_fill_u32(c.bloom, 0u, static_cast<size_t>(c.n) * c.l.bloom_sets * 16, c.s);
+    if (rc != GLIDE_OK) return rc;
+    rc = glide_hip_fill_u32(c.segs.state, 0u, 2 * kMaxSegments, c.s);   // state and updates are adjacent
     if (rc != GLIDE_OK) return rc;
     hipLaunchKernelGGL(nnd_prepare_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, data, c.n, dim, c.l.dim_pad, c.half_rows, c.norms);
     hipLaunchKernelGGL(nnd_init_kernel, dim3(ceil_div(c.n * c.l.width, 256)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.n,
@@ -797,11 +837,18 @@ int nnd_merge(const NndCtx& c, bool with_stats) {
     const uint32_t m = c.l.width + c.l.cap;
     if (m <= 128) {
         hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
-                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats);
+                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs);
     } else {
         hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
-                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats);
+                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs);
     }
+    return launch_status();
+}
+
+int nnd_converge(const NndCtx& c, uint32_t dim, float termination_threshold) {
+    // update_counter < termination_threshold * nrow * dim / counter_interval (nn_descent.cuh:1280), evaluated in float
+    const float limit = termination_threshold * static_cast<float>(c.n) * static_cast<float>(dim) / static_cast<float>(kCounterInterval);
+    hipLaunchKernelGGL(nnd_converge_kernel, dim3(ceil_div(c.segs.count, 256)), dim3(256), 0, c.s, c.segs, limit);
     return launch_status();
 }
 
@@ -814,9 +861,10 @@ int nnd_finalize(const NndCtx& c, uint32_t knn_degree, uint32_t* knn_graph, unsi
 }  // namespace
 
 int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts,
-                        const uint32_t* segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations, uint32_t seed,
-                        uint32_t* knn_graph, void* workspace, size_t workspace_bytes, unsigned long long* stats_out, void* stream) {
-    if (!reorder_data || !knn_graph) return GLIDE_ERR_BAD_ARGUMENT;
+                        const uint32_t* segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
+                        float termination_threshold, uint32_t seed, uint32_t* knn_graph, void* workspace, size_t workspace_bytes,
+                        unsigned long long* stats_out, void* stream) {
+    if (!reorder_data || !knn_graph || !(termination_threshold >= 0.f)) return GLIDE_ERR_BAD_ARGUMENT;
     if (reorder_num == 0 && segment_starts && segment_lengths && workspace && dim && segment_num && knn_degree) return GLIDE_OK;
     NndCtx c;
     int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
@@ -826,6 +874,7 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
         if ((rc = nnd_reverse(c)) != GLIDE_OK) return rc;
         if ((rc = nnd_join(c)) != GLIDE_OK) return rc;
         if ((rc = nnd_merge(c, stats_out != nullptr)) != GLIDE_OK) return rc;
+        if ((rc = nnd_converge(c, dim, termination_threshold)) != GLIDE_OK) return rc;
     }
     return nnd_finalize(c, knn_degree, knn_graph, stats_out);
 }
@@ -836,7 +885,8 @@ int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree
     const NndLayout l = nnd_layout(reorder_num, dim, knn_degree);
     out->half_rows = l.half_rows; out->norms = l.norms; out->list_ids = l.list_ids; out->list_dists = l.list_dists;
     out->fwd_new = l.fwd_new; out->fwd_old = l.fwd_old; out->rev_new = l.rev_new; out->rev_old = l.rev_old;
-    out->counts = l.counts; out->inbox_counts = l.inbox_counts; out->inbox = l.inbox; out->bloom = l.bloom; out->total = l.total;
+    out->counts = l.counts; out->inbox_counts = l.inbox_counts; out->inbox = l.inbox; out->bloom = l.bloom;
+    out->segment_state = l.seg_state; out->segment_updates = l.seg_updates; out->total = l.total;
     out->width = l.width; out->inbox_cap = l.cap; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
     return GLIDE_OK;
 }
@@ -869,6 +919,15 @@ int glide_hip_nnd_merge(uint32_t reorder_num, uint32_t dim, const uint32_t* segm
     NndCtx c;
     int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
     return rc != GLIDE_OK ? rc : nnd_merge(c, true);
+}
+
+int glide_hip_nnd_converge(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
+                           uint32_t segment_num, uint32_t knn_degree, float termination_threshold, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+    if (!(termination_threshold >= 0.f)) return GLIDE_ERR_BAD_ARGUMENT;
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    return rc != GLIDE_OK ? rc : nnd_converge(c, dim, termination_threshold);
 }
 
 int glide_hip_nnd_finalize(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,

@@ -28,7 +28,8 @@ host_matrix<int> build_nnd(device_resources& handle, NNDescentParameter& param, 
     gpu_timer timer;
     timer.start();
     hip_try(glide_hip_nnd_build(d_data->data_handle(), num, dim, d_start.data_handle(), d_length.data_handle(), segment_num, graph_degree,
-                                param.max_iterations, param.seed, d_knn.data_handle(), ws.get(), wb, nullptr, handle.stream()),
+                                param.max_iterations, param.termination_threshold, param.seed, d_knn.data_handle(), ws.get(), wb, nullptr,
+                                handle.stream()),
             "glide_hip_nnd_build");
     const float build_time = timer.stop();
     d_data.reset();   // the reference consumes the input matrix (nn_descent.cuh:1257)
@@ -52,7 +53,8 @@ namespace glide {
 template <typename Data_t>
 pinned_matrix<int> build_knn_for_large(device_resources& handle, uint32_t knn_degree, host_vector_view<uint32_t> h_segment_start_view,
                                        host_vector_view<uint32_t> h_segment_length_view, const pinned_matrix<Data_t>& h_reorder_data,
-                                       std::string& result_file, uint32_t iterations = 20, uint32_t seed = 0) {
+                                       std::string& result_file, uint32_t iterations = 20, uint32_t seed = 0,
+                                       float termination_threshold = 0.0001f) {
     (void) handle;
     const uint32_t segments = h_segment_start_view.size(), dim = h_reorder_data.extent(1);
     const size_t num = h_reorder_data.extent(0);
@@ -88,7 +90,8 @@ pinned_matrix<int> build_knn_for_large(device_resources& handle, uint32_t knn_de
         if (s + 1 < segments) stage(s + 1);
         st.before_compute(b);
         hip_try(glide_hip_nnd_build(d_data[b].data_handle(), len, dim, d_seg.data_handle() + 2 * s, d_seg.data_handle() + 2 * s + 1, 1, knn_degree,
-                                    iterations, seed + s, d_knn[b].data_handle(), ws.get(), wb, nullptr, st.compute_stream()),
+                                    iterations, termination_threshold, seed + s, d_knn[b].data_handle(), ws.get(), wb, nullptr,
+                                    st.compute_stream()),
                 "glide_hip_nnd_build");
         hip_try(glide_hip_memcpy_d2h_async(knn_graph.row(h_segment_start_view(s)), d_knn[b].data_handle(),
                                            static_cast<size_t>(len) * knn_degree * sizeof(uint32_t), st.compute_stream()),

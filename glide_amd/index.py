@@ -199,7 +199,8 @@ def build_nnd(param, d_reorder_data, h_segment_start, h_segment_length, result=N
     ws = capi.DeviceArray(wb // 16 + 1, np.dtype("V16"))
     d_stats = capi.DeviceArray.from_numpy(np.zeros(2, np.uint64)) if stats else None
     with _Timer() as t:
-        capi.nnd_build(d_reorder_data, num, dim, d_ss, d_sl, len(h_segment_start), degree, param.max_iterations, param.seed,
+        capi.nnd_build(d_reorder_data, num, dim, d_ss, d_sl, len(h_segment_start), degree, param.max_iterations,
+                       param.termination_threshold, param.seed,
                        d_knn, ws, wb, d_stats)
     ws.free()
     if result is not None:

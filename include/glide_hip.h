@@ -117,13 +117,17 @@ int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim,
  * partition-local ids: knn_graph is reorder_num x knn_degree, nearest first.  `iterations` rounds of
  * sample -> reverse sample -> local join (64 x 64 fp16 matrix-core tiles, fp32 accumulate, norm-trick
  * epilogue, one offer per row/column) -> merge are run; lists, flags and samples stay in `workspace`.
+ * termination_threshold (NNDescentParameter::termination_threshold, params.cuh:21; 0 disables): a partition whose
+ * list insertions on every 100th row fall below termination_threshold * reorder_num * dim / 100 in a round
+ * (nn_descent.cuh:1123,1280) runs one more round and is then left alone.  At most 2048 partitions.
  * stats_out (nullable, 2 device u64): offers received by the merge step, offers dropped by a full inbox.
  * Limits: knn_degree <= 65 (list width round_up32(1.3 * knn_degree) <= 96, Bloom filter <= 2048 bits), dim % 4 == 0. */
 size_t glide_hip_nnd_workspace_bytes(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree);
 int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim,
                         const uint32_t *segment_starts, const uint32_t *segment_lengths, uint32_t segment_num,
-                        uint32_t knn_degree, uint32_t iterations, uint32_t seed, uint32_t *knn_graph,
-                        void *workspace, size_t workspace_bytes, unsigned long long *stats_out, void *stream);
+                        uint32_t knn_degree, uint32_t iterations, float termination_threshold, uint32_t seed,
+                        uint32_t *knn_graph, void *workspace, size_t workspace_bytes, unsigned long long *stats_out,
+                        void *stream);
 
 /* The same build one stage per call, on the same workspace (the stages of GNND::build's loop, nn_descent.cuh:1289-1368):
  *   prepare         preprocess_data_kernel :445 (fp16 rows + fp32 squared norms), init_random_graph :1003,
@@ -131,8 +135,9 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *   reverse_sample  add_rev_edges_kernel :490-507
  *   local_join      local_join_kernel :668-914; offers go to the per-node inbox instead of a spin-locked list
  *   merge           update_graph :1106-1126 + sample_graph_new :973-1001 + sample_segment_graph :1073-1104
+ *   converge        the termination test of update_and_sample :1270-1284 (marks partitions that rest from now on)
  *   finalize        the shrink step :1376-1402
- * glide_hip_nnd_build = prepare, `iterations` x (reverse_sample, local_join, merge), finalize.
+ * glide_hip_nnd_build = prepare, `iterations` x (reverse_sample, local_join, merge, converge), finalize.
  * glide_hip_nnd_layout reports where each array lives in the workspace (byte offsets), so a caller or a test can
  * inspect or replace any of them between stages:
  *   list_ids   num x width u32: partition-local id | 0x80000000 ("already sampled"), 0xffffffff = empty; nearest first
@@ -140,9 +145,11 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *   fwd_new / fwd_old / rev_new / rev_old  num x 32 u32 sample lists; counts num x 4 u32 = their lengths
  *                   (reverse lengths count every arrival and may exceed 32; 32 are stored)
  *   inbox      num x inbox_cap x (u32 distance bits, u32 id); inbox_counts num u32 (arrivals, may exceed inbox_cap)
- *   bloom      num x bloom_sets x 512 bits */
+ *   bloom      num x bloom_sets x 512 bits
+ *   segment_state   u32 per partition: 0 active, 1 last round, 2 resting;  segment_updates  u32 per partition */
 typedef struct {
-    uint64_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, counts, inbox_counts, inbox, bloom, total;
+    uint64_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, counts, inbox_counts, inbox, bloom,
+        segment_state, segment_updates, total;
     uint32_t width, inbox_cap, row_halfs, bloom_sets;
 } glide_nnd_layout;
 int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree, glide_nnd_layout *out);
@@ -158,6 +165,9 @@ int glide_hip_nnd_local_join(uint32_t reorder_num, uint32_t dim, const uint32_t 
 int glide_hip_nnd_merge(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
                         const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
                         void *workspace, size_t workspace_bytes, void *stream);
+int glide_hip_nnd_converge(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                           const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
+                           float termination_threshold, void *workspace, size_t workspace_bytes, void *stream);
 int glide_hip_nnd_finalize(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
                            const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
                            uint32_t *knn_graph, unsigned long long *stats_out, void *workspace, size_t workspace_bytes,

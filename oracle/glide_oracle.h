@@ -139,6 +139,11 @@ int go_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim, 
                  const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
                  uint32_t iterations, uint32_t seed, int32_t *knn_graph, int threads);
 
+/* the same with NNDescentParameter::termination_threshold (params.cuh:21; update counter nn_descent.cuh:1123,1270-1284) */
+int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                    const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
+                    float termination_threshold, uint32_t seed, int32_t *knn_graph, int threads);
+
 /* exact kNN by brute force (ties by smaller id); squared L2 ranking, reported per metric */
 void go_bruteforce_knn(const float *data, uint32_t num, uint32_t dim, const float *queries, uint32_t query_num,
                        uint32_t k, int metric, int exclude_self, uint32_t *ids, float *dists, int threads);

@@ -1,7 +1,8 @@
 // CPU oracle, NN-descent part.  TEST INFRASTRUCTURE ONLY -- see glide_oracle.h.
 //
 // Restates the reference's per-partition NN-descent (nn_descent.cuh) as the *intended* algorithm:
-// every partition is updated in every iteration and the iteration count is fixed.  The reference's
+// every partition is updated in every iteration until max_iterations or until its own update counter falls below the
+// termination limit (go_nnd_build_ex; go_nnd_build runs the fixed count).  The reference's
 // own host loop stops updating partitions >= 1 after two rounds (it passes a length where an end is
 // expected, nn_descent.cuh:1276-1279 vs :1129-1135); that behaviour is not reproduced.
 // Bit-level parity is unpinned (the reference is unseeded and racy); tests check graph recall.
@@ -236,9 +237,11 @@ void local_join(Partition &P, uint32_t L, std::vector<float> &xn, std::vector<fl
     }
 }
 
-// update_graph nn_descent.cuh:1106-1126
-void update_lists(Partition &P, const std::vector<int> &src_ids, const std::vector<float> &src_dists) {
-#pragma omp parallel for schedule(static)
+// update_graph nn_descent.cuh:1106-1126; returns the update counter: insertions on rows whose index in the whole
+// build (row_index_base + i) is a multiple of counter_interval = 100 (:1123)
+int64_t update_lists(Partition &P, const std::vector<int> &src_ids, const std::vector<float> &src_dists, uint32_t row_index_base) {
+    int64_t counter = 0;
+#pragma omp parallel for schedule(static) reduction(+ : counter)
     for (int64_t i = 0; i < static_cast<int64_t>(P.n); i++) {
         for (uint32_t j = 0; j < kSeg; j++) {
             int nid = src_ids[static_cast<size_t>(i) * kSeg + j];
@@ -246,14 +249,16 @@ void update_lists(Partition &P, const std::vector<int> &src_ids, const std::vect
             if (d == FLT_MAX) break;
             if (static_cast<uint32_t>(id_of(nid)) == static_cast<uint32_t>(i)) continue;
             uint32_t sub = static_cast<uint32_t>(id_of(nid)) % P.num_sub;
-            insert_ordered(P.lists.data() + static_cast<size_t>(i) * P.W + sub * kSeg,
-                           P.ldists.data() + static_cast<size_t>(i) * P.W + sub * kSeg, kSeg, nid, d);
+            uint32_t pos = insert_ordered(P.lists.data() + static_cast<size_t>(i) * P.W + sub * kSeg,
+                                          P.ldists.data() + static_cast<size_t>(i) * P.W + sub * kSeg, kSeg, nid, d);
+            if ((row_index_base + static_cast<uint32_t>(i)) % 100u == 0 && pos != kSeg) counter++;
         }
     }
+    return counter;
 }
 
 void build_partition(const float *data, const float *norms_in, uint32_t n, uint32_t dim, uint32_t K, uint32_t iterations, uint32_t seed,
-                     int32_t *out /* n x K local ids */, uint32_t row_index_base) {
+                     int32_t *out /* n x K local ids */, uint32_t row_index_base, float termination_limit) {
     Partition P;
     P.n = n;
     P.dim = dim;
@@ -297,10 +302,16 @@ void build_partition(const float *data, const float *norms_in, uint32_t n, uint3
     std::vector<int> host_ids(static_cast<size_t>(n) * kSeg, INT_MAX), cur_old(static_cast<size_t>(n) * kSamples);
     std::vector<float> host_dists(static_cast<size_t>(n) * kSeg, FLT_MAX);
     std::vector<uint32_t> n_cur_old(n);
-    for (uint32_t it = 0; it < iterations; it++) {
+    // Termination (update_and_sample :1270-1284, loop :1305-1308): when the counter of a merge falls below the limit the
+    // partition is marked; the join of that iteration is already running and still completes, later iterations skip it.
+    bool converged = false;
+    for (uint32_t it = 0; it < iterations && !converged; it++) {
         cur_old = P.fwd_old;            // upload of h_graph_old / list sizes (:1290-1302)
         n_cur_old = P.n_fwd_old;
-        if (it > 0) update_lists(P, host_ids, host_dists);   // update_and_sample (:1270-1284)
+        if (it > 0) {                   // update_and_sample (:1270-1284)
+            const int64_t counter = update_lists(P, host_ids, host_dists, row_index_base);
+            if (static_cast<float>(counter) < termination_limit) converged = true;
+        }
         sample_lists(P, false);
         std::vector<int> next_old = P.fwd_old;
         std::vector<uint32_t> n_next_old = P.n_fwd_old;
@@ -335,7 +346,7 @@ void build_partition(const float *data, const float *norms_in, uint32_t n, uint3
             P.n_fwd_new[i] = c;
         }
     }
-    update_lists(P, host_ids, host_dists);  // nn_descent.cuh:1368
+    update_lists(P, host_ids, host_dists, row_index_base);  // nn_descent.cuh:1368
 
     // shrink nn_descent.cuh:1376-1402.  For K > 32 the reference copies whole sub-lists in storage order and
     // therefore never returns ids with id % num_sub == num_sub-1; here sub-lists are merged by distance first.
@@ -358,10 +369,10 @@ void build_partition(const float *data, const float *norms_in, uint32_t n, uint3
 
 }  // namespace
 
-extern "C" int go_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim,
-                            const uint32_t *segment_starts, const uint32_t *segment_lengths, uint32_t segment_num,
-                            uint32_t knn_degree, uint32_t iterations, uint32_t seed, int32_t *knn_graph,
-                            int threads) {
+extern "C" int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, uint32_t dim,
+                               const uint32_t *segment_starts, const uint32_t *segment_lengths, uint32_t segment_num,
+                               uint32_t knn_degree, uint32_t iterations, float termination_threshold, uint32_t seed,
+                               int32_t *knn_graph, int threads) {
 #ifdef _OPENMP
     if (threads > 0) omp_set_num_threads(threads);
 #endif
@@ -382,8 +393,18 @@ extern "C" int go_nnd_build(const float *reorder_data, uint32_t reorder_num, uin
         uint32_t start = segment_starts[s], len = segment_lengths[s];
         if (len == 0) continue;
         if (start + len > reorder_num) return -2;
+        // termination_threshold * nrow * dim / counter_interval with nrow = all rows of the build (nn_descent.cuh:1280)
+        const float limit = termination_threshold * static_cast<float>(reorder_num) * static_cast<float>(dim) / 100.0f;
         build_partition(half.data() + static_cast<size_t>(start) * dim, norms.data() + start, len, dim, knn_degree, iterations, seed,
-                        knn_graph + static_cast<size_t>(start) * knn_degree, start);
+                        knn_graph + static_cast<size_t>(start) * knn_degree, start, limit);
     }
     return 0;
+}
+
+extern "C" int go_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim,
+                            const uint32_t *segment_starts, const uint32_t *segment_lengths, uint32_t segment_num,
+                            uint32_t knn_degree, uint32_t iterations, uint32_t seed, int32_t *knn_graph,
+                            int threads) {
+    return go_nnd_build_ex(reorder_data, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, iterations, 0.0f,
+                           seed, knn_graph, threads);
 }

@@ -14,7 +14,7 @@ def hip():
     return capi
 
 
-def gpu_nnd(hip, rdata, seg_start, seg_len, k, iterations, seed=0):
+def gpu_nnd(hip, rdata, seg_start, seg_len, k, iterations, seed=0, threshold=0.0):
     n, dim = rdata.shape
     d_data = hip.DeviceArray.from_numpy(rdata, np.float32)
     d_ss, d_sl = hip.DeviceArray.from_numpy(seg_start, np.uint32), hip.DeviceArray.from_numpy(seg_len, np.uint32)
@@ -22,7 +22,7 @@ def gpu_nnd(hip, rdata, seg_start, seg_len, k, iterations, seed=0):
     wb = hip.nnd_workspace_bytes(n, dim, k)
     ws = hip.DeviceArray(wb // 16 + 1, np.dtype("V16"))
     stats = hip.DeviceArray.from_numpy(np.zeros(2, np.uint64))
-    hip.nnd_build(d_data, n, dim, d_ss, d_sl, seg_start.size, k, iterations, seed, knn, ws, wb, stats)
+    hip.nnd_build(d_data, n, dim, d_ss, d_sl, seg_start.size, k, iterations, threshold, seed, knn, ws, wb, stats)
     hip.synchronize()
     return knn.numpy(), stats.numpy()
 
@@ -98,11 +98,26 @@ def test_nnd_dim960(hip):
     assert r >= 0.85
 
 
+def test_nnd_termination_threshold(hip):
+    """With the reference's default threshold both sides stop early, at about the same graph recall; the GPU run
+    then costs fewer offers than the fixed-length run."""
+    from oracle import oracle as O
+    rdata = lowdim_data(30000, 128, seed=21)
+    seg_start, seg_len = np.array([0, 18000], np.uint32), np.array([18000, 12000], np.uint32)
+    full, st_full = gpu_nnd(hip, rdata, seg_start, seg_len, 32, 20)
+    early, st_early = gpu_nnd(hip, rdata, seg_start, seg_len, 32, 20, threshold=1e-4)
+    cpu = O.nnd_build(rdata, seg_start, seg_len, 32, 20, 0, termination_threshold=1e-4).astype(np.uint32)
+    r_full, r_early, r_cpu = (partition_recall(k, rdata, seg_start, seg_len, 32) for k in (full, early, cpu))
+    print("graph recall@32: 20 rounds %.4f, with threshold gpu %.4f cpu %.4f; offers %d vs %d" % (r_full, r_early, r_cpu, st_early[0], st_full[0]))
+    assert st_early[0] < 0.8 * st_full[0]
+    assert r_early >= r_cpu - 0.005 and r_early >= 0.98
+
+
 def test_nnd_rejects_unsupported(hip):
     d = hip.DeviceArray(1024, np.float32)
     with pytest.raises(hip.GlideHipError) as e:
-        hip.nnd_build(d, 8, 128, d, d, 1, 100, 1, 0, d, d, 1 << 30)
+        hip.nnd_build(d, 8, 128, d, d, 1, 100, 1, 0.0, 0, d, d, 1 << 30)
     assert e.value.code == -1
     with pytest.raises(hip.GlideHipError) as e:
-        hip.nnd_build(d, 8, 128, d, d, 1, 32, 1, 0, d, d, 16)      # workspace too small
+        hip.nnd_build(d, 8, 128, d, d, 1, 32, 1, 0.0, 0, d, d, 16)      # workspace too small
     assert e.value.code == -2

@@ -41,6 +41,7 @@ class Workspace:
             fwd_new=f(l.fwd_new, n * S).reshape(n, S), fwd_old=f(l.fwd_old, n * S).reshape(n, S),
             rev_new=f(l.rev_new, n * S).reshape(n, S), rev_old=f(l.rev_old, n * S).reshape(n, S),
             counts=f(l.counts, n * 4).reshape(n, 4), inbox_counts=f(l.inbox_counts, n),
+            segment_state=f(l.segment_state, 16), segment_updates=f(l.segment_updates, 16),
             inbox=f(l.inbox, n * l.inbox_cap * 2).reshape(n, l.inbox_cap, 2), bloom=f(l.bloom, n * l.bloom_sets * 16).reshape(n, l.bloom_sets * 16),
             norms=f(l.norms, n, np.float32))
 
@@ -116,7 +117,8 @@ def _bloom_bits(key, sets):
 
 
 def model_merge(st, node, width, cap, sets):
-    """One node of the merge stage; returns (list_ids, list_dists, fwd_new, n_new, fwd_old, n_old, bloom words)."""
+    """One node of the merge stage; returns (list_ids, list_dists, fwd_new, n_new, fwd_old, n_old, bloom words,
+    number of offers that entered the list)."""
     ids, dists = [int(v) for v in st["list_ids"][node]], st["list_dists"][node]
     fwd_old = [v & ~OLD for v in ids if v != INV and v & OLD]
     n_in = min(int(st["inbox_counts"][node]), cap)
@@ -135,7 +137,7 @@ def model_merge(st, node, width, cap, sets):
         same = prev is not None and prev[0] == e[0] and prev[1] == e[1]
         if e[2] == 0:
             if not same:
-                out.append((e[1] | e[3], e[0]))
+                out.append((e[1] | e[3], e[0], 0))
         elif not same or prev[2] == 0:          # first offered copy of this id
             known = same
             if rank < S:
@@ -146,16 +148,17 @@ def model_merge(st, node, width, cap, sets):
                     for b in bits:
                         words[b >> 5] |= np.uint32(1 << (b & 31))
                 if not known:
-                    out.append((e[1] | (OLD if fresh else 0), e[0]))
+                    out.append((e[1] | (OLD if fresh else 0), e[0], 1))
             rank += 1
         prev = e
     out = out[:width]
     l_ids = np.full(width, INV, np.uint32)
     l_d = np.full(width, np.finfo(np.float32).max, np.float32)
-    for i, (v, db) in enumerate(out):
+    inserted = sum(o[2] for o in out)
+    for i, (v, db, _) in enumerate(out):
         l_ids[i] = v
         l_d[i] = np.array([db], np.uint32).view(np.float32)[0]
-    return l_ids, l_d, fwd_new, len(fwd_new), fwd_old[:S], min(len(fwd_old), S), words
+    return l_ids, l_d, fwd_new, len(fwd_new), fwd_old[:S], min(len(fwd_old), S), words, inserted
 
 
 @pytest.mark.parametrize("degree", [32, 64])
@@ -221,8 +224,11 @@ def test_stages_match_model(hip, degree):
         hip.nnd_merge(*args)
         hip.synchronize()
         merged = ws.read()
+        updates = [0, 0]
         for node in range(num):
-            l_ids, l_d, fn, n_new, fo, n_old, words = model_merge(after, node, width, cap, sets)
+            l_ids, l_d, fn, n_new, fo, n_old, words, inserted = model_merge(after, node, width, cap, sets)
+            if node % 100 == 0:
+                updates[0 if node < seg_len[0] else 1] += inserted
             np.testing.assert_array_equal(merged["list_ids"][node], l_ids, err_msg="list ids of node %d" % node)
             np.testing.assert_array_equal(merged["list_dists"][node], l_d)
             assert merged["counts"][node].tolist() == [n_new, n_old, 0, 0]
@@ -230,7 +236,25 @@ def test_stages_match_model(hip, degree):
             assert merged["fwd_old"][node, :n_old].tolist() == fo
             np.testing.assert_array_equal(merged["bloom"][node], words)
         assert (merged["inbox_counts"] == 0).all()
-        st = merged
+        assert merged["segment_updates"][:2].tolist() == updates
+        # termination test: limit = threshold * rows * dim / 100; a partition below it gets one more round, then rests
+        threshold = [0.0, 1e9, 1e9][it]
+        before = merged["segment_state"][:2].tolist()
+        hip.nnd_converge(num, dim, d_ss, d_sl, 2, degree, threshold, ws.buf, ws.bytes)
+        hip.synchronize()
+        st = ws.read()
+        expect = [2 if b == 1 else (1 if b == 0 and u < threshold * num * dim / 100 else b) for b, u in zip(before, updates)]
+        assert st["segment_state"][:2].tolist() == expect and st["segment_updates"][:2].tolist() == [0, 0]
+        assert expect == [[0, 0], [1, 1], [2, 2]][it]
+
+    # a resting partition is skipped by every stage
+    hip.nnd_reverse_sample(*args)
+    hip.nnd_local_join(*args)
+    hip.nnd_merge(*args)
+    hip.synchronize()
+    rest = ws.read()
+    for key in ("list_ids", "list_dists", "fwd_new", "fwd_old", "bloom", "inbox_counts"):
+        np.testing.assert_array_equal(rest[key], st[key], err_msg=key)
 
     d_knn = hip.DeviceArray((num, degree), np.uint32)
     hip.nnd_finalize(num, dim, d_ss, d_sl, 2, degree, d_knn, None, ws.buf, ws.bytes)
