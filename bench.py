@@ -299,7 +299,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": main_res["workload"], "graph_degree": 32, "top_k": 10, "beam": main_res["beam"],
                    "build_beam": 64, "refine_beam": 128, "relaxant": 1.05, "boundary_factor": 1.04, "sample_factor": 0.01,
-                   "nnd_iterations": main_res["nnd_iterations"]},
+                   "nnd_iterations": main_res["nnd_iterations"], "nnd_termination_threshold": 1e-4},
         "device": info["name"],
     }
     for k in ("build_sec", "build_stages", "graph_recall_at_32", "graph_recall_at_32_global", "recall_at_10", "recall_target_met",

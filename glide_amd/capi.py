@@ -341,6 +341,10 @@ def nnd_finalize(reorder_num, dim, segment_starts, segment_lengths, segment_num,
                                        vp(stream)), "glide_hip_nnd_finalize")
 
 
+def widen_u8(src, count, dst, stream=None):
+    check(lib().glide_hip_widen_u8(_ptr(src), C.c_size_t(count), _ptr(dst), vp(stream)), "glide_hip_widen_u8")
+
+
 def copy_bytes(dst, src, nbytes, stream=None):
     check(lib().glide_hip_copy_bytes(_ptr(dst), _ptr(src), C.c_size_t(nbytes), vp(stream)), "glide_hip_copy_bytes")
 

@@ -5,6 +5,18 @@
 namespace glide {
 
 // one 32-lane half per row pair; generic dim (any multiple of 4, looped in 128-dim chunks)
+// uint8 rows -> fp32 rows (the reference's large-path kernels cast every byte where they use it, search_kernel.cuh:493-544);
+// four values per thread and step, the tail value by value
+__global__ __launch_bounds__(256) void widen_u8_kernel(const unsigned char* src, size_t count, float* dst) {
+    const size_t quads = count / 4;
+    for (size_t q = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; q < quads; q += static_cast<size_t>(gridDim.x) * 256) {
+        const uint32_t w = reinterpret_cast<const uint32_t*>(src)[q];
+        reinterpret_cast<float4*>(dst)[q] = make_float4(static_cast<float>(w & 0xff), static_cast<float>((w >> 8) & 0xff),
+                                                        static_cast<float>((w >> 16) & 0xff), static_cast<float>(w >> 24));
+    }
+    if (blockIdx.x == 0 && threadIdx.x < count % 4) dst[quads * 4 + threadIdx.x] = static_cast<float>(src[quads * 4 + threadIdx.x]);
+}
+
 __global__ __launch_bounds__(64) void distance_batch_kernel(const float* a, const float* b, uint32_t n, uint32_t dim,
                                                             int metric, float* out) {
     const int lane = lane_id();
@@ -97,6 +109,15 @@ int glide_hip_distance_batch(const float* a, const float* b, uint32_t n, uint32_
     if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
     if (n == 0) return GLIDE_OK;
     hipLaunchKernelGGL(distance_batch_kernel, dim3((n + 1) / 2), dim3(64), 0, as_stream(stream), a, b, n, dim, metric, out);
+    return launch_status();
+}
+
+int glide_hip_widen_u8(const unsigned char* src, size_t count, float* dst, void* stream) {
+    if (!src || !dst || reinterpret_cast<uintptr_t>(dst) % 16 || reinterpret_cast<uintptr_t>(src) % 4) return GLIDE_ERR_BAD_ARGUMENT;
+    if (count == 0) return GLIDE_OK;
+    const size_t quads = (count + 3) / 4;
+    const size_t blocks = (quads + 255) / 256;
+    hipLaunchKernelGGL(widen_u8_kernel, dim3(static_cast<uint32_t>(blocks < 16384 ? blocks : 16384)), dim3(256), 0, as_stream(stream), src, count, dst);
     return launch_status();
 }
 

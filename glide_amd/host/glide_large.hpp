@@ -1,5 +1,5 @@
 // class GLIDE_large: data, graph and map live in pinned host memory; one partition at a time is staged through the
-// GPU.  Reference: glide_large.cuh:14-212, glide_large_impl.cuh:14-507 (instantiated there for uint8 rows; float here).
+// GPU.  Reference: glide_large.cuh:14-212, glide_large_impl.cuh:14-507 (instantiated there for uint8 rows; uint8 or float here).
 // Partitions are independent on this path (no boundary list, no cross-partition merge), so build -> reverse edges ->
 // refine run back to back on a staged partition instead of in three passes over the host arrays, and the copy of
 // the next partition overlaps the kernels of the current one.
@@ -20,7 +20,6 @@ namespace glide {
 
 template <typename Data_t, typename Index_t>
 class GLIDE_large {
-    static_assert(sizeof(Data_t) == 4, "float rows");
 
 public:
     // glide_large_impl.cuh:14-28: an index to be built
@@ -56,7 +55,7 @@ public:
         const uint32_t knn_degree = h_knn_graph.extent(1), deg = graph_degree();
         uint32_t max_len = 0;
         for (uint32_t s = 0; s < segment_num(); s++) max_len = std::max(max_len, h_segment_length(s));
-        device_matrix<float> d_data[2] = {device_matrix<float>(max_len, dim()), device_matrix<float>(max_len, dim())};
+        staged_rows<Data_t> d_data[2] = {staged_rows<Data_t>(max_len, dim()), staged_rows<Data_t>(max_len, dim())};
         device_matrix<uint32_t> d_knn[2] = {device_matrix<uint32_t>(max_len, knn_degree), device_matrix<uint32_t>(max_len, knn_degree)};
         device_matrix<uint32_t> d_graph(max_len, deg), d_rev(max_len, deg);
         device_vector<uint32_t> d_rev_count(max_len);
@@ -68,7 +67,7 @@ public:
             const int b = s & 1;
             const size_t start = h_segment_start(s), len = h_segment_length(s);
             st.before_copy(b);
-            hip_try(glide_hip_memcpy_h2d_async(d_data[b].data_handle(), h_data.row(start), len * dim() * sizeof(float), st.copy_stream()), "h2d data");
+            d_data[b].upload_async(h_data.row(start), len, st.copy_stream());
             hip_try(glide_hip_memcpy_h2d_async(d_knn[b].data_handle(), h_knn_graph.row(start), len * knn_degree * sizeof(uint32_t), st.copy_stream()), "h2d knn");
             st.after_copy(b);
         };
@@ -84,6 +83,7 @@ public:
             const uint32_t len = h_segment_length(s);
             if (s + 1 < segment_num()) stage(s + 1);
             st.before_compute(b);
+            d_data[b].widen(len, cs);
             SearchParameter& p = search_param_knn;
             hip_try(glide_hip_build_segment(d_data[b].data_handle(), len, dim(), d_knn[b].data_handle(), knn_degree, h_start_point(s), deg, p.beam,
                                             p.max_iterations, p.min_iterations, p.hash_bit, p.hash_reset_interval, build_param.relaxant_factor, mc,
@@ -126,7 +126,7 @@ public:
         copy_to_device(d_centroids.data_handle(), h_centroids.data_handle(), h_centroids.size());
         uint32_t max_len = 0;
         for (uint32_t s = 0; s < segment_num(); s++) max_len = std::max(max_len, h_segment_length(s));
-        device_matrix<float> d_data[2] = {device_matrix<float>(max_len, dim()), device_matrix<float>(max_len, dim())};
+        staged_rows<Data_t> d_data[2] = {staged_rows<Data_t>(max_len, dim()), staged_rows<Data_t>(max_len, dim())};
         device_matrix<uint32_t> d_graph[2] = {device_matrix<uint32_t>(max_len, deg), device_matrix<uint32_t>(max_len, deg)};
         device_vector<uint32_t> d_map[2] = {device_vector<uint32_t>(max_len), device_vector<uint32_t>(max_len)};
         const int mc = metric_code(metric);
@@ -136,7 +136,7 @@ public:
             const int b = s & 1;
             const size_t start = h_segment_start(s), len = h_segment_length(s);
             st.before_copy(b);
-            hip_try(glide_hip_memcpy_h2d_async(d_data[b].data_handle(), h_data.row(start), len * dim() * sizeof(float), st.copy_stream()), "h2d data");
+            d_data[b].upload_async(h_data.row(start), len, st.copy_stream());
             hip_try(glide_hip_memcpy_h2d_async(d_graph[b].data_handle(), h_graph.row(start), len * deg * sizeof(uint32_t), st.copy_stream()), "h2d graph");
             hip_try(glide_hip_memcpy_h2d_async(d_map[b].data_handle(), h_map.data_handle() + start, len * sizeof(uint32_t), st.copy_stream()), "h2d map");
             st.after_copy(b);
@@ -151,7 +151,16 @@ public:
         std::memcpy(&fmax_bits, &fmax, 4);
         hip_try(glide_hip_fill_u32(reinterpret_cast<uint32_t*>(d_final_dists.data_handle()), fmax_bits, d_final_dists.size(), cs), "glide_hip_fill_u32");
         hip_try(glide_hip_event_record(t0, cs), "glide_hip_event_record");
-        hip_try(glide_hip_select_segments(d_query_view.data_handle(), query_number, dim(), d_centroids.data_handle(), c, min_segment_num,
+        // uint8 queries (large_search.cu:111) are widened once; every kernel below reads fp32 queries
+        device_matrix<float> d_query_f32(sizeof(Data_t) == 1 ? query_number : 0, dim());
+        const float* d_queries = reinterpret_cast<const float*>(d_query_view.data_handle());
+        if (sizeof(Data_t) == 1) {
+            hip_try(glide_hip_widen_u8(reinterpret_cast<const unsigned char*>(d_query_view.data_handle()), static_cast<size_t>(query_number) * dim(),
+                                       d_query_f32.data_handle(), cs),
+                    "glide_hip_widen_u8");
+            d_queries = d_query_f32.data_handle();
+        }
+        hip_try(glide_hip_select_segments(d_queries, query_number, dim(), d_centroids.data_handle(), c, min_segment_num,
                                           boundary_factor, mc, d_segment_ids.data_handle(), cs),
                 "glide_hip_select_segments");
         if (segment_num()) stage(0);
@@ -159,8 +168,9 @@ public:
             const int b = s & 1;
             if (s + 1 < segment_num()) stage(s + 1);
             st.before_compute(b);
+            d_data[b].widen(h_segment_length(s), cs);
             hip_try(glide_hip_search_sub(d_data[b].data_handle(), dim(), d_graph[b].data_handle(), deg, d_map[b].data_handle(),
-                                         d_query_view.data_handle(), query_number, d_segment_ids.data_handle(), c, s, h_start_point(s), top_k,
+                                         d_queries, query_number, d_segment_ids.data_handle(), c, s, h_start_point(s), top_k,
                                          param.beam, param.max_iterations, param.min_iterations, param.hash_bit, param.hash_reset_interval, mc,
                                          d_final_ids.data_handle(), d_final_dists.data_handle(), nullptr, cs),
                     "glide_hip_search_sub");

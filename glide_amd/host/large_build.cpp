@@ -36,13 +36,18 @@ int main(int argc, char** argv) {
     if (search_param_refine.beam != 0) size_param(search_param_refine, search_param_refine.beam);
 
     auto h_knn_graph = load_matrix_pinned<uint32_t>(knn_file);
-    GLIDE_large<float, uint64_t> index(handle, build_param.graph_degree, build_param.metric, reorder_file, map_file, centroid_file, segment_file);
     {
         std::ofstream result_out(result_file, std::ios::app);
         result_out << build_param.graph_degree << ",";
     }
-    index.build(build_param, search_param_knn, search_param_refine, h_knn_graph, result_file);
-    save_matrix_pinned(graph_base_file + ".graph", index.graph_view());
-    save_vector_data(graph_base_file + ".sp", index.start_point_view());
+    auto run = [&](auto tag) {   // uint8 rows as in the reference (large_build.cu:84) or fp32 rows, by the length of the .reorder file
+        using Data_t = decltype(tag);
+        GLIDE_large<Data_t, uint64_t> index(handle, build_param.graph_degree, build_param.metric, reorder_file, map_file, centroid_file, segment_file);
+        index.build(build_param, search_param_knn, search_param_refine, h_knn_graph, result_file);
+        save_matrix_pinned(graph_base_file + ".graph", index.graph_view());
+        save_vector_data(graph_base_file + ".sp", index.start_point_view());
+    };
+    if (fbin_element_bytes(reorder_file) == 1) run(uint8_t{});
+    else run(float{});
     return 0;
 }

@@ -1,5 +1,6 @@
 // large_preprocess data_file preprocess_file result_file centroid_num sample_factor metric
-// Reference: large_preprocess.cu:21-80 (same argv and output files; float rows here, uint8 there).
+// Reference: large_preprocess.cu:21-80 (same argv and output files).  The rows may be uint8, as the reference reads them,
+// or fp32; the element size is taken from the length of the data file.
 #include <cstdlib>
 #include <fstream>
 #include <iostream>
@@ -9,6 +10,24 @@
 #include "partition_large.hpp"
 
 using namespace glide;
+
+template <typename Data_t>
+static void run(device_resources& handle, PartitionParameter& param, const std::string& data_file, const std::string& preprocess_file,
+                std::string& result_file, uint32_t batch_num) {
+    auto h_data = load_matrix_pinned<Data_t>(data_file);
+    const size_t num = h_data.extent(0), dim = h_data.extent(1);
+    pinned_matrix<Data_t> h_reorder(num, dim);
+    host_vector<uint32_t> h_map(num), h_segment_start(param.centroid_num), h_segment_length(param.centroid_num);
+    device_matrix<float> d_centroids(param.centroid_num, dim);
+    preprocess_for_large<Data_t>(handle, param, h_data, h_reorder, h_map.view(), h_segment_start.view(), h_segment_length.view(), d_centroids.view(),
+                                batch_num, result_file);
+    host_matrix<float> h_centroids(param.centroid_num, dim);
+    copy_to_host(h_centroids.data_handle(), d_centroids.data_handle(), h_centroids.size());
+    save_matrix_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view());
+    save_segment(preprocess_file + ".segment", std::as_const(h_segment_start).view(), std::as_const(h_segment_length).view());
+    save_vector_data(preprocess_file + ".map", std::as_const(h_map).view());
+    save_matrix_pinned(preprocess_file + ".reorder", h_reorder);
+}
 
 int main(int argc, char** argv) {
     if (argc != 7) {
@@ -29,18 +48,7 @@ int main(int argc, char** argv) {
         std::ofstream result_out(result_file, std::ios::app);
         result_out << "pre_time,knn_time,degree,index_time,beam,search_time,QPS,recall" << std::endl;
     }
-    auto h_data = load_matrix_pinned<float>(data_file);
-    const size_t num = h_data.extent(0), dim = h_data.extent(1);
-    pinned_matrix<float> h_reorder(num, dim);
-    host_vector<uint32_t> h_map(num), h_segment_start(param.centroid_num), h_segment_length(param.centroid_num);
-    device_matrix<float> d_centroids(param.centroid_num, dim);
-    preprocess_for_large<float>(handle, param, h_data, h_reorder, h_map.view(), h_segment_start.view(), h_segment_length.view(), d_centroids.view(),
-                                batch_num, result_file);
-    host_matrix<float> h_centroids(param.centroid_num, dim);
-    copy_to_host(h_centroids.data_handle(), d_centroids.data_handle(), h_centroids.size());
-    save_matrix_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view());
-    save_segment(preprocess_file + ".segment", std::as_const(h_segment_start).view(), std::as_const(h_segment_length).view());
-    save_vector_data(preprocess_file + ".map", std::as_const(h_map).view());
-    save_matrix_pinned(preprocess_file + ".reorder", h_reorder);
+    if (fbin_element_bytes(data_file) == 1) run<uint8_t>(handle, param, data_file, preprocess_file, result_file, batch_num);
+    else run<float>(handle, param, data_file, preprocess_file, result_file, batch_num);
     return 0;
 }

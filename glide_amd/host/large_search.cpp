@@ -41,18 +41,23 @@ int main(int argc, char** argv) {
         std::ofstream result_out(result_file, std::ios::app);
         result_out << param.beam << ",";
     }
-    GLIDE_large<float, uint64_t> index(handle, metric, reorder_file, map_file, centroid_file, segment_file, sp_file, graph_file);
-    adjust_search_params(param.min_iterations, param.max_iterations, param.beam);
-    param.hash_bit = calculate_hash_bitlen(param.beam, index.graph_degree(), param.hash_max_fill_rate, param.hashmap_min_bitlen);
-    param.hash_reset_interval = calculate_hash_reset_interval(param.beam, index.graph_degree(), param.hash_max_fill_rate, param.hash_bit);
-
-    auto h_query = load_matrix_data<float, uint32_t>(query_file);
     auto h_truth = load_matrix_data<uint32_t, uint32_t>(truth_file);
-    device_matrix<float> d_query(h_query.extent(0), h_query.extent(1));
-    copy_to_device(d_query.data_handle(), h_query.data_handle(), h_query.size());
-    host_matrix<uint32_t> result_ids(h_query.extent(0), param.top_k);
-    host_matrix<float> result_dists(h_query.extent(0), param.top_k);
-    index.search(param, min_segment_num, boundary_factor, d_query.view(), result_ids.view(), result_dists.view(), result_file);
+    const uint32_t query_number = h_truth.extent(0);
+    host_matrix<uint32_t> result_ids(query_number, param.top_k);
+    host_matrix<float> result_dists(query_number, param.top_k);
+    auto run = [&](auto tag) {   // rows and queries are uint8 as in the reference (large_search.cu:99-112) or fp32, by the .reorder file
+        using Data_t = decltype(tag);
+        GLIDE_large<Data_t, uint64_t> index(handle, metric, reorder_file, map_file, centroid_file, segment_file, sp_file, graph_file);
+        adjust_search_params(param.min_iterations, param.max_iterations, param.beam);
+        param.hash_bit = calculate_hash_bitlen(param.beam, index.graph_degree(), param.hash_max_fill_rate, param.hashmap_min_bitlen);
+        param.hash_reset_interval = calculate_hash_reset_interval(param.beam, index.graph_degree(), param.hash_max_fill_rate, param.hash_bit);
+        auto h_query = load_matrix_data<Data_t, uint32_t>(query_file);
+        device_matrix<Data_t> d_query(h_query.extent(0), h_query.extent(1));
+        copy_to_device(d_query.data_handle(), h_query.data_handle(), h_query.size());
+        index.search(param, min_segment_num, boundary_factor, d_query.view(), result_ids.view(), result_dists.view(), result_file);
+    };
+    if (fbin_element_bytes(reorder_file) == 1) run(uint8_t{});
+    else run(float{});
     const float recall = calculate_recall(result_ids, h_truth, param.top_k);
     std::cout << "total_recall: " << recall << std::endl;
     std::ofstream result_out(result_file, std::ios::app);

@@ -61,7 +61,7 @@ pinned_matrix<int> build_knn_for_large(device_resources& handle, uint32_t knn_de
     uint32_t max_len = 0;
     for (uint32_t s = 0; s < segments; s++) max_len = std::max(max_len, h_segment_length_view(s));
     pinned_matrix<int> knn_graph(num, knn_degree);
-    device_matrix<float> d_data[2] = {device_matrix<float>(max_len, dim), device_matrix<float>(max_len, dim)};
+    staged_rows<Data_t> d_data[2] = {staged_rows<Data_t>(max_len, dim), staged_rows<Data_t>(max_len, dim)};
     device_matrix<uint32_t> d_knn[2] = {device_matrix<uint32_t>(max_len, knn_degree), device_matrix<uint32_t>(max_len, knn_degree)};
     const size_t wb = glide_hip_nnd_workspace_bytes(max_len, dim, knn_degree);
     device_buffer ws(wb);
@@ -73,9 +73,7 @@ pinned_matrix<int> build_knn_for_large(device_resources& handle, uint32_t knn_de
     auto stage = [&](uint32_t s) {
         const int b = s & 1;
         st.before_copy(b);
-        hip_try(glide_hip_memcpy_h2d_async(d_data[b].data_handle(), h_reorder_data.row(h_segment_start_view(s)),
-                                           static_cast<size_t>(h_segment_length_view(s)) * dim * sizeof(float), st.copy_stream()),
-                "glide_hip_memcpy_h2d_async");
+        d_data[b].upload_async(h_reorder_data.row(h_segment_start_view(s)), h_segment_length_view(s), st.copy_stream());
         st.after_copy(b);
     };
     void* t0 = nullptr;
@@ -89,6 +87,7 @@ pinned_matrix<int> build_knn_for_large(device_resources& handle, uint32_t knn_de
         const uint32_t len = h_segment_length_view(s);
         if (s + 1 < segments) stage(s + 1);
         st.before_compute(b);
+        d_data[b].widen(len, st.compute_stream());
         hip_try(glide_hip_nnd_build(d_data[b].data_handle(), len, dim, d_seg.data_handle() + 2 * s, d_seg.data_handle() + 2 * s + 1, 1, knn_degree,
                                     iterations, termination_threshold, seed + s, d_knn[b].data_handle(), ws.get(), wb, nullptr,
                                     st.compute_stream()),

@@ -76,6 +76,45 @@ void save_matrix_pinned(const std::string& path, const pinned_matrix<T>& m) {
     }
 }
 
+// Size in bytes of one element of an fbin file, from its length: header (num, dim) + num * dim elements.  The reference's
+// large executables read uint8 rows (large_preprocess.cu:56); this build also takes fp32 rows in the same layout.
+inline size_t fbin_element_bytes(const std::string& path) {
+    std::ifstream file(path, std::ios::binary | std::ios::ate);
+    if (!file) { std::cerr << "Error opening file: " << path << std::endl; return 0; }
+    const size_t bytes = static_cast<size_t>(file.tellg());
+    file.seekg(0);
+    uint32_t num = 0, dim = 0;
+    file.read(reinterpret_cast<char*>(&num), sizeof(uint32_t));
+    file.read(reinterpret_cast<char*>(&dim), sizeof(uint32_t));
+    const size_t count = static_cast<size_t>(num) * dim;
+    return count ? (bytes - 8) / count : 0;
+}
+
+// One staging slot for a block of rows: uploaded in their stored type, read by every kernel as fp32.  Float rows are
+// copied straight into place; uint8 rows are copied raw (a quarter of the PCIe traffic) and widened on the GPU.
+template <typename Data_t>
+class staged_rows {
+    static_assert(sizeof(Data_t) == 4 || sizeof(Data_t) == 1, "float or uint8 rows");
+public:
+    staged_rows(size_t max_rows, uint32_t dim) : rows_(max_rows, dim), raw_(sizeof(Data_t) == 1 ? max_rows * dim + 16 : 16) {}
+    // on the copy stream
+    void upload_async(const Data_t* src, size_t rows, void* stream) {
+        hip_try(glide_hip_memcpy_h2d_async(stored(), src, rows * rows_.extent(1) * sizeof(Data_t), stream), "glide_hip_memcpy_h2d_async");
+    }
+    // on the compute stream, once the copy is known to be complete
+    void widen(size_t rows, void* stream) {
+        if (sizeof(Data_t) == 1)
+            hip_try(glide_hip_widen_u8(static_cast<const unsigned char*>(raw_.get()), rows * rows_.extent(1), rows_.data_handle(), stream),
+                    "glide_hip_widen_u8");
+    }
+    float* data_handle() const { return rows_.data_handle(); }
+    // the rows in their stored type (same memory as data_handle() for float rows)
+    Data_t* stored() const { return sizeof(Data_t) == 1 ? static_cast<Data_t*>(raw_.get()) : reinterpret_cast<Data_t*>(rows_.data_handle()); }
+private:
+    device_matrix<float> rows_;
+    device_buffer raw_;
+};
+
 // two streams + events for "copy partition s+1 while partition s computes"
 class stager {
 public:

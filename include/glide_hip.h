@@ -267,6 +267,11 @@ int glide_hip_memcpy_h2d_async(void *dst, const void *src, size_t bytes, void *s
 int glide_hip_memcpy_d2h_async(void *dst, const void *src, size_t bytes, void *stream);
 int glide_hip_stream_wait_event(void *stream, void *event);
 
+/* uint8 rows -> fp32 rows on the device (count values; src 4-byte aligned, dst 16-byte aligned).  The reference's large
+ * path keeps uint8 rows and casts each byte to float where a kernel reads it (search_kernel.cuh:493-544,
+ * graph_kernel.cuh:675-821); here a staged partition is widened once after its upload and every kernel reads fp32. */
+int glide_hip_widen_u8(const unsigned char *src, size_t count, float *dst, void *stream);
+
 /* ---- test hooks for the device primitives (subsystems 5, 6 and the hash set) ------------------------------ */
 /* A plain copy kernel (bytes % 16 == 0, 16-byte aligned): no counterpart in the reference; it is the transfer
  * of known size against which hardware byte counters (FETCH_SIZE / WRITE_SIZE) are calibrated. */

@@ -138,3 +138,43 @@ def test_large_pipeline_cli(tmp_path):
     assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= 0.9
     row = open(result).read().strip().splitlines()[1].split(",")
     assert len(row) == 8
+
+
+def test_large_pipeline_cli_uint8(tmp_path):
+    """The reference's large executables read uint8 rows and uint8 queries (large_preprocess.cu:56, large_search.cu:111).
+    Bytes are widened to fp32 on the GPU, so a uint8 run must reproduce the fp32 run on the same values: same
+    partitioning, and -- from the same kNN file -- the same graph and the same search results."""
+    from glide_amd import datasets as D
+    from oracle import oracle as O
+    n, dim, nq, c = 6000, 128, 150, 4
+    data, queries = lowdim_data(n, dim, seed=61), lowdim_data(nq, dim, seed=62)      # integer values 0..255
+    truth, _ = O.bruteforce_knn(data, queries, 100)
+    out = {}
+    for kind, cast in (("f32", np.float32), ("u8", np.uint8)):
+        d = tmp_path / kind
+        d.mkdir()
+        f = lambda name: str(d / name)
+        D.write_fbin(f("base.fbin"), data.astype(cast))
+        D.write_fbin(f("query.fbin"), queries.astype(cast))
+        D.write_fbin(f("truth"), truth.astype(np.uint32))
+        pre, result = f("pre"), f("result.csv")
+        run(os.path.join(BIN, "large_preprocess"), f("base.fbin"), pre, result, c, 0.05, "Euclidean")
+        rdata = D.read_fbin(pre + ".reorder", cast)
+        assert rdata.dtype == cast and rdata.shape == (n, dim)
+        run(os.path.join(BIN, "large_knn"), pre, f("knn"), result, 32)
+        knn = D.read_fbin(f("knn"), np.uint32)
+        starts, lengths = D.read_segment(pre + ".segment")
+        s, l = int(starts[0]), int(lengths[0])
+        gt, _ = O.bruteforce_knn(rdata[s:s + l].astype(np.float32), rdata[s:s + 150].astype(np.float32), 32, exclude_self=True)
+        assert D.recall(knn[s:s + 150], gt, 32) >= 0.95
+        if kind == "u8":                       # same kNN graph into both builds
+            D.write_fbin(f("knn"), out["f32"]["knn"])
+        run(os.path.join(BIN, "large_build"), pre, f("knn"), f("graph"), result, "Euclidean", 32, 32, 1.05, 64, 128)
+        text = run(os.path.join(BIN, "large_search"), pre, f("query.fbin"), f("truth"), f("graph"), result, "Euclidean", 10, 64, 2, 1.1)
+        out[kind] = dict(rdata=rdata.astype(np.float32), map=D.read_vector(pre + ".map"), starts=starts, lengths=lengths, knn=knn,
+                         centroids=D.read_fbin(pre + ".centroid"), graph=D.read_fbin(f("graph") + ".graph", np.uint32),
+                         sp=D.read_vector(f("graph") + ".sp"), recall=float(text.split("total_recall:")[1].split()[0]))
+    a, b = out["f32"], out["u8"]
+    for key in ("rdata", "map", "starts", "lengths", "centroids", "graph", "sp"):
+        assert np.array_equal(a[key], b[key]), key
+    assert a["recall"] == b["recall"] and b["recall"] >= 0.9

@@ -116,3 +116,15 @@ def test_argument_errors(hip):
     with pytest.raises(hip.GlideHipError) as e:
         hip.distance_batch(None, d, 1, 4, 0, d)
     assert e.value.code == -2
+
+
+@pytest.mark.parametrize("count", [1, 3, 4, 127, 128, 1000003])
+def test_widen_u8(hip, count):
+    src = np.random.default_rng(count).integers(0, 256, size=count + 3, dtype=np.uint8)
+    d_src = hip.DeviceArray.from_numpy(src)
+    d_dst = hip.DeviceArray.full((count + 1,), -1.0, np.float32)
+    hip.widen_u8(d_src, count, d_dst)
+    hip.synchronize()
+    out = d_dst.numpy()
+    np.testing.assert_array_equal(out[:count], src[:count].astype(np.float32))
+    assert out[count] == -1.0
