@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg1-navigable"])
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg1-navigable", "cfg2", "cfg3"])
     ap.add_argument("--nnd-iterations", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-navigable", action="store_true", help="skip the extra navigable-data variant")
@@ -49,10 +49,12 @@ def parse():
 
 
 WORKLOADS = {
-    # name: (num, partitions, knn degree, NN-descent iterations, queries, description)
-    "cfg0": (100_000, 10, 64, 8, 1_000, "cfg0: 100k x 128 fp32 clipped/rounded 64-component GMM, L2, degree 32, NN-descent k=64 x 8 iterations, 1k queries"),
-    "cfg1": (1_000_000, 16, 32, 20, 10_000, "cfg1: 1M x 128 fp32 clipped/rounded 64-component GMM, L2, 16 partitions, degree 32, 10k queries top-10, beams 32/64/128/256"),
-    "cfg1-navigable": (1_000_000, 16, 32, 20, 10_000, "cfg1 shapes on integer-valued data of low intrinsic dimension (12-d latent, 0..255): 1M x 128, 16 partitions, degree 32, 10k queries top-10"),
+    # name: (num, partitions, knn degree, NN-descent iterations, queries, description, dim, metric, graph degree)
+    "cfg0": (100_000, 10, 64, 8, 1_000, "cfg0: 100k x 128 fp32 clipped/rounded 64-component GMM, L2, degree 32, NN-descent k=64 x 8 iterations, 1k queries", 128, 0, 32),
+    "cfg1": (1_000_000, 16, 32, 20, 10_000, "cfg1: 1M x 128 fp32 clipped/rounded 64-component GMM, L2, 16 partitions, degree 32, 10k queries top-10, beams 32/64/128/256", 128, 0, 32),
+    "cfg1-navigable": (1_000_000, 16, 32, 20, 10_000, "cfg1 shapes on integer-valued data of low intrinsic dimension (12-d latent, 0..255): 1M x 128, 16 partitions, degree 32, 10k queries top-10", 128, 0, 32),
+    "cfg2": (1_000_000, 16, 32, 20, 10_000, "cfg2: 1M x 96 fp32 L2-normalised 256-component GMM, cosine, 16 partitions, degree 32, 10k queries top-10", 96, 1, 32),
+    "cfg3": (1_000_000, 16, 64, 20, 1_000, "cfg3: 1M x 960 fp32 Beta(0.5,2) x per-cluster scales, L2, 16 partitions, degree 64, 1k queries top-10", 960, 0, 64),
 }
 
 
@@ -71,6 +73,10 @@ def make_data(workload, num, nq):
                 out[s:e] = np.rint(np.clip(z @ a * 20 + 128 + r.standard_normal((e - s, 128)).astype(np.float32) * 3, 0, 255))
             return out
         return gen(num, 1234), gen(nq, 4321)
+    if workload == "cfg2":
+        return D.gmm_normalized(num, 96, seed=1234), D.gmm_normalized(nq, 96, seed=4321)
+    if workload == "cfg3":
+        return D.beta_scaled(num, 960, seed=1234), D.beta_scaled(nq, 960, seed=4321)
     return D.gmm_clipped(num, 128, seed=1234), D.gmm_clipped(nq, 128, seed=4321)
 
 
@@ -93,17 +99,17 @@ def run_workload(args, workload, torch, want_cpu):
     import numpy as np
     from glide_amd import capi, datasets as D, index as G
 
-    num, parts, knn_degree, nnd_iters, nq, desc = WORKLOADS[workload]
+    num, parts, knn_degree, nnd_iters, nq, desc, dim, metric, degree = WORKLOADS[workload]
     if args.nnd_iterations:
         nnd_iters = args.nnd_iterations
-    degree, top_k = 32, 10
+    top_k = 10
     t0 = time.time()
     data, queries = make_data(workload, num, nq)
     gen_s = time.time() - t0
 
     d_data = capi.DeviceArray.from_numpy(data)
     res = {}
-    pp = G.PartitionParameter(centroid_num=parts, boundary_factor=1.04, sample_factor=0.01)   # reference test.sh:10-12
+    pp = G.PartitionParameter(centroid_num=parts, boundary_factor=1.04, sample_factor=0.01, metric=metric)   # reference test.sh:10-12
     d_re, d_map, h_start, h_len, d_cent = G.preprocess(pp, d_data, res)
     nn = G.NNDescentParameter(graph_degree=knn_degree, max_iterations=nnd_iters)
     d_knn = G.build_nnd(nn, d_re, h_start, h_len, res, stats=True)
@@ -141,7 +147,7 @@ def run_workload(args, workload, torch, want_cpu):
     graph_recall_global = float(glob[0]) if glob else None
     del rdata, knn
 
-    index = G.GLIDE(degree, d_data, d_cent, G.Metric.Euclidean)
+    index = G.GLIDE(degree, d_data, d_cent, metric)
     bp = G.IndexParameter(graph_degree=degree, knn_degree=knn_degree, relaxant_factor=1.05)   # test.sh:16
     sp_knn = G.make_search_parameter(64, knn_degree)         # test.sh:17 build beam
     sp_ref = G.make_search_parameter(128, knn_degree)        # test.sh:18 refine beam (hash sized with knn_degree, small_build.cu:76-82)
@@ -165,7 +171,7 @@ def run_workload(args, workload, torch, want_cpu):
         index.search(sp, d_q, result=r, out=(d_ids, d_dists))
         rec = D.recall(d_ids.numpy(), gt, top_k)
         # algorithmic bytes of one launch: query rows + centroid table once + graph rows + scored data rows + results
-        alg = nq * 128 * 4 + parts * 128 * 4 + int(c[2]) * degree * 4 + int(c[1]) * 128 * 4 + nq * top_k * 8
+        alg = nq * dim * 4 + parts * dim * 4 + int(c[2]) * degree * 4 + int(c[1]) * dim * 4 + nq * top_k * 8
         sweep.append(dict(beam=beam, recall_at_10=rec, qps=r["QPS"], ms=r["search_time"] * 1e3, iterations_per_query=c[0] / nq,
                           rows_per_query=c[1] / nq, algorithmic_bytes=alg))
     ok = [s for s in sweep if s["recall_at_10"] >= 0.95]
@@ -180,8 +186,8 @@ def run_workload(args, workload, torch, want_cpu):
     w0 = time.time()
     e0.record()
     for _ in range(args.steps):
-        capi.search(index.d_data, num, 128, index.d_graph, degree, index.d_centroids, parts, index.d_start_points, d_q, nq, top_k,
-                    sp.beam, sp.max_iterations, sp.min_iterations, sp.hash_bit, sp.hash_reset_interval, 0, d_ids, d_dists)
+        capi.search(index.d_data, num, dim, index.d_graph, degree, index.d_centroids, parts, index.d_start_points, d_q, nq, top_k,
+                    sp.beam, sp.max_iterations, sp.min_iterations, sp.hash_bit, sp.hash_reset_interval, metric, d_ids, d_dists)
     e1.record()
     gpu_ms = e0.elapsed_ms(e1)
     capi.synchronize()
@@ -201,16 +207,17 @@ def run_workload(args, workload, torch, want_cpu):
         qps=nq * args.steps / (wall_ms * 1e-3), ms_per_step=ms_per_step, kernel_ms=kernel_ms,
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=MEASURED_TRAFFIC_BYTES.get((workload, chosen["beam"])),
-                      kernel="search_kernel<64,%d,1>" % (64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256),
+                      kernel="search_kernel<%d,%d,%d>" % (64 if degree <= 64 else 128, 64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256,
+                                                          1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8),
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )
 
     if want_cpu:
-        out["cpu_baseline"] = cpu_baseline(data, queries, graph, d_cent.numpy(), index.d_start_points.numpy(), sp, top_k, gt)
+        out["cpu_baseline"] = cpu_baseline(data, queries, graph, d_cent.numpy(), index.d_start_points.numpy(), sp, top_k, gt, metric)
     return out
 
 
-def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt):
+def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt, metric=0):
     """The CPU restatement of the reference algorithm, timed on this box's host cores on a bounded sample."""
     import numpy as np
     from glide_amd import datasets as D
@@ -224,7 +231,7 @@ def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt):
     nq = min(queries.shape[0], 4000)
     t = time.time()
     ids, _, _ = O.search(data, graph, centroids, start_points, queries[:nq], top_k, sp.beam, sp.max_iterations, sp.min_iterations,
-                         sp.hash_bit, sp.hash_reset_interval, 0, threads=cores)
+                         sp.hash_bit, sp.hash_reset_interval, metric, threads=cores)
     search_s = time.time() - t
     # NN-descent build of one 30k-point partition-sized sample with the same degree / 10 iterations
     n_s = min(30_000, data.shape[0])
@@ -232,7 +239,7 @@ def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt):
     O.nnd_build(data[:n_s], np.array([0], np.uint32), np.array([n_s], np.uint32), 32, 10, 0, threads=cores)
     nnd_s = time.time() - t
     t = time.time()
-    O.bruteforce_knn(data[:200_000], queries[:200], top_k, threads=cores)
+    O.bruteforce_knn(data[:200_000], queries[:200], top_k, metric, threads=cores)
     bf_s = time.time() - t
     return dict(value=nq / search_s, unit="queries/s", cores=cores, kind="port",
                 sample="beam search of the first %d queries (same index, beam %d) with the CPU restatement, %d threads" % (nq, sp.beam, cores),
@@ -297,7 +304,7 @@ def main():
         "value": main_res["qps"], "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": main_res["workload"], "graph_degree": 32, "top_k": 10, "beam": main_res["beam"],
+        "config": {"workload": main_res["workload"], "graph_degree": WORKLOADS[args.workload][8], "top_k": 10, "beam": main_res["beam"],
                    "build_beam": 64, "refine_beam": 128, "relaxant": 1.05, "boundary_factor": 1.04, "sample_factor": 0.01,
                    "nnd_iterations": main_res["nnd_iterations"], "nnd_termination_threshold": 1e-4},
         "device": info["name"],
