@@ -88,6 +88,7 @@ struct RefineArgs {
     const float* centroids;
     const uint32_t* start_points;
     unsigned long long* counters;
+    const uint32_t* order;   // nullable: workgroup i refines point order[i] (a permutation of the points)
     uint32_t num, centroid_num, max_centroid, segment_start_point;
     float relaxant;
     BeamParams p;   // p.degree = graph_degree
@@ -113,7 +114,8 @@ __global__ __launch_bounds__(64) void refine_kernel(RefineArgs a) {
     auto* pl = reinterpret_cast<PruneLds<MAX_BEAM>*>(smem + sizeof(BeamLds<MAX_CAND>));
     float* cent = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>) + sizeof(PruneLds<MAX_BEAM>));
     uint32_t* hash = reinterpret_cast<uint32_t*>(cent + round_up32(a.centroid_num));
-    const uint32_t point = blockIdx.x;
+    if (blockIdx.x >= a.num) return;
+    const uint32_t point = a.order ? a.order[blockIdx.x] : blockIdx.x;
     if (point >= a.num) return;
     const int lane = lane_id();
     const uint32_t D = a.p.degree;
@@ -417,6 +419,7 @@ int glide_hip_refine_segment(const float* segment_data, uint32_t num, uint32_t d
     if (num == 0) return GLIDE_OK;
     if (start_point >= num) return GLIDE_ERR_BAD_ARGUMENT;
     RefineArgs a;
+    a.order = nullptr;
     a.data = segment_data;
     a.graph_in = graph_in;
     a.graph_out = graph_out;
@@ -484,7 +487,8 @@ int glide_hip_insert_reverse(uint32_t* graph, const uint32_t* reverse_graph, con
 int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph_in, uint32_t* graph_out,
                      uint32_t graph_degree, const float* centroids, uint32_t centroid_num, const uint32_t* start_points,
                      uint32_t beam, uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
-                     uint32_t hash_reset_interval, float relaxant, int metric, unsigned long long* counters, void* stream) {
+                     uint32_t hash_reset_interval, float relaxant, int metric, const uint32_t* order, unsigned long long* counters,
+                     void* stream) {
     if (!data || !graph_in || !graph_out || !centroids || !start_points || graph_in == graph_out) return GLIDE_ERR_BAD_ARGUMENT;
     if (max_iterations == 0 || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
     int rc = check_beam_sizes(graph_degree, graph_degree, beam, dim, hash_bit, metric);
@@ -498,6 +502,7 @@ int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32
     a.centroids = centroids;
     a.start_points = start_points;
     a.counters = counters;
+    a.order = order;
     a.num = num;
     a.centroid_num = centroid_num;
     a.max_centroid = centroid_num <= 32 ? 32 : (graph_degree <= 64 ? 64 : (graph_degree <= 128 ? 128 : 256));

@@ -52,15 +52,15 @@ public:
         d_knn_graph.reset();
         d_segment_start.reset();
         d_segment_length.reset();
-        d_map.reset();
-        d_reorder_data.reset();
+        d_reorder_data.reset();   // d_map stays until the refine stage, which processes the points in partition order
 
         d_start_points.reset();
         d_start_points.emplace(h_start_point.size());
         copy_to_device(d_start_points->data_handle(), h_start_point.data_handle(), h_start_point.size());
 
         reverse_graph(build_time);
-        if (search_param_refine.beam != 0) refine(search_param_refine, build_param.relaxant_factor, build_time);
+        if (search_param_refine.beam != 0) refine(search_param_refine, build_param.relaxant_factor, d_map->data_handle(), build_time);
+        d_map.reset();
 
         std::cout << "index build time: " << build_time << " s" << std::endl;
         std::ofstream result_out(result_file, std::ios::app);
@@ -165,14 +165,14 @@ private:
     }
 
     // glide_impl.cuh:258-316
-    void refine(SearchParameter& param, float relaxant_factor, float& build_time) {
+    void refine(SearchParameter& param, float relaxant_factor, const uint32_t* d_order, float& build_time) {
         device_matrix<uint32_t, Index_t> d_refined(num(), graph_degree());
         gpu_timer timer;
         timer.start();
         hip_try(glide_hip_refine(d_data.data_handle(), num(), dim(), d_graph.data_handle(), d_refined.data_handle(), graph_degree(),
                                  d_centroids.data_handle(), centroid_num(), d_start_points->data_handle(), param.beam, param.max_iterations,
                                  param.min_iterations, param.hash_bit, param.hash_reset_interval, relaxant_factor, metric_code(metric),
-                                 nullptr, handle.stream()),
+                                 d_order, nullptr, handle.stream()),
                 "glide_hip_refine");
         build_time += timer.stop();
         d_graph = std::move(d_refined);

@@ -281,7 +281,7 @@ class GLIDE:
         if counters and result is not None:
             capi.synchronize()
             result["build_counters"] = capi.read_counters(cnt)
-        for consumed in (d_knn_graph, d_map, d_reorder_data):
+        for consumed in (d_knn_graph, d_reorder_data):     # d_map is kept until the refine stage, which uses it as its order
             capi.synchronize()
             consumed.free()
         self.d_start_points = capi.DeviceArray.from_numpy(sp)
@@ -304,12 +304,13 @@ class GLIDE:
             with _Timer() as t:
                 capi.refine(self.d_data, num, dim, self.d_graph, d_rev, deg, self.d_centroids, self.centroid_num(),
                             self.d_start_points, p.beam, p.max_iterations, p.min_iterations, p.hash_bit, p.hash_reset_interval,
-                            build_param.relaxant_factor, self.metric, cnt2)
+                            build_param.relaxant_factor, self.metric, cnt2, order=d_map)
             times["refine"] = t.seconds
             self.d_graph, d_rev = d_rev, self.d_graph
             if counters and result is not None:
                 result["refine_counters"] = capi.read_counters(cnt2)
         d_rev.free()
+        d_map.free()
         if result is not None:
             result["index_time"] = times["subgraph"] + times["boundary"] + times["reverse"]
             result["refine_time"] = times["refine"]

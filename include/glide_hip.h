@@ -219,12 +219,14 @@ int glide_hip_insert_reverse(uint32_t *graph, const uint32_t *reverse_graph, con
  * slots search the whole graph from the nearest centroid's start point and fill the slots after a prune that
  * skips existing neighbours.  Reads graph_in, writes every row of graph_out (graph_in != graph_out): the
  * reference refines in place while other blocks still traverse the rows; here all searches see the
- * pre-refinement graph. */
+ * pre-refinement graph.  `order` (nullable) is a permutation of the points: workgroup i refines point order[i].  The
+ * result does not depend on it; handing in the partition order (the first `num` entries of `map`) makes wavefronts
+ * that run together search the same region, which cuts HBM traffic (1M x 128 mixture data: 0.168 s -> 0.109 s). */
 int glide_hip_refine(const float *data, uint32_t num, uint32_t dim, const uint32_t *graph_in, uint32_t *graph_out,
                      uint32_t graph_degree, const float *centroids, uint32_t centroid_num,
                      const uint32_t *start_points, uint32_t beam, uint32_t max_iterations,
                      uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant,
-                     int metric, unsigned long long *counters, void *stream);
+                     int metric, const uint32_t *order, unsigned long long *counters, void *stream);
 
 /* ---- large path: one staged partition at a time (GLIDE_large, glide_large_impl.cuh) ---------------------------
  * The partition's rows, kNN graph / graph and map are device arrays holding only that partition (ids are

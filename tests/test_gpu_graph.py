@@ -129,6 +129,14 @@ def test_refine_bit_exact(hip, small_index, stages):
     st = stages["st_ref"]
     assert hip.read_counters(cntd) == [st["iterations"], st["rows_scored"], st["graph_rows"]]
     assert np.array_equal(g_in.numpy(), stages["rev"])      # input untouched
+    # the processing order (here: partition order, as the host layer passes it) does not change the result
+    g_out2 = hip.DeviceArray.full((n, 32), 0xDEADBEEF)
+    order = hip.DeviceArray.from_numpy(idx["map"][:n].astype(np.uint32))
+    assert np.array_equal(np.sort(idx["map"][:n]), np.arange(n))
+    hip.refine(data, n, dim, g_in, g_out2, 32, cent, idx["centroids"].shape[0], spd, sp["beam"], sp["max_iterations"],
+               sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 1.05, 0, order=order)
+    hip.synchronize()
+    assert np.array_equal(g_out2.numpy(), stages["ref"])
 
 
 def test_built_graph_is_searchable(hip, small_index, stages):
