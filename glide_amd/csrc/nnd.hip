@@ -23,7 +23,8 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 constexpr uint32_t kSamples = 32;     // NUM_SAMPLES (nn_descent.cuh:391)
 constexpr uint32_t kBi = 64;          // MAX_NUM_BI_SAMPLES (:392)
 constexpr uint32_t kOld = 0x80000000u;  // "old" flag in a list entry (the reference uses the sign bit, :53-72)
-constexpr int kRowHalfs = 128 + 8;    // LDS row stride in halfs for a 128-dim chunk
+constexpr int kJoinChunk = 64;         // dims staged per step of the join
+constexpr int kRowHalfs = kJoinChunk + 8;   // LDS row stride in halfs for one chunk
 constexpr int kDStride = 65;
 
 struct Segments {
@@ -229,12 +230,12 @@ __device__ __forceinline__ bool lds_set_insert(uint32_t* table, uint32_t key) { 
 // No filtering of offers against the target's current list: the reference also explores offers that do not enter
 // the list (they are the "new" samples of the next round, nn_descent.cuh:973-1001).
 
-// A (rows) x B (rows) dot products of a 128-dim chunk for this wave's 32 x 32 quadrant.
+// A (rows) x B (rows) dot products of one chunk of dims for this wave's 32 x 32 quadrant.
 // v_mfma_f32_32x32x16_f16 (gfx950): lane supplies A[i = lane%32][k = 8*(lane/32) .. +7] and B[k = same][j = lane%32].
 __device__ __forceinline__ void mfma_chunk(float16v& acc, const _Float16 (*A)[kRowHalfs], const _Float16 (*B)[kRowHalfs], int rb, int cb, int lane) {
     const int t = lane & 31, kh = lane >> 5;
 #pragma unroll
-    for (int kk = 0; kk < 128; kk += 16) {
+    for (int kk = 0; kk < kJoinChunk; kk += 16) {
         const half8v av = *reinterpret_cast<const half8v*>(&A[rb * 32 + t][kk + 8 * kh]);
         const half8v bv = *reinterpret_cast<const half8v*>(&B[cb * 32 + t][kk + 8 * kh]);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, acc, 0, 0, 0);
@@ -272,7 +273,9 @@ __device__ __forceinline__ void line_argmin(const float (*dist)[kDStride], uint3
     }
 }
 
-__global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
+// Six workgroups per CU (80 registers per lane, 20 KB of LDS each): the join is bound by the latency of its
+// gather -> matrix -> arg-min -> offer chain, so residency matters more than registers; seven would spill.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     JoinLds& L = *reinterpret_cast<JoinLds*>(smem);
     const uint32_t node = blockIdx.x;
@@ -326,25 +329,35 @@ __global__ __launch_bounds__(256) void nnd_join_kernel(JoinArgs a) {
     const bool need_nn = (rb * 32 < static_cast<int>(n_new)) && (cb * 32 < static_cast<int>(n_new));
     const bool need_no = (rb * 32 < static_cast<int>(n_new)) && (cb * 32 < static_cast<int>(n_old));
 
-    for (uint32_t k0 = 0; k0 < a.dim_pad; k0 += 128) {
-        if (k0) __syncthreads();
-        // gather: 16 lanes x 16 B per 128-dim chunk row, 16 rows per pass, new rows then old rows
+    // Chunks of kJoinChunk dims go global -> registers -> LDS: 8 lanes x 16 B per row and chunk, 32 rows per pass (new
+    // rows, then old rows).  The loads of chunk k+1 are issued before the matrix instructions of chunk k.  Short chunks
+    // keep the workgroup at 20 KB of LDS, so seven of them share a CU instead of four.
+    float4 pre[4];
+    auto prefetch = [&](uint32_t k0) {
 #pragma unroll
-        for (uint32_t r0 = 0; r0 < 128; r0 += 16) {
-            const uint32_t r = r0 + (tid >> 4), q = tid & 15;
+        for (int pass = 0; pass < 4; pass++) {
+            const uint32_t r = pass * 32 + (tid >> 3), q = tid & 7;
             const bool is_old = r >= 64;
             const uint32_t rr = r & 63;
-            const uint32_t n = is_old ? n_old : n_new;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             const uint32_t d0 = k0 + q * 8;
-            if (rr < n) {
+            pre[pass] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (rr < (is_old ? n_old : n_new)) {
                 const uint32_t id = (is_old ? L.old_ids : L.new_ids)[rr];
-                if (d0 < a.dim_pad) v = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
+                if (d0 < a.dim_pad) pre[pass] = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
                 if (k0 == 0 && q == 0) (is_old ? L.old_norms : L.new_norms)[rr] = a.norms[seg_start + id];   // same round trip as the row
             }
-            *reinterpret_cast<float4*>(&(is_old ? L.rows.xo : L.rows.xn)[rr][q * 8]) = v;
+        }
+    };
+    prefetch(0);
+    for (uint32_t k0 = 0; k0 < a.dim_pad; k0 += kJoinChunk) {
+        if (k0) __syncthreads();   // every wave is done with the previous chunk
+#pragma unroll
+        for (int pass = 0; pass < 4; pass++) {
+            const uint32_t r = pass * 32 + (tid >> 3), q = tid & 7;
+            *reinterpret_cast<float4*>(&(r >= 64 ? L.rows.xo : L.rows.xn)[r & 63][q * 8]) = pre[pass];
         }
         __syncthreads();
+        if (k0 + kJoinChunk < a.dim_pad) prefetch(k0 + kJoinChunk);
         if (need_nn) mfma_chunk(acc_nn, L.rows.xn, L.rows.xn, rb, cb, lane);
         if (need_no) mfma_chunk(acc_no, L.rows.xn, L.rows.xo, rb, cb, lane);
     }
