@@ -11,7 +11,6 @@
 // (one atomic counter per node, no locks, no cross-workgroup read-after-write inside a kernel) and a merge kernel
 // folds each inbox into the node's sorted list with a wave-wide bitonic sort; sampling uses the new/old flag kept
 // in the list instead of a host-side Bloom filter.  All ids are partition-local.
-#include <cstdlib>
 #include "common.hpp"
 #include "host_util.hpp"
 
@@ -193,7 +192,6 @@ struct JoinArgs {
     const uint32_t* rev_new;
     const uint32_t* rev_old;
     const uint32_t* counts;
-    const float* list_dists;    // thresholds: a node's current worst distance
     uint32_t* inbox_counts;
     uint2* inbox;               // num x inbox_cap (dist bits, id)
     unsigned long long* stats;  // [0] offers emitted, [1] offers dropped by a full inbox (nullable)
@@ -727,7 +725,7 @@ using namespace glide;
 
 namespace {
 uint32_t nnd_width(uint32_t degree) { return round_up32(static_cast<uint32_t>(degree * (degree <= 32 ? 1.0 : 1.3))); }  // nn_descent.cuh:1427-1428
-uint32_t nnd_inbox_cap(uint32_t width) { return (getenv("GLIDE_EXP_CAP512") ? 512 : 256) - width; }   // list + inbox fill one 256-element sort
+uint32_t nnd_inbox_cap(uint32_t width) { return 256 - width; }   // list + inbox fill one 256-element sort
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
 struct NndLayout {
@@ -839,7 +837,7 @@ int nnd_reverse(const NndCtx& c) {
 int nnd_join(const NndCtx& c) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
-    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.counts, c.list_dists, c.inbox_counts, c.inbox, c.stats,
+    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.counts, c.inbox_counts, c.inbox, c.stats,
                 c.n, c.l.dim_pad, c.l.width, c.l.cap, c.segs};
     hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja);
     return launch_status();
