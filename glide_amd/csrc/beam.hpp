@@ -31,6 +31,13 @@ struct BeamLds {  // per-wave LDS (the hash table follows, 1 << hash_bit words)
     uint32_t vlist[MAX_CAND];
 };
 
+// Host-side sizes of the dynamic LDS regions: the candidate lists for a degree bucket, and the staging area that the
+// two-half beam merge (beams above 256) keeps behind the hash table: 512 distances, 512 ids, two turning points.
+inline size_t beam_lds_bytes(uint32_t degree) {
+    return degree <= 64 ? sizeof(BeamLds<64>) : degree <= 128 ? sizeof(BeamLds<128>) : sizeof(BeamLds<256>);
+}
+inline size_t beam_stage_bytes(uint32_t beam) { return beam > 256 ? (2 * 512 + 4) * sizeof(uint32_t) : 0; }
+
 __device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
 
 // Distances from `ref` to `count` listed rows, RowShape<DIMV>::ROWS rows per step (one per lane group), U steps in
@@ -69,6 +76,9 @@ struct Beam {
     RowRegs<DIMV> q;
     BeamLds<MAX_CAND>* lds;
     uint32_t* hash;
+    float* stage_dist;       // MAX_BEAM > 256 only: LDS copy of the beam for the two-warp merge (follows the hash table)
+    uint32_t* stage_id;
+    uint32_t* stage_ws;
     BeamParams p;
     BeamCounters cnt;
     int lane;
@@ -79,6 +89,9 @@ struct Beam {
         hash = hash_;
         p = p_;
         lane = lane_id();
+        stage_dist = reinterpret_cast<float*>(hash_ + (size_t{1} << p_.hash_bit));
+        stage_id = reinterpret_cast<uint32_t*>(stage_dist + MAX_BEAM);
+        stage_ws = stage_id + MAX_BEAM;
         load_row<DIMV>(q, query, p.dim, RowShape<DIMV>::lane_in_row(lane));
         hash_clear(hash, p.hash_bit, lane);
         wave_sync();
@@ -115,11 +128,9 @@ struct Beam {
         wave_sync();
     }
 
-    // reference update_result_buffer: sort the candidates, then fold them into the beam
-    __device__ __forceinline__ void absorb(bool first) {
-        // No row scored: every candidate distance is FLT_MAX, the sort would not move anything (equal keys are never
-        // exchanged) and no candidate can displace a beam entry, so the beam stays as it is.
-        if (!first && last_scored == 0) return;
+    // Candidate sort, one network over the wavefront (reference sort_for_candidate, single-warp branch,
+    // search_kernel.cuh:9-37): strided load, sort, blocked store of every element.
+    __device__ __forceinline__ void sort_candidates_one() {
         float ck[NC];
         uint32_t cv[NC];
 #pragma unroll
@@ -139,6 +150,148 @@ struct Beam {
             lds->cand_id[e] = cv[r];
         }
         wave_sync();
+    }
+
+    // Candidate sort for more than 128 slots (reference two-warp branch, search_kernel.cuh:38-94): the two 32-lane
+    // halves of the wavefront are the two warps.  Each sorts its half of the slots, a half-cleaner across the halves
+    // leaves the smaller keys with half 0, each half merges.  Only slots below min(degree, beam) are defined afterwards.
+    __device__ __forceinline__ void sort_candidates_two() {
+        constexpr int PER = MAX_CAND / 2, N = PER / 32;
+        const uint32_t w = lane >> 5, l = lane & 31;
+        float key[N];
+        uint32_t val[N];
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const uint32_t j = l + 32 * i + PER * w;
+            key[i] = j < p.degree ? lds->cand_dist[j] : FLT_MAX;
+            val[i] = j < p.degree ? lds->cand_id[j] : kInvalid;
+        }
+        WaveNet<PER, 32>::sort(key, val, lane);
+        wave_sync();
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const uint32_t jl = N * l + i, j = jl + PER * w;
+            if (j < p.degree && jl < p.beam) {
+                lds->cand_dist[j] = key[i];
+                lds->cand_id[j] = val[i];
+            }
+        }
+        wave_sync();
+        const uint32_t warps_used = (p.beam + PER - 1) / PER;
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const uint32_t jl = N * l + i, kl = PER - 1 - jl, j = jl + PER * w, k = MAX_CAND - 1 - j;
+            if (w < warps_used && j < p.degree && k < p.degree && kl < p.beam) {
+                const float other = lds->cand_dist[k];
+                if (key[i] != other && ((w == 0) == (key[i] > other))) {
+                    key[i] = other;
+                    val[i] = lds->cand_id[k];
+                }
+            }
+        }
+        wave_sync();
+        WaveNet<PER, 32>::merge(key, val, lane);
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const uint32_t jl = N * l + i, j = jl + PER * w;
+            if (w < warps_used && j < p.degree && j < p.beam) {
+                lds->cand_dist[j] = key[i];
+                lds->cand_id[j] = val[i];
+            }
+        }
+        wave_sync();
+    }
+
+    // Beam merge for beams above 256 (reference two-warp branch of sort_for_beam, search_kernel.cuh:149-232), on a copy
+    // of the beam in LDS: candidates displace larger entries from the tail, the two halves are compare-exchanged
+    // element by element, the smallest touched index of each half is tracked, and each 32-lane half of the wavefront
+    // merges one half of the beam laid out as [untouched prefix | padding | touched rest].  Returns false when no
+    // candidate entered (the beam is unchanged).
+    __device__ __forceinline__ bool merge_beam_two() {
+        constexpr int PER = MAX_BEAM / 2, N = PER / 32;
+        float* sd = stage_dist;
+        uint32_t* si = stage_id;
+        const uint32_t half = p.beam / 2;
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            sd[NB * lane + r] = bk[r];
+            si[NB * lane + r] = bv[r];
+        }
+        if (lane < 3) stage_ws[lane] = half;
+        wave_sync();
+        bool replaced = false;
+        const uint32_t limit = p.degree < p.beam ? p.degree : p.beam;
+        for (uint32_t k = lane; k < limit; k += kWave) {
+            const uint32_t j = p.beam - 1 - k;
+            const float c = lds->cand_dist[k];
+            if (sd[j] > c) {
+                sd[j] = c;
+                si[j] = lds->cand_id[k];
+                if (j < half) atomicMin(&stage_ws[2], j);
+                else atomicMin(&stage_ws[1], j - half);
+                replaced = true;
+            }
+        }
+        if (ballot(replaced) == 0) return false;
+        wave_sync();
+        for (uint32_t j = lane; j < half; j += kWave) {
+            const uint32_t k = j + half;
+            const float k0 = sd[j], k1 = sd[k];
+            if (k0 > k1) {
+                sd[j] = k1;
+                sd[k] = k0;
+                const uint32_t v0 = si[j];
+                si[j] = si[k];
+                si[k] = v0;
+                atomicMin(&stage_ws[0], j);
+            }
+        }
+        wave_sync();
+        if (lane == 0 && stage_ws[2] < half) stage_ws[1] = stage_ws[2];
+        wave_sync();
+        const uint32_t w = lane >> 5, l = lane & 31;
+        const uint32_t turning = stage_ws[w];
+        float key[N];
+        uint32_t val[N];
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            uint32_t k = p.beam, j = N * l + i;
+            if (j < turning) {
+                k = j + half * w;
+            } else if (j >= PER - half) {
+                j -= PER - half;
+                if (turning <= j && j < half) k = j + half * w;
+            }
+            key[i] = k < p.beam ? sd[k] : FLT_MAX;
+            val[i] = k < p.beam ? si[k] : kInvalid;
+        }
+        wave_sync();
+        WaveNet<PER, 32>::merge(key, val, lane);
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const uint32_t j = N * l + i;
+            if (j < half) {
+                sd[j + half * w] = key[i];
+                si[j + half * w] = val[i];
+            }
+        }
+        wave_sync();
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t e = NB * lane + r;
+            bk[r] = e < p.beam ? sd[e] : FLT_MAX;
+            bv[r] = e < p.beam ? si[e] : kInvalid;
+        }
+        return true;
+    }
+
+    // reference update_result_buffer: sort the candidates, then fold them into the beam
+    __device__ __forceinline__ void absorb(bool first) {
+        // No row scored: every candidate distance is FLT_MAX, the sort would not move anything (equal keys are never
+        // exchanged) and no candidate can displace a beam entry, so the beam stays as it is.
+        if (!first && last_scored == 0) return;
+        if constexpr (MAX_CAND > 128) sort_candidates_two();
+        else sort_candidates_one();
         if (first) {
 #pragma unroll
             for (int r = 0; r < NB; r++) {
@@ -147,6 +300,8 @@ struct Beam {
                 bk[r] = take ? lds->cand_dist[e] : FLT_MAX;
                 bv[r] = take ? lds->cand_id[e] : kInvalid;
             }
+        } else if constexpr (MAX_BEAM > 256) {
+            merge_beam_two();
         } else {
             bool replaced = false;
 #pragma unroll

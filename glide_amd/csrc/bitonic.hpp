@@ -5,15 +5,18 @@
 // the element indices, not of the lane width, so the same comparator sequence is executed here with
 // e = NR*lane64 + r, NR = M/64 (M = 32 uses lanes 0..31 with NR = 1; lanes 32..63 run a private copy).
 // Same comparators in the same stage order => identical output sequence, ties included.
+// With LANES = 32 the two halves of the wavefront run two independent networks of M elements each (NR = M/32):
+// the reference's two-warp variants, one warp per half.
 #pragma once
 #include "common.hpp"
 
 namespace glide {
 
-template <int M>
+template <int M, int LANES = (M >= 64 ? 64 : 32)>
 struct WaveNet {
     static_assert(M == 32 || M == 64 || M == 128 || M == 256 || M == 512, "network size");
-    static constexpr int NR = M >= 64 ? M / 64 : 1;
+    static_assert((LANES == 64 || LANES == 32) && M >= LANES, "lanes per network");
+    static constexpr int NR = M / LANES;
 
     // compare-exchange of two registers of the same lane (bitonic.cuh:25-34)
     static __device__ __forceinline__ void cmpx_reg(float& k0, uint32_t& v0, float& k1, uint32_t& v1, bool asc) {
@@ -29,7 +32,7 @@ struct WaveNet {
         constexpr int LM = J / NR;
         uint64_t m = 0;
         for (int l = 0; l < 64; l++) {
-            const int e = NR * l + r;
+            const int e = NR * (l % LANES) + r;
             const bool asc = (K >= M) ? true : ((e & K) == 0);
             const bool lower = (l & LM) == 0;
             if (lower == asc) m |= 1ull << l;
@@ -60,7 +63,7 @@ struct WaveNet {
 #pragma unroll
             for (int r = 0; r < NR; r++) {
                 if ((r & J) == 0) {
-                    const int e = NR * lane + r;
+                    const int e = NR * (lane % LANES) + r;
                     const bool asc = (K >= M) ? true : ((e & K) == 0);
                     cmpx_reg(k[r], v[r], k[r | J], v[r | J], asc);
                 }

@@ -123,7 +123,7 @@ __global__ __launch_bounds__(64) void refine_kernel(RefineArgs a) {
     uint32_t* out_row = a.graph_out + static_cast<size_t>(point) * D;
 
     uint32_t need = 0;
-    for (uint32_t base = 0; base < 128; base += 64) {
+    for (uint32_t base = 0; base < kMaxDegree; base += 64) {
         const uint32_t i = base + lane;
         const uint32_t g = i < D ? in_row[i] : kInvalid;
         pl->s_graph[i] = g;
@@ -274,7 +274,8 @@ template <int MAX_CAND>
 build_fn pick_build_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_build_dim<MAX_CAND, 64>(dim);
     if (beam <= 128) return pick_build_dim<MAX_CAND, 128>(dim);
-    return pick_build_dim<MAX_CAND, 256>(dim);
+    if (beam <= 256) return pick_build_dim<MAX_CAND, 256>(dim);
+    return pick_build_dim<MAX_CAND, 512>(dim);
 }
 template <int MAX_CAND, int MAX_BEAM>
 refine_fn pick_refine_dim(uint32_t dim) {
@@ -287,26 +288,28 @@ template <int MAX_CAND>
 refine_fn pick_refine_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_refine_dim<MAX_CAND, 64>(dim);
     if (beam <= 128) return pick_refine_dim<MAX_CAND, 128>(dim);
-    return pick_refine_dim<MAX_CAND, 256>(dim);
+    if (beam <= 256) return pick_refine_dim<MAX_CAND, 256>(dim);
+    return pick_refine_dim<MAX_CAND, 512>(dim);
 }
 
 size_t prune_lds_bytes(uint32_t beam) {
-    return beam <= 64 ? sizeof(PruneLds<64>) : beam <= 128 ? sizeof(PruneLds<128>) : sizeof(PruneLds<256>);
+    return beam <= 64 ? sizeof(PruneLds<64>) : beam <= 128 ? sizeof(PruneLds<128>) : beam <= 256 ? sizeof(PruneLds<256>) : sizeof(PruneLds<512>);
 }
 
 int check_beam_sizes(uint32_t degree, uint32_t graph_degree, uint32_t beam, uint32_t dim, uint32_t hash_bit, int metric) {
     if (degree == 0 || graph_degree == 0 || beam == 0 || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
-    if (degree > 128 || graph_degree > 128 || beam > 256 || dim % 4 != 0 || dim > 1024 || hash_bit < 1 || hash_bit > 13)
+    if (degree > kMaxDegree || graph_degree > kMaxDegree || beam > 512 || dim % 4 != 0 || dim > 1024 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     return GLIDE_OK;
 }
 
 int launch_build(BuildArgs& a, hipStream_t stream) {
-    const uint32_t max_cand = a.p.degree <= 64 ? 64 : 128;
-    build_fn fn = max_cand == 64 ? pick_build_beam<64>(a.p.beam, a.p.dim) : pick_build_beam<128>(a.p.beam, a.p.dim);
-    const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) + prune_lds_bytes(a.p.beam) +
-                             (size_t{1} << a.p.hash_bit) * sizeof(uint32_t);
+    build_fn fn = a.p.degree <= 64 ? pick_build_beam<64>(a.p.beam, a.p.dim)
+                : a.p.degree <= 128 ? pick_build_beam<128>(a.p.beam, a.p.dim) : pick_build_beam<256>(a.p.beam, a.p.dim);
+    const size_t lds_bytes = beam_lds_bytes(a.p.degree) + prune_lds_bytes(a.p.beam) + (size_t{1} << a.p.hash_bit) * sizeof(uint32_t) +
+                             beam_stage_bytes(a.p.beam);
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(a.point_count), dim3(64), lds_bytes, stream, a);
     return launch_status();
 }
@@ -432,10 +435,11 @@ int glide_hip_refine_segment(const float* segment_data, uint32_t num, uint32_t d
     a.segment_start_point = start_point;
     a.relaxant = relaxant;
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
-    const uint32_t max_cand = graph_degree <= 64 ? 64 : 128;
-    refine_fn fn = max_cand == 64 ? pick_refine_beam<64>(beam, dim) : pick_refine_beam<128>(beam, dim);
-    const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) + prune_lds_bytes(beam) +
-                             (size_t{1} << hash_bit) * sizeof(uint32_t);
+    refine_fn fn = graph_degree <= 64 ? pick_refine_beam<64>(beam, dim)
+                 : graph_degree <= 128 ? pick_refine_beam<128>(beam, dim) : pick_refine_beam<256>(beam, dim);
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + prune_lds_bytes(beam) + (size_t{1} << hash_bit) * sizeof(uint32_t) +
+                             beam_stage_bytes(beam);
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }
@@ -509,10 +513,11 @@ int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32
     a.segment_start_point = 0;
     a.relaxant = relaxant;
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
-    const uint32_t max_cand = graph_degree <= 64 ? 64 : 128;
-    refine_fn fn = max_cand == 64 ? pick_refine_beam<64>(beam, dim) : pick_refine_beam<128>(beam, dim);
-    const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) + prune_lds_bytes(beam) +
-                             round_up32(centroid_num) * sizeof(float) + (size_t{1} << hash_bit) * sizeof(uint32_t);
+    refine_fn fn = graph_degree <= 64 ? pick_refine_beam<64>(beam, dim)
+                 : graph_degree <= 128 ? pick_refine_beam<128>(beam, dim) : pick_refine_beam<256>(beam, dim);
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + prune_lds_bytes(beam) + round_up32(centroid_num) * sizeof(float) +
+                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }

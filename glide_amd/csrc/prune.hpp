@@ -6,15 +6,17 @@
 
 namespace glide {
 
+constexpr uint32_t kMaxDegree = 256;   // largest graph / kNN degree (reference kernel_config.cuh:53-60)
+
 template <int MAX_BEAM>
 struct PruneLds {
     uint32_t pool_id[MAX_BEAM];
     float pool_dist[MAX_BEAM];
     uint32_t keep[MAX_BEAM];
-    uint32_t neighbor[128];   // round_up32(graph_degree) <= 128
-    uint32_t s_graph[128];
-    uint32_t fresh[128];
-    uint32_t dup_mask[4];
+    uint32_t neighbor[kMaxDegree];   // round_up32(graph_degree) <= kMaxDegree
+    uint32_t s_graph[kMaxDegree];
+    uint32_t fresh[kMaxDegree];
+    uint32_t dup_mask[kMaxDegree / 32];
 };
 
 // Beam registers -> LDS pool in rank order with the explored bit stripped (graph_kernel.cuh:65-67), dropping
@@ -76,7 +78,7 @@ template <int MAX_BEAM, int DIMV>
 __device__ __forceinline__ uint32_t prune_pool(PruneLds<MAX_BEAM>* pl, uint32_t pool_size, const float* data, uint32_t dim,
                                                uint32_t segment_start, uint32_t graph_degree, float relaxant, int metric,
                                                int lane, uint32_t& rows_scored) {
-    for (uint32_t i = lane; i < 128; i += 64) pl->neighbor[i] = kInvalid;
+    for (uint32_t i = lane; i < kMaxDegree; i += 64) pl->neighbor[i] = kInvalid;
     wave_sync();
     uint32_t nsize = 0;
     while (nsize < graph_degree && pool_size > 0) {
@@ -100,7 +102,7 @@ template <int MAX_BEAM, int DIMV>
 __device__ __forceinline__ uint32_t prune_pool_refine(PruneLds<MAX_BEAM>* pl, uint32_t pool_size, const float* data, uint32_t dim,
                                                       uint32_t self, uint32_t graph_degree, uint32_t need, float relaxant,
                                                       int metric, int lane, uint32_t& rows_scored) {
-    for (uint32_t i = lane; i < 128; i += 64) pl->neighbor[i] = kInvalid;
+    for (uint32_t i = lane; i < kMaxDegree; i += 64) pl->neighbor[i] = kInvalid;
     wave_sync();
     uint32_t nsize = 0;
     while (nsize < need && pool_size > 0) {
@@ -137,8 +139,8 @@ template <int MAX_BEAM>
 __device__ __forceinline__ void merge_boundary_row(PruneLds<MAX_BEAM>* pl, uint32_t* row, const uint32_t* map,
                                                    uint32_t graph_degree, int lane) {
     const uint32_t max_degree = round_up32(graph_degree);
-    for (uint32_t i = lane; i < 128; i += 64) pl->s_graph[i] = i < graph_degree ? row[i] : kInvalid;
-    if (lane < 4) pl->dup_mask[lane] = 0;
+    for (uint32_t i = lane; i < kMaxDegree; i += 64) pl->s_graph[i] = i < graph_degree ? row[i] : kInvalid;
+    if (lane < static_cast<int>(kMaxDegree / 32)) pl->dup_mask[lane] = 0;
     wave_sync();
     uint32_t nfresh = 0, ndup = 0;
     for (uint32_t base = 0; base < max_degree; base += 64) {

@@ -233,7 +233,8 @@ template <int MAX_CAND>
 sub_fn pick_sub_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_sub_dim<MAX_CAND, 64>(dim);
     if (beam <= 128) return pick_sub_dim<MAX_CAND, 128>(dim);
-    return pick_sub_dim<MAX_CAND, 256>(dim);
+    if (beam <= 256) return pick_sub_dim<MAX_CAND, 256>(dim);
+    return pick_sub_dim<MAX_CAND, 512>(dim);
 }
 
 template <int MAX_CAND, int MAX_BEAM>
@@ -247,7 +248,8 @@ template <int MAX_CAND>
 search_fn pick_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_dim<MAX_CAND, 64>(dim);
     if (beam <= 128) return pick_dim<MAX_CAND, 128>(dim);
-    return pick_dim<MAX_CAND, 256>(dim);
+    if (beam <= 256) return pick_dim<MAX_CAND, 256>(dim);
+    return pick_dim<MAX_CAND, 512>(dim);
 }
 
 // Grid size for the one-query-per-wavefront search kernel.  With small beams the kernel is bound by row gathers; when
@@ -282,7 +284,7 @@ extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, c
         return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0) return GLIDE_OK;
-    if (graph_degree > 128 || beam > 256 || centroid_num > 256 || dim % 4 != 0 || dim > 1024 || top_k > beam ||
+    if (graph_degree > 256 || beam > 512 || centroid_num > 256 || dim % 4 != 0 || dim > 1024 || top_k > beam ||
         hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     if (reinterpret_cast<uintptr_t>(data) % 16 || reinterpret_cast<uintptr_t>(queries) % 16 ||
@@ -312,10 +314,10 @@ extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, c
     a.p.min_iterations = min_iterations;
     a.p.metric = metric;
 
-    const uint32_t max_cand = graph_degree <= 64 ? 64 : 128;
-    search_fn fn = max_cand == 64 ? pick_beam<64>(beam, dim) : pick_beam<128>(beam, dim);
-    const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) +
-                             round_up32(centroid_num) * sizeof(float) + (size_t{1} << hash_bit) * sizeof(uint32_t);
+    search_fn fn = graph_degree <= 64 ? pick_beam<64>(beam, dim) : graph_degree <= 128 ? pick_beam<128>(beam, dim) : pick_beam<256>(beam, dim);
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + round_up32(centroid_num) * sizeof(float) +
+                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(balanced_grid(query_num, beam, lds_bytes)), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }
@@ -345,7 +347,7 @@ extern "C" int glide_hip_search_sub(const float* segment_data, uint32_t dim, con
     if (dim == 0 || graph_degree == 0 || centroid_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0) return GLIDE_OK;
-    if (graph_degree > 128 || beam > 256 || dim % 4 != 0 || dim > 1024 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
+    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 1024 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;   // top_k buckets: kernel_config.cuh:312-323
     SubArgs a;
     a.data = segment_data;
@@ -363,9 +365,9 @@ extern "C" int glide_hip_search_sub(const float* segment_data, uint32_t dim, con
     a.top_k = top_k;
     a.max_topk = top_k <= 32 ? 32 : (top_k <= 64 ? 64 : 128);
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
-    const uint32_t max_cand = graph_degree <= 64 ? 64 : 128;
-    sub_fn fn = max_cand == 64 ? pick_sub_beam<64>(beam, dim) : pick_sub_beam<128>(beam, dim);
-    const size_t lds_bytes = (max_cand == 64 ? sizeof(BeamLds<64>) : sizeof(BeamLds<128>)) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t);
+    sub_fn fn = graph_degree <= 64 ? pick_sub_beam<64>(beam, dim) : graph_degree <= 128 ? pick_sub_beam<128>(beam, dim) : pick_sub_beam<256>(beam, dim);
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(query_num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }

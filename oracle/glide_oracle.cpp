@@ -165,7 +165,7 @@ void sort_with_key_value(uint32_t max_number, uint32_t number, uint32_t *vals, f
 }
 
 // search_kernel.cuh:9-37 (single-warp branch)
-void sort_for_candidate(uint32_t max_cand, float *cd, uint32_t *ci, uint32_t degree, uint32_t beam) {
+void sort_for_candidate_1(uint32_t max_cand, float *cd, uint32_t *ci, uint32_t degree, uint32_t beam) {
     const uint32_t N = max_cand / 32;
     float k[256];
     uint32_t v[256];
@@ -183,9 +183,127 @@ void sort_for_candidate(uint32_t max_cand, float *cd, uint32_t *ci, uint32_t deg
         }
 }
 
+// search_kernel.cuh:38-94 (two-warp branch, taken when MAX_CANDIDATE > 128: every launch has at least 64 threads).
+// Each warp sorts its half of the slots; a half-cleaner across the halves leaves the smaller keys with warp 0 and the
+// larger with warp 1; each warp then merges its half.  Sequential restatement of the data-parallel steps (no step
+// reads a location another thread of the same step writes).
+void sort_for_candidate_2(uint32_t max_cand, float *cd, uint32_t *ci, uint32_t degree, uint32_t beam) {
+    const uint32_t per_warp = (max_cand + 1) / 2, N = (per_warp + 31) / 32;
+    float key[2][256];
+    uint32_t val[2][256];
+    for (uint32_t w = 0; w < 2; w++) {
+        for (uint32_t lane = 0; lane < 32; lane++)
+            for (uint32_t i = 0; i < N; i++) {
+                const uint32_t j = lane + 32 * i + per_warp * w;
+                key[w][N * lane + i] = j < degree ? cd[j] : FLT_MAX;
+                val[w][N * lane + i] = j < degree ? ci[j] : kInvalid;
+            }
+        warp_sort(key[w], val[w], N);
+    }
+    for (uint32_t w = 0; w < 2; w++)
+        for (uint32_t jl = 0; jl < 32 * N; jl++) {
+            const uint32_t j = jl + per_warp * w;
+            if (j < degree && jl < beam) {
+                cd[swz(j)] = key[w][jl];
+                ci[swz(j)] = val[w][jl];
+            }
+        }
+    const uint32_t warps_used = std::min<uint32_t>((beam + per_warp - 1) / per_warp, 2);
+    for (uint32_t w = 0; w < warps_used; w++)
+        for (uint32_t jl = 0; jl < 32 * N; jl++) {
+            const uint32_t kl = per_warp - 1 - jl, j = jl + per_warp * w, k = max_cand - 1 - j;
+            if (j >= degree || k >= degree || kl >= beam) continue;
+            const float other = cd[swz(k)];
+            if (key[w][jl] == other) continue;
+            if ((w == 0) == (key[w][jl] > other)) {
+                key[w][jl] = other;
+                val[w][jl] = ci[swz(k)];
+            }
+        }
+    for (uint32_t w = 0; w < warps_used; w++) warp_merge(key[w], val[w], N, 32);
+    for (uint32_t w = 0; w < warps_used; w++)
+        for (uint32_t jl = 0; jl < 32 * N; jl++) {
+            const uint32_t j = jl + per_warp * w;
+            if (j < degree && j < beam) {
+                cd[swz(j)] = key[w][jl];
+                ci[swz(j)] = val[w][jl];
+            }
+        }
+}
+
+void sort_for_candidate(uint32_t max_cand, float *cd, uint32_t *ci, uint32_t degree, uint32_t beam) {
+    if (max_cand > 128) sort_for_candidate_2(max_cand, cd, ci, degree, beam);
+    else sort_for_candidate_1(max_cand, cd, ci, degree, beam);
+}
+
+void sort_for_beam_1(uint32_t max_b, float *bd, uint32_t *bi, uint32_t beam, const float *cd, const uint32_t *ci, uint32_t degree,
+                     bool first);
+
+// search_kernel.cuh:149-232 (two-warp branch, taken when MAX_BEAM > 256).  In place on the beam buffer: candidates
+// displace larger beam entries from the tail, the two halves are compare-exchanged element by element, the smallest
+// touched index of each half ("turning point") is tracked, and each warp merges its half, laid out as
+// [untouched prefix | padding | touched rest] over MAX_BEAM / 2 slots.
+void sort_for_beam_2(uint32_t max_b, float *bd, uint32_t *bi, uint32_t beam, const float *cd, const uint32_t *ci, uint32_t degree,
+                     bool first) {
+    if (first) {
+        sort_for_beam_1(max_b, bd, bi, beam, cd, ci, degree, true);
+        return;
+    }
+    const uint32_t per_warp = (max_b + 1) / 2, N = (per_warp + 31) / 32, half = beam / 2;
+    uint32_t ws[3] = {half, half, half};
+    for (uint32_t k = 0; k < std::min(degree, beam); k++) {
+        const uint32_t j = beam - 1 - k;
+        if (bd[swz(j)] > cd[swz(k)]) {
+            bd[swz(j)] = cd[swz(k)];
+            bi[swz(j)] = ci[swz(k)];
+            if (j < half) ws[2] = std::min(ws[2], j);
+            else ws[1] = std::min(ws[1], j - half);
+        }
+    }
+    for (uint32_t j = 0; j < half; j++) {
+        const uint32_t k = j + half;
+        if (bd[swz(j)] > bd[swz(k)]) {
+            std::swap(bd[swz(j)], bd[swz(k)]);
+            std::swap(bi[swz(j)], bi[swz(k)]);
+            ws[0] = std::min(ws[0], j);
+        }
+    }
+    if (ws[2] < half) ws[1] = ws[2];
+    float key[2][256];
+    uint32_t val[2][256];
+    for (uint32_t w = 0; w < 2; w++) {
+        const uint32_t turning = ws[w];
+        for (uint32_t slot = 0; slot < 32 * N; slot++) {
+            uint32_t k = beam, j = slot;
+            if (j < turning) {
+                k = j + half * w;
+            } else if (j >= max_b / 2 - half) {
+                j -= max_b / 2 - half;
+                if (turning <= j && j < half) k = j + half * w;
+            }
+            key[w][slot] = k < beam ? bd[swz(k)] : FLT_MAX;
+            val[w][slot] = k < beam ? bi[swz(k)] : kInvalid;
+        }
+    }
+    for (uint32_t w = 0; w < 2; w++) {
+        warp_merge(key[w], val[w], N, 32);
+        for (uint32_t j = 0; j < 32 * N; j++)
+            if (j < half) {
+                bd[swz(j + half * w)] = key[w][j];
+                bi[swz(j + half * w)] = val[w][j];
+            }
+    }
+}
+
+void sort_for_beam(uint32_t max_b, float *bd, uint32_t *bi, uint32_t beam, const float *cd, const uint32_t *ci, uint32_t degree,
+                   bool first) {
+    if (max_b > 256) sort_for_beam_2(max_b, bd, bi, beam, cd, ci, degree, first);
+    else sort_for_beam_1(max_b, bd, bi, beam, cd, ci, degree, first);
+}
+
 // search_kernel.cuh:97-148 (single-warp branch)
-void sort_for_beam(uint32_t max_b, float *bd, uint32_t *bi, uint32_t beam, const float *cd, const uint32_t *ci,
-                   uint32_t degree, bool first) {
+void sort_for_beam_1(uint32_t max_b, float *bd, uint32_t *bi, uint32_t beam, const float *cd, const uint32_t *ci,
+                     uint32_t degree, bool first) {
     if (first) {
         for (uint32_t i = 0; i < beam; i++) {
             bd[swz(i)] = i < degree ? cd[swz(i)] : FLT_MAX;
@@ -340,8 +458,7 @@ bool make_cfg(SearchCfg &c, uint32_t beam, uint32_t degree, uint32_t max_iter, u
     c.metric = metric;
     c.max_cand = max_candidate(degree);
     c.max_b = max_beam(beam);
-    // single-warp sort variants only (reference switches to two-warp variants above these sizes)
-    if (c.max_cand == 0 || c.max_cand > 128 || c.max_b == 0 || c.max_b > 256) return false;
+    if (c.max_cand == 0 || c.max_b == 0) return false;
     if (beam == 0 || degree == 0 || hash_bit > 20) return false;
     return true;
 }

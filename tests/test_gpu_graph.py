@@ -148,3 +148,50 @@ def test_built_graph_is_searchable(hip, small_index, stages):
     sp = O.search_params(64, 32)
     ids, _, _ = run_gpu_search(hip, idx["data"], stages["ref"], idx["centroids"], idx["start_points"], idx["queries"], 10, sp)
     assert recall(ids, gt, 10) >= 0.95
+
+
+def test_wide_degree_and_beam_bit_exact(hip):
+    """Degree 160 with beams 320 (build) and 512 (refine): the candidate sort and the beam merge both run as two
+    half-wave networks (reference search_kernel.cuh:38-94, :149-232) and the prune tables hold up to 256 entries."""
+    from conftest import lowdim_data
+    from oracle import oracle as O
+    K = D = 160
+    n, c = 2500, 2
+    data = lowdim_data(n, 64, seed=11)
+    idx = O.build_index(data, c, graph_degree=32, knn_degree=32, nnd_iterations=2, refine_beam=0)
+    rdata = idx["reorder_data"]
+    rn = rdata.shape[0]
+    assert rn > n
+    knn = np.full((rn, K), INV, np.uint32)                     # exact neighbours inside each partition
+    for s, l in zip(idx["seg_start"].tolist(), idx["seg_len"].tolist()):
+        ids, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + l], min(K, l - 1), 0, exclude_self=True)
+        knn[s:s + l, :ids.shape[1]] = ids
+    idx = dict(idx, knn=knn, data=data)
+    sp = O.search_params(320, K)
+    e_sub, st_sub = O.build_subgraph(rdata, n, knn, idx["map"], idx["seg_start"], idx["seg_len"], idx["local_start_points"], D, sp, 1.05)
+    e_bnd, _ = O.build_boundary(rdata, n, knn, idx["map"], int(idx["local_start_points"][c]), e_sub.copy(), sp, 1.05)
+    e_rev = O.reverse_edges(e_bnd)
+    sp_ref = O.search_params(512, K)
+    e_ref, st_ref = O.refine(data, e_rev, idx["centroids"], idx["start_points"], sp_ref, 1.05)
+
+    print("wide build", sp, flush=True)
+    d, graph, cnt = gpu_build_sub(hip, idx, sp, D=D)
+    assert np.array_equal(graph.numpy(), e_sub)
+    assert hip.read_counters(cnt) == [st_sub["iterations"], st_sub["rows_scored"], st_sub["graph_rows"]]
+    print("wide boundary", flush=True)
+    hip.build_boundary(d["rdata"], n, rn, 64, d["knn"], K, d["map"], int(idx["local_start_points"][c]), D, sp["beam"],
+                       sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 1.05, 0, graph)
+    hip.synchronize()
+    assert np.array_equal(graph.numpy(), e_bnd)
+    print("wide reverse", flush=True)
+    assert np.array_equal(gpu_reverse(hip, e_bnd)[0], e_rev)
+    print("wide refine", sp_ref, flush=True)
+    g_in = hip.DeviceArray.from_numpy(e_rev, np.uint32)
+    g_out = hip.DeviceArray.full((n, D), 0xDEADBEEF)
+    cntd = hip.new_counters()
+    hip.refine(hip.DeviceArray.from_numpy(data, np.float32), n, 64, g_in, g_out, D, hip.DeviceArray.from_numpy(idx["centroids"], np.float32), c,
+               hip.DeviceArray.from_numpy(idx["start_points"], np.uint32), sp_ref["beam"], sp_ref["max_iterations"], sp_ref["min_iterations"],
+               sp_ref["hash_bit"], sp_ref["hash_reset_interval"], 1.05, 0, cntd)
+    hip.synchronize()
+    assert np.array_equal(g_out.numpy(), e_ref)
+    assert hip.read_counters(cntd) == [st_ref["iterations"], st_ref["rows_scored"], st_ref["graph_rows"]]

@@ -26,7 +26,7 @@ def run_gpu_search(hip, data, graph, centroids, start_points, queries, top_k, sp
     return ids.numpy(), dists.numpy(), (hip.read_counters(cnt) if counters else None)
 
 
-@pytest.mark.parametrize("beam,top_k", [(32, 10), (64, 10), (96, 32), (128, 10), (256, 100)])
+@pytest.mark.parametrize("beam,top_k", [(32, 10), (64, 10), (96, 32), (128, 10), (256, 100), (288, 10), (384, 100), (512, 10)])
 def test_search_bit_exact_on_integer_data(hip, small_index, beam, top_k):
     from oracle import oracle as O
     idx = small_index
@@ -98,12 +98,35 @@ def test_search_degree64_dim960(hip):
         assert np.array_equal(gids, eids) and np.array_equal(gdists, edists)
 
 
+@pytest.mark.parametrize("deg", [160, 256])
+def test_search_degree_above_128(hip, deg):
+    """Degrees above 128 sort the candidate list as two half-wave networks, beams above 256 merge the same way
+    (reference search_kernel.cuh:38-94 and :149-232); integer data, so ties between distinct ids are frequent."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(deg)
+    n, dim = 3000, 64
+    data = np.rint(rng.random((n, dim)) * 7).astype(np.float32)
+    queries = np.rint(rng.random((60, dim)) * 7).astype(np.float32)
+    graph = rng.integers(0, n, (n, deg)).astype(np.uint32)
+    graph[rng.random(graph.shape) < 0.1] = 0xFFFFFFFF
+    centroids = data[:8].copy()
+    start_points = rng.integers(0, n, 8).astype(np.uint32)
+    for beam in (64, 256, 320, 512):
+        sp = O.search_params(beam, deg)
+        args = (data, graph, centroids, start_points, queries, 10)
+        eids, edists, est = O.search(*args, **sp)
+        print("degree", deg, "beam", beam, sp, flush=True)
+        gids, gdists, gcnt = run_gpu_search(hip, *args, sp, counters=True)
+        assert np.array_equal(gids, eids) and np.array_equal(gdists, edists)
+        assert gcnt == [est["iterations"], est["rows_scored"], est["graph_rows"]]
+
+
 def test_search_rejects_unsupported_sizes(hip):
     d = hip.DeviceArray(4096, np.float32)
     base = dict(data=d, num=8, dim=128, graph=d, graph_degree=32, centroids=d, centroid_num=2, start_points=d, queries=d,
                 query_num=1, top_k=10, beam=64, max_iterations=10, min_iterations=0, hash_bit=8, hash_reset_interval=2,
                 metric=0, result_ids=d, result_dists=d)
-    for key, bad in (("beam", 512), ("graph_degree", 256), ("centroid_num", 300), ("dim", 130), ("top_k", 65)):
+    for key, bad in (("beam", 544), ("graph_degree", 257), ("centroid_num", 300), ("dim", 130), ("top_k", 65)):
         with pytest.raises(hip.GlideHipError) as e:
             hip.search(**{**base, key: bad})
         assert e.value.code == -1, key

@@ -173,3 +173,65 @@ def test_distance_cosine_identity_and_integer_exactness():
     exact = ((x.astype(np.int64) - y.astype(np.int64)) ** 2).sum(1)
     assert np.array_equal(O.distance_batch(x, y, O.COSINE), exact.astype(np.float32))  # sums stay below 2^24
     assert np.array_equal(O.distance_batch(x, y, O.EUCLIDEAN), np.sqrt(exact.astype(np.float64)).astype(np.float32))
+
+
+def _swz(j):
+    return j ^ (j >> 5)
+
+
+@pytest.mark.parametrize("max_cand,degree,beam", [(64, 32, 32), (64, 64, 200), (128, 96, 64), (128, 128, 300), (256, 160, 64),
+                                                  (256, 256, 100), (256, 200, 256), (256, 256, 512), (256, 130, 130)])
+def test_sort_for_candidate_selects_the_smallest(max_cand, degree, beam):
+    """Distinct keys: the first min(degree, beam) slots (swizzled) end up holding the smallest candidates in ascending
+    order, for the one-warp (search_kernel.cuh:9-37) and the two-warp (:38-94) variant alike."""
+    rng = np.random.default_rng(max_cand + degree + beam)
+    size = 1024
+    dist = np.full(size, np.float32(3e38))
+    ids = np.full(size, 0xFFFFFFFF, np.uint32)
+    dist[:degree] = rng.permutation(degree * 4)[:degree].astype(np.float32)
+    ids[:degree] = np.arange(degree) + 1000
+    d, i = O.sort_for_candidate(max_cand, dist, ids, degree, beam)
+    keep = min(degree, beam)
+    order = np.argsort(dist[:degree])[:keep]
+    got_d = np.array([d[_swz(j)] for j in range(keep)])
+    got_i = np.array([i[_swz(j)] for j in range(keep)])
+    np.testing.assert_array_equal(got_d, dist[:degree][order])
+    np.testing.assert_array_equal(got_i, ids[:degree][order])
+
+
+@pytest.mark.parametrize("max_beam,beam,degree", [(64, 64, 32), (128, 100, 64), (256, 256, 128), (256, 200, 32), (512, 512, 32),
+                                                  (512, 300, 64), (512, 400, 256), (512, 512, 256), (512, 258, 32)])
+def test_sort_for_beam_merges_to_the_smallest(max_beam, beam, degree):
+    """Distinct keys, even beam: the beam after the merge is the ascending list of the `beam` smallest of beam + candidates,
+    for the one-warp (search_kernel.cuh:97-148) and the two-warp (:149-232) variant alike; repeated over several rounds
+    so that the two-warp variant's turning points start from every kind of previous state."""
+    rng = np.random.default_rng(max_beam + beam + degree)
+    max_cand = 64 if degree <= 64 else 128 if degree <= 128 else 256
+    size = 2048
+    pool = rng.permutation(100000).astype(np.float32)
+    used = 0
+    bd = np.full(size, np.float32(3e38))
+    bi = np.full(size, 0xFFFFFFFF, np.uint32)
+    truth = []
+    for rnd in range(6):
+        n_valid = int(rng.integers(0, degree + 1))
+        cd = np.full(size, np.float32(3e38))
+        ci = np.full(size, 0xFFFFFFFF, np.uint32)
+        cd[:n_valid] = pool[used:used + n_valid] * (0.2 if rnd % 2 else 1.0)
+        ci[:n_valid] = np.arange(used, used + n_valid)
+        used += n_valid
+        cd[:n_valid] += np.arange(n_valid) * 1e-3 * 0          # keys stay distinct integers or fifths
+        # make keys distinct against everything seen so far
+        seen = {k for k, _ in truth}
+        for t in range(n_valid):
+            while float(cd[t]) in seen:
+                cd[t] += 0.5
+            seen.add(float(cd[t]))
+        cand = sorted(zip(cd[:n_valid].tolist(), ci[:n_valid].tolist()))
+        sd, si = O.sort_for_candidate(max_cand, cd, ci, degree, beam)
+        bd, bi = O.sort_for_beam(max_beam, bd, bi, beam, sd, si, degree, rnd == 0)
+        truth = sorted(truth + cand)[:beam] if rnd else cand[:beam]
+        got = [(float(bd[_swz(j)]), int(bi[_swz(j)])) for j in range(len(truth))]
+        assert got == [(float(np.float32(k)), v) for k, v in truth], (rnd, max_beam, beam, degree)
+        for j in range(len(truth), beam):
+            assert bd[_swz(j)] >= np.float32(3e38)
