@@ -11,6 +11,9 @@
  *   params                 hand-computed table + closed forms                       (pinned)
  *   bitonic sort / merge   distinct keys == std::sort, 0/1 principle on small M,
  *                          tie behaviour = literal comparator sequence of bitonic.cuh (pinned)
+ *   two-warp sort / merge  (degree > 128, beam > 256) distinct keys: the smallest `beam` keys in
+ *                          ascending order == std::sort (pinned); ties follow the reference's
+ *                          comparator and shared-memory sequence as written
  *   hashmap                hand-derived table layouts, set invariants               (pinned)
  *   distance               float64 closed form, rel <= 1e-5                         (pinned)
  *   partition assign       float64 brute-force argmin / ratio test                  (pinned)
