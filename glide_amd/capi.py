@@ -173,6 +173,16 @@ def search(data, num, dim, graph, graph_degree, centroids, centroid_num, start_p
                                  _ptr(counters), vp(stream)), "glide_hip_search")
 
 
+def search_merged(data, num, dim, graph, graph_degree, centroids, centroid_num, start_points, queries, query_num, top_k,
+                  beam, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric, result_ids, result_dists,
+                  counters=None, stream=None):
+    check(lib().glide_hip_search_merged(_ptr(data), u32(num), u32(dim), _ptr(graph), u32(graph_degree), _ptr(centroids),
+                                        u32(centroid_num), _ptr(start_points), _ptr(queries), u32(query_num), u32(top_k),
+                                        u32(beam), u32(max_iterations), u32(min_iterations), u32(hash_bit),
+                                        u32(hash_reset_interval), C.c_int(metric), _ptr(result_ids), _ptr(result_dists),
+                                        _ptr(counters), vp(stream)), "glide_hip_search_merged")
+
+
 def distance_batch(a, b, n, dim, metric, out, stream=None):
     check(lib().glide_hip_distance_batch(_ptr(a), _ptr(b), u32(n), u32(dim), C.c_int(metric), _ptr(out), vp(stream)),
           "glide_hip_distance_batch")
@@ -355,6 +365,16 @@ def build_segment(segment_data, num, dim, knn_graph, knn_degree, start_point, gr
                                         u32(start_point), u32(graph_degree), u32(beam), u32(max_iterations),
                                         u32(min_iterations), u32(hash_bit), u32(hash_reset_interval), f32(relaxant),
                                         C.c_int(metric), _ptr(graph), _ptr(counters), vp(stream)), "glide_hip_build_segment")
+
+
+def place_segment_graph(segment_graph, segment_length, graph_degree, segment_start, merged_graph, stream=None):
+    check(lib().glide_hip_place_segment_graph(_ptr(segment_graph), u32(segment_length), u32(graph_degree), u32(segment_start),
+                                              _ptr(merged_graph), vp(stream)), "glide_hip_place_segment_graph")
+
+
+def merge_boundary_graph(boundary_graph, boundary_num, graph_degree, home_rows, merged_graph, stream=None):
+    check(lib().glide_hip_merge_boundary_graph(_ptr(boundary_graph), u32(boundary_num), u32(graph_degree), _ptr(home_rows),
+                                               _ptr(merged_graph), vp(stream)), "glide_hip_merge_boundary_graph")
 
 
 def refine_segment(segment_data, num, dim, graph_in, graph_out, graph_degree, start_point, beam, max_iterations,

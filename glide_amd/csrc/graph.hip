@@ -259,6 +259,31 @@ __global__ __launch_bounds__(256) void insert_reverse_kernel(uint32_t* graph, co
     }
 }
 
+// ------------------------------------------------------------------------------------------ merged large build
+// A staged partition's sub-graph holds partition-local ids.  Its rows go to rows segment_start .. of the merged graph
+// with segment_start added to every id (what map_to_graph does through `map` on the small path,
+// graph_kernel.cuh:145-150; here the merged graph stays in reorder-id space, so the map is an offset).
+__global__ __launch_bounds__(256) void place_segment_kernel(const uint32_t* segment_graph, size_t words, uint32_t segment_start, uint32_t* merged) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= words) return;
+    const uint32_t v = segment_graph[i];
+    merged[i] = v == kInvalid ? kInvalid : v + segment_start;
+}
+
+// map_to_graph_boundary (graph_kernel.cuh:160-247) as a pass of its own: boundary copy i found the neighbours
+// boundary_graph[i] (ids local to the boundary segment); they are merged into the row of the point it is a copy of,
+// home_rows[i], every neighbour l being named by its own home row home_rows[l].  One wavefront per boundary copy.
+__global__ __launch_bounds__(64) void merge_boundary_kernel(const uint32_t* boundary_graph, uint32_t boundary_num, uint32_t D,
+                                                            const uint32_t* home_rows, uint32_t* merged) {
+    __shared__ PruneLds<64> pl;
+    const uint32_t i = blockIdx.x;
+    if (i >= boundary_num) return;
+    const int lane = lane_id();
+    for (uint32_t j = lane; j < kMaxDegree; j += 64) pl.neighbor[j] = j < D ? boundary_graph[static_cast<size_t>(i) * D + j] : kInvalid;
+    wave_sync();
+    merge_boundary_row<64>(&pl, merged + static_cast<size_t>(home_rows[i]) * D, home_rows, D, lane);
+}
+
 // ------------------------------------------------------------------------------------------ dispatch
 using build_fn = void (*)(BuildArgs);
 using refine_fn = void (*)(RefineArgs);
@@ -485,6 +510,27 @@ int glide_hip_insert_reverse(uint32_t* graph, const uint32_t* reverse_graph, con
     if (num == 0) return GLIDE_OK;
     hipLaunchKernelGGL(insert_reverse_kernel, dim3(ceil_div(num, 4)), dim3(256), 0, as_stream(stream), graph, reverse_graph,
                        reverse_counts, num, graph_degree);
+    return launch_status();
+}
+
+int glide_hip_place_segment_graph(const uint32_t* segment_graph, uint32_t segment_length, uint32_t graph_degree, uint32_t segment_start,
+                                  uint32_t* merged_graph, void* stream) {
+    if (!segment_graph || !merged_graph || graph_degree == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (segment_length == 0) return GLIDE_OK;
+    const size_t words = static_cast<size_t>(segment_length) * graph_degree;
+    uint32_t* dst = merged_graph + static_cast<size_t>(segment_start) * graph_degree;
+    hipLaunchKernelGGL(place_segment_kernel, dim3(static_cast<uint32_t>((words + 255) / 256)), dim3(256), 0, as_stream(stream), segment_graph, words,
+                       segment_start, dst);
+    return launch_status();
+}
+
+int glide_hip_merge_boundary_graph(const uint32_t* boundary_graph, uint32_t boundary_num, uint32_t graph_degree, const uint32_t* home_rows,
+                                   uint32_t* merged_graph, void* stream) {
+    if (!boundary_graph || !home_rows || !merged_graph || graph_degree == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (graph_degree > kMaxDegree) return GLIDE_ERR_UNSUPPORTED;
+    if (boundary_num == 0) return GLIDE_OK;
+    hipLaunchKernelGGL(merge_boundary_kernel, dim3(boundary_num), dim3(64), 0, as_stream(stream), boundary_graph, boundary_num, graph_degree,
+                       home_rows, merged_graph);
     return launch_status();
 }
 

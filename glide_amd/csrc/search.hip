@@ -273,12 +273,12 @@ uint32_t balanced_grid(uint32_t items, uint32_t beam, size_t lds_bytes) {
 
 using namespace glide;
 
-extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph, uint32_t graph_degree,
-                                const float* centroids, uint32_t centroid_num, const uint32_t* start_points,
-                                const float* queries, uint32_t query_num, uint32_t top_k, uint32_t beam,
-                                uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
-                                uint32_t hash_reset_interval, int metric, uint32_t* result_ids, float* result_dists,
-                                unsigned long long* counters, void* stream) {
+namespace {
+int launch_search(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph, uint32_t graph_degree, const float* centroids,
+                  uint32_t centroid_num, bool rank_all_centroids, const uint32_t* start_points, const float* queries, uint32_t query_num,
+                  uint32_t top_k, uint32_t beam, uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                  uint32_t hash_reset_interval, int metric, uint32_t* result_ids, float* result_dists, unsigned long long* counters,
+                  void* stream) {
     if (!data || !graph || !centroids || !start_points || !queries || !result_ids || !result_dists) return GLIDE_ERR_BAD_ARGUMENT;
     if (num == 0 || dim == 0 || graph_degree == 0 || centroid_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0)
         return GLIDE_ERR_BAD_ARGUMENT;
@@ -303,6 +303,7 @@ extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, c
     a.centroid_num = centroid_num;
     // reference kernel_config.cuh:161-171: bucket from graph_degree once there are more than 32 centroids
     a.max_centroid = centroid_num <= 32 ? 32 : (graph_degree <= 64 ? 64 : (graph_degree <= 128 ? 128 : 256));
+    if (rank_all_centroids) a.max_centroid = centroid_num <= 32 ? 32 : (centroid_num <= 64 ? 64 : (centroid_num <= 128 ? 128 : 256));
     a.top_k = top_k;
     a.query_num = query_num;
     a.p.beam = beam;
@@ -320,6 +321,27 @@ extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, c
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(balanced_grid(query_num, beam, lds_bytes)), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
+}
+}  // namespace
+
+extern "C" int glide_hip_search(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph, uint32_t graph_degree,
+                                const float* centroids, uint32_t centroid_num, const uint32_t* start_points,
+                                const float* queries, uint32_t query_num, uint32_t top_k, uint32_t beam,
+                                uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                                uint32_t hash_reset_interval, int metric, uint32_t* result_ids, float* result_dists,
+                                unsigned long long* counters, void* stream) {
+    return launch_search(data, num, dim, graph, graph_degree, centroids, centroid_num, false, start_points, queries, query_num, top_k, beam,
+                         max_iterations, min_iterations, hash_bit, hash_reset_interval, metric, result_ids, result_dists, counters, stream);
+}
+
+extern "C" int glide_hip_search_merged(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph, uint32_t graph_degree,
+                                       const float* centroids, uint32_t centroid_num, const uint32_t* start_points,
+                                       const float* queries, uint32_t query_num, uint32_t top_k, uint32_t beam,
+                                       uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                                       uint32_t hash_reset_interval, int metric, uint32_t* result_ids, float* result_dists,
+                                       unsigned long long* counters, void* stream) {
+    return launch_search(data, num, dim, graph, graph_degree, centroids, centroid_num, true, start_points, queries, query_num, top_k, beam,
+                         max_iterations, min_iterations, hash_bit, hash_reset_interval, metric, result_ids, result_dists, counters, stream);
 }
 
 extern "C" int glide_hip_select_segments(const float* queries, uint32_t query_num, uint32_t dim, const float* centroids, uint32_t centroid_num,

@@ -1,5 +1,7 @@
-// large_preprocess data_file preprocess_file result_file centroid_num sample_factor metric
-// Reference: large_preprocess.cu:21-80 (same argv and output files).  The rows may be uint8, as the reference reads them,
+// large_preprocess data_file preprocess_file result_file centroid_num sample_factor metric [boundary_factor]
+// Reference: large_preprocess.cu:21-80 (same argv and output files).  With the optional boundary_factor the
+// partitioning is made for a merged index (GLIDE_large::build_with_merge): the .segment file then holds one segment
+// more than there are centroids, the copies of the points close to a second partition, behind all points in .reorder.  The rows may be uint8, as the reference reads them,
 // or fp32; the element size is taken from the length of the data file.
 #include <cstdlib>
 #include <fstream>
@@ -29,9 +31,23 @@ static void run(device_resources& handle, PartitionParameter& param, const std::
     save_matrix_pinned(preprocess_file + ".reorder", h_reorder);
 }
 
+template <typename Data_t>
+static void run_merge(device_resources& handle, PartitionParameter& param, const std::string& data_file, const std::string& preprocess_file,
+                      std::string& result_file, uint32_t batch_num) {
+    auto h_data = load_matrix_pinned<Data_t>(data_file);
+    device_matrix<float> d_centroids(param.centroid_num, h_data.extent(1));
+    auto part = preprocess_for_large_merge<Data_t>(handle, param, h_data, d_centroids.view(), batch_num, result_file);
+    host_matrix<float> h_centroids(param.centroid_num, h_data.extent(1));
+    copy_to_host(h_centroids.data_handle(), d_centroids.data_handle(), h_centroids.size());
+    save_matrix_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view());
+    save_segment(preprocess_file + ".segment", std::as_const(part.h_segment_start).view(), std::as_const(part.h_segment_length).view());
+    save_vector_data(preprocess_file + ".map", std::as_const(part.h_map).view());
+    save_matrix_pinned(preprocess_file + ".reorder", part.h_reorder_data);
+}
+
 int main(int argc, char** argv) {
-    if (argc != 7) {
-        std::cout << argv[0] << " data_file preprocess_file result_file centroid_num sample_factor metric" << std::endl;
+    if (argc != 7 && argc != 8) {
+        std::cout << argv[0] << " data_file preprocess_file result_file centroid_num sample_factor metric [boundary_factor]" << std::endl;
         exit(-1);
     }
     device_resources handle(std::getenv("GLIDE_DEVICE") ? std::atoi(std::getenv("GLIDE_DEVICE")) : 0);
@@ -48,7 +64,14 @@ int main(int argc, char** argv) {
         std::ofstream result_out(result_file, std::ios::app);
         result_out << "pre_time,knn_time,degree,index_time,beam,search_time,QPS,recall" << std::endl;
     }
-    if (fbin_element_bytes(data_file) == 1) run<uint8_t>(handle, param, data_file, preprocess_file, result_file, batch_num);
-    else run<float>(handle, param, data_file, preprocess_file, result_file, batch_num);
+    const bool bytes = fbin_element_bytes(data_file) == 1;
+    if (argc == 8) {
+        param.boundary_factor = std::stof(argv[7]);
+        if (bytes) run_merge<uint8_t>(handle, param, data_file, preprocess_file, result_file, batch_num);
+        else run_merge<float>(handle, param, data_file, preprocess_file, result_file, batch_num);
+    } else {
+        if (bytes) run<uint8_t>(handle, param, data_file, preprocess_file, result_file, batch_num);
+        else run<float>(handle, param, data_file, preprocess_file, result_file, batch_num);
+    }
     return 0;
 }

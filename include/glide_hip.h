@@ -235,6 +235,33 @@ int glide_hip_refine(const float *data, uint32_t num, uint32_t dim, const uint32
  * partition-local); the caller stages them (the reference copies each partition from host memory,
  * glide_large_impl.cuh:109-166).  Data type: float (the reference's large executables instantiate uint8). */
 
+/* ---- merged large build (GLIDE_large::build_with_merge, declared at glide_large.cuh:89-97 without a definition) --
+ * The merged graph lives in device memory in reorder-id space: row r belongs to reorder row r (r < num) and holds
+ * reorder ids.  The two passes below are the large-path forms of map_to_graph (graph_kernel.cuh:145-150) and
+ * map_to_graph_boundary (graph_kernel.cuh:160-247), which the small path runs fused into its build kernels. */
+
+/* glide_hip_search on a merged large index.  The only difference: every centroid is ranked to pick the entry point
+ * (the bucket of the centroid sort comes from centroid_num), where glide_hip_search takes the bucket from
+ * graph_degree as the reference's small path does (kernel_config.cuh:161-171) and so ranks at most the first 64
+ * centroids of a degree-32 index; a large index has up to 256 partitions. */
+int glide_hip_search_merged(const float *data, uint32_t num, uint32_t dim, const uint32_t *graph, uint32_t graph_degree,
+                            const float *centroids, uint32_t centroid_num, const uint32_t *start_points,
+                            const float *queries, uint32_t query_num, uint32_t top_k, uint32_t beam,
+                            uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                            uint32_t hash_reset_interval, int metric, uint32_t *result_ids, float *result_dists,
+                            unsigned long long *counters, void *stream);
+
+/* Rows of one staged partition's sub-graph (partition-local ids, from glide_hip_build_segment) go to rows
+ * segment_start.. of the merged graph, every id shifted by segment_start; empty slots stay 0xffffffff. */
+int glide_hip_place_segment_graph(const uint32_t *segment_graph, uint32_t segment_length, uint32_t graph_degree,
+                                  uint32_t segment_start, uint32_t *merged_graph, void *stream);
+
+/* boundary_graph (boundary_num x graph_degree, ids local to the boundary segment) is the sub-graph built over the
+ * boundary copies.  Copy i is merged into merged_graph row home_rows[i] (the row of the point it duplicates) by the
+ * rule of map_to_graph_boundary, a neighbour l being entered as home_rows[l].  No two copies share a home row. */
+int glide_hip_merge_boundary_graph(const uint32_t *boundary_graph, uint32_t boundary_num, uint32_t graph_degree,
+                                   const uint32_t *home_rows, uint32_t *merged_graph, void *stream);
+
 /* Replaces build_for_large_kernel (graph_kernel.cuh:675-728; launch glide_large_impl.cuh:140): sub-graph of one
  * partition, rows written with partition-local ids. */
 int glide_hip_build_segment(const float *segment_data, uint32_t num, uint32_t dim, const uint32_t *knn_graph,

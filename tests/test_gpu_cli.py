@@ -140,6 +140,80 @@ def test_large_pipeline_cli(tmp_path):
     assert len(row) == 8
 
 
+def test_large_merged_pipeline_cli(tmp_path):
+    """large_* executables on a partitioning with a boundary segment: partitions built one by one, placed into one
+    graph, joined through the boundary copies, reverse edges over the whole graph (GLIDE_large::build_with_merge);
+    the merged index is searched resident in device memory.  Every stage against the oracle."""
+    from glide_amd import datasets as D
+    from oracle import oracle as O
+    n, dim, nq, c = 9003, 128, 200, 5
+    data, queries = lowdim_data(n, dim, seed=61), lowdim_data(nq, dim, seed=62)
+    truth, _ = O.bruteforce_knn(data, queries, 100)
+    f = lambda name: str(tmp_path / name)
+    D.write_fbin(f("base.fbin"), data)
+    D.write_fbin(f("query.fbin"), queries)
+    D.write_fbin(f("truth"), truth.astype(np.uint32))
+    pre, knn_file, graph_base, result = f("pre"), f("knn"), f("graph"), f("result.csv")
+
+    run(os.path.join(BIN, "large_preprocess"), f("base.fbin"), pre, result, c, 0.05, "Euclidean", 1.04)
+    centroids = D.read_fbin(pre + ".centroid")
+    starts, lengths = D.read_segment(pre + ".segment")
+    mp = D.read_vector(pre + ".map")
+    rdata = D.read_fbin(pre + ".reorder")
+    copies = int(lengths[c])
+    assert starts.size == c + 1 and lengths[:c].sum() == n and starts[c] == n and copies > 0
+    assert rdata.shape == (n + copies, dim) and mp.size == n + copies
+    assert np.array_equal(rdata, data[mp]) and np.array_equal(np.sort(mp[:n]), np.arange(n))
+    e_idx, e_len, near = O.partition_assign(data, centroids, 1.04)
+    ratio = near[:, 1] / near[:, 0]
+    if (np.abs(ratio - 1) > 1e-4).all() and (np.abs(ratio - 1.04) > 1e-4).all():   # no point on a border or on the threshold
+        assert np.array_equal(e_len, lengths)
+        e_rdata, e_map = O.reorder(data, e_idx, O.segment_starts(e_len), n + copies)
+        assert np.array_equal(e_map, mp) and np.array_equal(e_rdata, rdata)       # input order inside every segment
+
+    run(os.path.join(BIN, "large_knn"), pre, knn_file, result, 32)
+    knn = D.read_fbin(knn_file, np.uint32)
+    assert knn.shape == (n + copies, 32)
+    for s, l in zip(starts.tolist(), lengths.tolist()):
+        assert (knn[s:s + l] < l).all()
+
+    run(os.path.join(BIN, "large_build"), pre, knn_file, graph_base, result, "Euclidean", 32, 32, 1.05, 64, 128)
+    graph = D.read_fbin(graph_base + ".graph", np.uint32)
+    sp = D.read_vector(graph_base + ".sp")
+    assert graph.shape == (n, 32) and sp.size == c + 1
+    sp_b = O.search_params(64, 32)
+    INV = 0xFFFFFFFF
+    merged = np.full((n, 32), INV, np.uint32)
+    for i in range(c):
+        s, l = int(starts[i]), int(lengths[i])
+        g, _ = O.build_segment(rdata[s:s + l], knn[s:s + l], int(sp[i]), 32, sp_b, 1.05)
+        merged[s:s + l] = np.where(g == INV, INV, g + np.uint32(s))
+    row_of = np.empty(n, np.uint32)
+    row_of[mp[:n]] = np.arange(n, dtype=np.uint32)
+    home = row_of[mp[n:]]
+    assert np.unique(home).size == copies
+    gb, _ = O.build_segment(rdata[n:], knn[n:], int(sp[c]), 32, sp_b, 1.05)
+    before = merged.copy()
+    for i in range(copies):
+        merged[home[i]] = O.merge_boundary_row(merged[home[i]], gb[i], home)
+    assert (merged != before).any()
+    assert np.array_equal(graph, O.reverse_edges(merged))
+    # cross-partition edges exist only through the boundary copies
+    part_of = np.searchsorted(starts[1:c + 1], np.arange(n), side="right")
+    valid = graph != INV
+    cross = part_of[np.where(valid, graph, 0)] != part_of[:, None]
+    assert (cross & valid).any()
+
+    out = run(os.path.join(BIN, "large_search"), pre, f("query.fbin"), f("truth"), graph_base, result, "Euclidean", 10, 64, 2, 1.1)
+    recall = float(out.split("total_recall:")[1].split()[0])
+    entries = (starts[:c] + sp[:c]).astype(np.uint32)
+    e_ids, _, _ = O.search(rdata[:n], graph, centroids, entries, queries, 10, **O.search_params(64, 32))
+    e_ids = np.where(e_ids < n, mp[np.minimum(e_ids, n - 1)], e_ids)
+    assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= 0.95
+    row = open(result).read().strip().splitlines()[1].split(",")
+    assert len(row) == 8
+
+
 def test_large_pipeline_cli_uint8(tmp_path):
     """The reference's large executables read uint8 rows and uint8 queries (large_preprocess.cu:56, large_search.cu:111).
     Bytes are widened to fp32 on the GPU, so a uint8 run must reproduce the fp32 run on the same values: same

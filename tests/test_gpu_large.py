@@ -98,3 +98,82 @@ def test_search_over_partitions_bit_exact(hip, large_index, top_k, beam):
         assert np.array_equal(g_d.numpy(), e_d), s
     gt, _ = O.bruteforce_knn(L["data"], L["queries"], 10)
     assert recall(e_ids[:, :10], gt, 10) >= 0.9          # two partitions per query
+
+
+def test_place_and_merge_boundary_bit_exact(hip):
+    """The two passes of the merged large build against the oracle's row merge, on rows that take both of its
+    branches (at least half of the copy's neighbours already present / fewer) and on rows with empty slots."""
+    from oracle import oracle as O
+    INV = 0xFFFFFFFF
+    rng = np.random.default_rng(5)
+    for D in (32, 40, 64, 160):
+        n, copies, start = 500, 180, 1000
+        local = rng.integers(0, n, (n, D)).astype(np.uint32)
+        local[rng.random(local.shape) < 0.2] = INV
+        merged = hip.DeviceArray.full((start + n, D), 7)
+        hip.place_segment_graph(hip.DeviceArray.from_numpy(local), n, D, start, merged)
+        hip.synchronize()
+        got = merged.numpy()
+        assert (got[:start] == 7).all()
+        assert np.array_equal(got[start:], np.where(local == INV, INV, local + np.uint32(start)))
+
+        home = rng.permutation(n)[:copies].astype(np.uint32)
+        base = rng.integers(0, n, (n, D)).astype(np.uint32)
+        fill = rng.integers(D // 2, D + 1, n)                       # rows as pruning leaves them: filled from the front
+        base[np.arange(D)[None, :] >= fill[:, None]] = INV
+        bgraph = rng.integers(0, copies, (copies, D)).astype(np.uint32)
+        bgraph[rng.random(bgraph.shape) < 0.3] = INV
+        for i in range(0, copies, 3):       # many neighbours already in the row: the fill-the-holes branch
+            row = base[home[i]]
+            k = int(D * 0.7)
+            present = np.flatnonzero(np.isin(home, row[row != INV]))
+            if present.size:
+                bgraph[i, :k] = rng.choice(present, k).astype(np.uint32)
+        expect = base.copy()
+        branches = set()
+        for i in range(copies):
+            nb = bgraph[i]
+            dup = sum(1 for l in nb[nb != INV] if home[l] in expect[home[i]][:fill[home[i]]])
+            branches.add(bool(dup >= D // 2))
+            expect[home[i]] = O.merge_boundary_row(expect[home[i]], nb, home)
+        assert branches == {True, False}
+        d_base = hip.DeviceArray.from_numpy(base)
+        hip.merge_boundary_graph(hip.DeviceArray.from_numpy(bgraph), copies, D, hip.DeviceArray.from_numpy(home), d_base)
+        hip.synchronize()
+        assert np.array_equal(d_base.numpy(), expect), D
+
+
+def test_search_merged_ranks_every_centroid(hip):
+    """glide_hip_search_merged picks the entry among all centroids; glide_hip_search keeps the reference's bucket rule
+    (first 64 centroids of a degree-32 index).  Expected results: the oracle's search started from the exact nearest
+    centroid of each query."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(9)
+    n, dim, deg, c, nq = 4000, 64, 32, 100, 120
+    data = np.rint(rng.random((n, dim)) * 9).astype(np.float32)
+    queries = np.rint(rng.random((nq, dim)) * 9).astype(np.float32)
+    graph = rng.integers(0, n, (n, deg)).astype(np.uint32)
+    centroids = data[rng.permutation(n)[:c]].copy()
+    start_points = rng.integers(0, n, c).astype(np.uint32)
+    sp = O.search_params(64, deg)
+    d2 = ((queries[:, None, :] - centroids[None, :, :]) ** 2).sum(-1)     # small integers: exact in float32
+    order = np.lexsort((np.arange(c)[None, :].repeat(nq, 0), d2), axis=1)
+    nearest = order[:, 0]
+    unique_min = np.sort(d2, axis=1)[:, 0] != np.sort(d2, axis=1)[:, 1]
+    assert (nearest >= 64).any() and unique_min.sum() > nq // 2
+    e_ids = np.empty((nq, 10), np.uint32)
+    for q in range(nq):
+        ids, _, _ = O.search(data, graph, centroids[nearest[q]:nearest[q] + 1], start_points[nearest[q]:nearest[q] + 1], queries[q:q + 1], 10, **sp)
+        e_ids[q] = ids[0]
+    dev = lambda a, t: hip.DeviceArray.from_numpy(a, t)
+    ids, dists = hip.DeviceArray((nq, 10), np.uint32), hip.DeviceArray((nq, 10), np.float32)
+    args = (dev(data, np.float32), n, dim, dev(graph, np.uint32), deg, dev(centroids, np.float32), c, dev(start_points, np.uint32),
+            dev(queries, np.float32), nq, 10, sp["beam"], sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 0)
+    hip.search_merged(*args, ids, dists)
+    hip.synchronize()
+    assert np.array_equal(ids.numpy()[unique_min], e_ids[unique_min])
+    hip.search(*args, ids, dists)
+    hip.synchronize()
+    o_ids, _, _ = O.search(data, graph, centroids, start_points, queries, 10, **sp)
+    assert np.array_equal(ids.numpy(), o_ids)
+    assert (ids.numpy() != e_ids).any()
