@@ -250,6 +250,15 @@ def refine(data, num, dim, graph_in, graph_out, graph_degree, centroids, centroi
                                  f32(relaxant), C.c_int(metric), _ptr(order), _ptr(counters), vp(stream)), "glide_hip_refine")
 
 
+def refine_merged(data, num, dim, graph_in, graph_out, graph_degree, centroids, centroid_num, start_points, beam,
+           max_iterations, min_iterations, hash_bit, hash_reset_interval, relaxant, metric, counters=None,
+           stream=None, order=None):
+    check(lib().glide_hip_refine_merged(_ptr(data), u32(num), u32(dim), _ptr(graph_in), _ptr(graph_out), u32(graph_degree),
+                                 _ptr(centroids), u32(centroid_num), _ptr(start_points), u32(beam),
+                                 u32(max_iterations), u32(min_iterations), u32(hash_bit), u32(hash_reset_interval),
+                                 f32(relaxant), C.c_int(metric), _ptr(order), _ptr(counters), vp(stream)), "glide_hip_refine_merged")
+
+
 def _size_fn(name):
     f = getattr(lib(), name)
     f.restype = C.c_size_t

@@ -534,11 +534,13 @@ int glide_hip_merge_boundary_graph(const uint32_t* boundary_graph, uint32_t boun
     return launch_status();
 }
 
-int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph_in, uint32_t* graph_out,
-                     uint32_t graph_degree, const float* centroids, uint32_t centroid_num, const uint32_t* start_points,
-                     uint32_t beam, uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
-                     uint32_t hash_reset_interval, float relaxant, int metric, const uint32_t* order, unsigned long long* counters,
-                     void* stream) {
+}  // extern "C"
+
+namespace {
+int launch_refine(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph_in, uint32_t* graph_out, uint32_t graph_degree,
+                  const float* centroids, uint32_t centroid_num, bool rank_all_centroids, const uint32_t* start_points, uint32_t beam,
+                  uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant, int metric,
+                  const uint32_t* order, unsigned long long* counters, void* stream) {
     if (!data || !graph_in || !graph_out || !centroids || !start_points || graph_in == graph_out) return GLIDE_ERR_BAD_ARGUMENT;
     if (max_iterations == 0 || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
     int rc = check_beam_sizes(graph_degree, graph_degree, beam, dim, hash_bit, metric);
@@ -556,6 +558,7 @@ int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32
     a.num = num;
     a.centroid_num = centroid_num;
     a.max_centroid = centroid_num <= 32 ? 32 : (graph_degree <= 64 ? 64 : (graph_degree <= 128 ? 128 : 256));
+    if (rank_all_centroids) a.max_centroid = centroid_num <= 32 ? 32 : (centroid_num <= 64 ? 64 : (centroid_num <= 128 ? 128 : 256));
     a.segment_start_point = 0;
     a.relaxant = relaxant;
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
@@ -567,5 +570,22 @@ int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32
     hipLaunchKernelGGL(fn, dim3(num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }
+}  // namespace
 
-}  // extern "C"
+extern "C" int glide_hip_refine(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph_in, uint32_t* graph_out,
+                                uint32_t graph_degree, const float* centroids, uint32_t centroid_num, const uint32_t* start_points,
+                                uint32_t beam, uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                                uint32_t hash_reset_interval, float relaxant, int metric, const uint32_t* order,
+                                unsigned long long* counters, void* stream) {
+    return launch_refine(data, num, dim, graph_in, graph_out, graph_degree, centroids, centroid_num, false, start_points, beam, max_iterations,
+                         min_iterations, hash_bit, hash_reset_interval, relaxant, metric, order, counters, stream);
+}
+
+extern "C" int glide_hip_refine_merged(const float* data, uint32_t num, uint32_t dim, const uint32_t* graph_in, uint32_t* graph_out,
+                                       uint32_t graph_degree, const float* centroids, uint32_t centroid_num, const uint32_t* start_points,
+                                       uint32_t beam, uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                                       uint32_t hash_reset_interval, float relaxant, int metric, const uint32_t* order,
+                                       unsigned long long* counters, void* stream) {
+    return launch_refine(data, num, dim, graph_in, graph_out, graph_degree, centroids, centroid_num, true, start_points, beam, max_iterations,
+                         min_iterations, hash_bit, hash_reset_interval, relaxant, metric, order, counters, stream);
+}

@@ -132,6 +132,16 @@ public:
     // graph (glide_impl.cuh:194-256).  No refinement pass: the declaration takes no refine parameter.
     void build_with_merge(IndexParameter& build_param, SearchParameter& search_param_knn, const pinned_matrix<uint32_t>& h_knn_graph,
                           std::string& result_file) {
+        SearchParameter no_refine;
+        no_refine.beam = 0;
+        build_with_merge(build_param, search_param_knn, no_refine, h_knn_graph, result_file);
+    }
+
+    // The same with the small path's last stage (refine_kernel, glide_impl.cuh:258-316) when search_param_refine.beam != 0:
+    // all rows are then uploaded next to the merged graph (50M x 128 fp32 = 25.6 GB of the 288 GB) and rows with empty
+    // slots are completed by a search over the whole graph.
+    void build_with_merge(IndexParameter& build_param, SearchParameter& search_param_knn, SearchParameter& search_param_refine,
+                          const pinned_matrix<uint32_t>& h_knn_graph, std::string& result_file) {
         if (!merged()) throw std::invalid_argument("build_with_merge: the partitioning has no boundary segment");
         std::mt19937 generator(build_param.seed);
         for (uint32_t i = 0; i < segment_num(); i++) {
@@ -196,7 +206,28 @@ public:
         hip_try(glide_hip_reverse_edges(d_merged.data_handle(), n, deg, d_rev.data_handle(), d_rev_count.data_handle(), ws.get(), wb, cs),
                 "glide_hip_reverse_edges");
         hip_try(glide_hip_insert_reverse(d_merged.data_handle(), d_rev.data_handle(), d_rev_count.data_handle(), n, deg, cs), "glide_hip_insert_reverse");
-        hip_try(glide_hip_memcpy_d2h_async(h_graph.data_handle(), d_merged.data_handle(), d_merged.size() * sizeof(uint32_t), cs), "d2h graph");
+        const uint32_t* result = d_merged.data_handle();
+        std::optional<device_matrix<float>> d_rows, d_centroids;
+        std::optional<device_vector<uint32_t>> d_entries;
+        std::optional<staged_rows<Data_t>> slot;
+        if (search_param_refine.beam != 0) {
+            SearchParameter& r = search_param_refine;
+            d_rows.emplace(n, dim());
+            slot.emplace(sizeof(Data_t) == 1 ? upload_piece(n) : 1, dim());
+            upload_rows(d_rows->data_handle(), *slot, cs);
+            d_centroids.emplace(c, dim());
+            d_entries.emplace(c);
+            std::vector<uint32_t> entry(c);
+            for (uint32_t s = 0; s < c; s++) entry[s] = h_segment_start(s) + h_start_point(s);
+            hip_try(glide_hip_memcpy_h2d(d_centroids->data_handle(), h_centroids.data_handle(), h_centroids.size() * sizeof(float), cs), "h2d centroids");
+            hip_try(glide_hip_memcpy_h2d(d_entries->data_handle(), entry.data(), c * sizeof(uint32_t), cs), "h2d entries");
+            hip_try(glide_hip_refine_merged(d_rows->data_handle(), n, dim(), d_merged.data_handle(), d_rev.data_handle(), deg,
+                                            d_centroids->data_handle(), c, d_entries->data_handle(), r.beam, r.max_iterations, r.min_iterations,
+                                            r.hash_bit, r.hash_reset_interval, build_param.relaxant_factor, mc, nullptr, nullptr, cs),
+                    "glide_hip_refine_merged");
+            result = d_rev.data_handle();
+        }
+        hip_try(glide_hip_memcpy_d2h_async(h_graph.data_handle(), result, d_merged.size() * sizeof(uint32_t), cs), "d2h graph");
         hip_try(glide_hip_event_record(t1, cs), "glide_hip_event_record");
         st.sync();
         float ms = 0.f;
@@ -295,11 +326,17 @@ public:
     void search_merged(SearchParameter& param, device_matrix_view<Data_t> d_query_view, host_matrix_view<uint32_t> h_result_ids_view,
                        host_matrix_view<float> h_result_distances_view, std::string& result_file) {
         const uint32_t query_number = d_query_view.extent(0), top_k = param.top_k, deg = graph_degree(), c = centroids_num(), n = point_num();
-        make_resident();
+        const bool first_use = make_resident();
         device_matrix<uint32_t> d_ids(query_number, top_k);
         device_matrix<float> d_dists(query_number, top_k);
         device_matrix<float> d_query_f32(sizeof(Data_t) == 1 ? query_number : 0, dim());
         const float* d_queries = reinterpret_cast<const float*>(d_query_view.data_handle());
+        if (first_use && query_number)   // part of bringing the index up: the first launch of a kernel loads its code
+            hip_try(glide_hip_search_merged(r_data->data_handle(), n, dim(), r_graph->data_handle(), deg, r_centroids->data_handle(), c,
+                                            r_start_points->data_handle(), r_data->data_handle(), 1, top_k, param.beam, param.max_iterations,
+                                            param.min_iterations, param.hash_bit, param.hash_reset_interval, metric_code(metric),
+                                            d_ids.data_handle(), d_dists.data_handle(), nullptr, handle.stream()),
+                    "glide_hip_search_merged");
         gpu_timer timer;
         timer.start();
         if (sizeof(Data_t) == 1) {
@@ -329,26 +366,37 @@ public:
     }
 
 private:
-    // one-time upload of a merged index (rows in pieces through a staging slot, so uint8 rows cross PCIe as bytes)
-    void make_resident() {
-        if (r_data) return;
+    static uint32_t upload_piece(uint32_t n) { return std::min<uint32_t>(n, 1u << 20); }
+
+    // rows [0, point_num()) to device memory as fp32, in stream order (uint8 rows cross PCIe as bytes, one piece at a
+    // time through `slot`, and are widened on the GPU)
+    void upload_rows(float* dst_rows, staged_rows<Data_t>& slot, void* stream) {
+        const uint32_t n = point_num(), piece = upload_piece(n);
+        for (uint32_t first = 0; first < n; first += piece) {
+            const uint32_t count = std::min(piece, n - first);
+            float* dst = dst_rows + static_cast<size_t>(first) * dim();
+            if (sizeof(Data_t) == 1) {
+                slot.upload_async(h_data.row(first), count, stream);
+                hip_try(glide_hip_widen_u8(reinterpret_cast<const unsigned char*>(slot.stored()), static_cast<size_t>(count) * dim(), dst, stream),
+                        "glide_hip_widen_u8");
+            } else {
+                hip_try(glide_hip_memcpy_h2d_async(dst, h_data.row(first), static_cast<size_t>(count) * dim() * sizeof(float), stream),
+                        "glide_hip_memcpy_h2d_async");
+            }
+        }
+    }
+
+    // one-time upload of a merged index
+    bool make_resident() {
+        if (r_data) return false;
         const uint32_t n = point_num(), c = centroids_num(), deg = graph_degree();
         gpu_timer timer;
         timer.start();
         r_data.emplace(n, dim());
-        const uint32_t piece = std::min<uint32_t>(n, 1u << 20);
-        staged_rows<Data_t> slot(sizeof(Data_t) == 1 ? piece : 1, dim());
-        for (uint32_t first = 0; first < n; first += piece) {
-            const uint32_t count = std::min(piece, n - first);
-            float* dst = r_data->data_handle() + static_cast<size_t>(first) * dim();
-            if (sizeof(Data_t) == 1) {
-                copy_to_device(slot.stored(), h_data.row(first), static_cast<size_t>(count) * dim());
-                hip_try(glide_hip_widen_u8(reinterpret_cast<const unsigned char*>(slot.stored()), static_cast<size_t>(count) * dim(), dst, handle.stream()),
-                        "glide_hip_widen_u8");
-                handle.sync();
-            } else {
-                copy_to_device(dst, reinterpret_cast<const float*>(h_data.row(first)), static_cast<size_t>(count) * dim());
-            }
+        {
+            staged_rows<Data_t> slot(sizeof(Data_t) == 1 ? upload_piece(n) : 1, dim());
+            upload_rows(r_data->data_handle(), slot, handle.stream());
+            handle.sync();
         }
         r_graph.emplace(n, deg);
         copy_to_device(r_graph->data_handle(), h_graph.data_handle(), h_graph.size());
@@ -359,6 +407,7 @@ private:
         r_start_points.emplace(c);
         copy_to_device(r_start_points->data_handle(), entry.data(), c);
         std::cout << "index upload time: " << timer.stop() << " s" << std::endl;
+        return true;
     }
 
     std::optional<device_matrix<float>> r_data;

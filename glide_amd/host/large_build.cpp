@@ -1,6 +1,6 @@
 // large_build preprocess_file knn_file graph_base_file result_file metric graph_degree knn_degree relaxant_factor beam refine_beam
 // Reference: large_build.cu:24-95.  A partitioning that carries a boundary segment (large_preprocess with a
-// boundary_factor) is built with GLIDE_large::build_with_merge; refine_beam is then unused.
+// boundary_factor) is built with GLIDE_large::build_with_merge.
 #include <cstdlib>
 #include <fstream>
 #include <iostream>
@@ -44,7 +44,7 @@ int main(int argc, char** argv) {
     auto run = [&](auto tag) {   // uint8 rows as in the reference (large_build.cu:84) or fp32 rows, by the length of the .reorder file
         using Data_t = decltype(tag);
         GLIDE_large<Data_t, uint64_t> index(handle, build_param.graph_degree, build_param.metric, reorder_file, map_file, centroid_file, segment_file);
-        if (index.merged()) index.build_with_merge(build_param, search_param_knn, h_knn_graph, result_file);
+        if (index.merged()) index.build_with_merge(build_param, search_param_knn, search_param_refine, h_knn_graph, result_file);
         else index.build(build_param, search_param_knn, search_param_refine, h_knn_graph, result_file);
         save_matrix_pinned(graph_base_file + ".graph", index.graph_view());
         save_vector_data(graph_base_file + ".sp", index.start_point_view());

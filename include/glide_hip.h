@@ -251,6 +251,14 @@ int glide_hip_search_merged(const float *data, uint32_t num, uint32_t dim, const
                             uint32_t hash_reset_interval, int metric, uint32_t *result_ids, float *result_dists,
                             unsigned long long *counters, void *stream);
 
+/* glide_hip_refine on a merged large graph: as glide_hip_refine, every centroid ranked for the entry point (see
+ * glide_hip_search_merged). */
+int glide_hip_refine_merged(const float *data, uint32_t num, uint32_t dim, const uint32_t *graph_in, uint32_t *graph_out,
+                            uint32_t graph_degree, const float *centroids, uint32_t centroid_num,
+                            const uint32_t *start_points, uint32_t beam, uint32_t max_iterations,
+                            uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, float relaxant,
+                            int metric, const uint32_t *order, unsigned long long *counters, void *stream);
+
 /* Rows of one staged partition's sub-graph (partition-local ids, from glide_hip_build_segment) go to rows
  * segment_start.. of the merged graph, every id shifted by segment_start; empty slots stay 0xffffffff. */
 int glide_hip_place_segment_graph(const uint32_t *segment_graph, uint32_t segment_length, uint32_t graph_degree,

@@ -142,7 +142,8 @@ def test_large_pipeline_cli(tmp_path):
 
 def test_large_merged_pipeline_cli(tmp_path):
     """large_* executables on a partitioning with a boundary segment: partitions built one by one, placed into one
-    graph, joined through the boundary copies, reverse edges over the whole graph (GLIDE_large::build_with_merge);
+    graph, joined through the boundary copies, reverse edges and refinement over the whole graph
+    (GLIDE_large::build_with_merge);
     the merged index is searched resident in device memory.  Every stage against the oracle."""
     from glide_amd import datasets as D
     from oracle import oracle as O
@@ -197,7 +198,12 @@ def test_large_merged_pipeline_cli(tmp_path):
     for i in range(copies):
         merged[home[i]] = O.merge_boundary_row(merged[home[i]], gb[i], home)
     assert (merged != before).any()
-    assert np.array_equal(graph, O.reverse_edges(merged))
+    entries = (starts[:c] + sp[:c]).astype(np.uint32)
+    rev = O.reverse_edges(merged)
+    expect, _ = O.refine(rdata[:n], rev, centroids, entries, O.search_params(128, 32), 1.05)
+    assert (rev == INV).any() and np.array_equal(graph, expect)
+    run(os.path.join(BIN, "large_build"), pre, knn_file, f("graph0"), f("result0.csv"), "Euclidean", 32, 32, 1.05, 64, 0)
+    assert np.array_equal(D.read_fbin(f("graph0") + ".graph", np.uint32), rev)       # refine_beam 0: no refinement pass
     # cross-partition edges exist only through the boundary copies
     part_of = np.searchsorted(starts[1:c + 1], np.arange(n), side="right")
     valid = graph != INV
@@ -206,7 +212,6 @@ def test_large_merged_pipeline_cli(tmp_path):
 
     out = run(os.path.join(BIN, "large_search"), pre, f("query.fbin"), f("truth"), graph_base, result, "Euclidean", 10, 64, 2, 1.1)
     recall = float(out.split("total_recall:")[1].split()[0])
-    entries = (starts[:c] + sp[:c]).astype(np.uint32)
     e_ids, _, _ = O.search(rdata[:n], graph, centroids, entries, queries, 10, **O.search_params(64, 32))
     e_ids = np.where(e_ids < n, mp[np.minimum(e_ids, n - 1)], e_ids)
     assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= 0.95
