@@ -196,8 +196,30 @@ def run_workload(args, workload, torch, want_cpu):
     kernel_ms = gpu_ms / args.steps
     achieved = chosen["algorithmic_bytes"] / (kernel_ms * 1e-3) / 1e9
 
+    # ---- the build kernels against their own rooflines: algorithmic bytes (from the kernels' counters: graph rows read
+    # and data rows scored, prune rows included) or flops over the stage's GPU time
+    det = {**res["pre_stages"], **res["build_stages"]}
+    reorder_rows = int(h_len.sum())
+
+    def hbm_stage(seconds, nbytes):
+        gbs = nbytes / seconds / 1e9 if seconds > 0 else 0.0
+        return dict(bound="hbm", seconds=seconds, algorithmic_bytes=int(nbytes), achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS)
+
+    stage_rooflines = {}
+    assign_flops = 2.0 * num * parts * dim
+    stage_rooflines["assign"] = dict(hbm_stage(det["assign"], num * dim * 4 + num * 12),
+                                     mfma_tflops=assign_flops / det["assign"] / 1e12 if det["assign"] > 0 else 0.0, mfma_peak_tflops=157.3)
+    stage_rooflines["reorder"] = hbm_stage(det["reorder"], (num + reorder_rows) * dim * 4)
+    if "build_counters" in res:
+        _, rows, grows = res["build_counters"]
+        stage_rooflines["subgraph+boundary"] = hbm_stage(det["subgraph"] + det["boundary"],
+                                                         reorder_rows * dim * 4 + grows * knn_degree * 4 + rows * dim * 4 + reorder_rows * degree * 4)
+    if "refine_counters" in res:
+        _, rows, grows = res["refine_counters"]
+        stage_rooflines["refine"] = hbm_stage(det["refine"], num * dim * 4 + 2 * num * degree * 4 + grows * degree * 4 + rows * dim * 4)
+
     out = dict(
-        workload=desc, gen_sec=gen_s, build_sec=build_sec,
+        workload=desc, gen_sec=gen_s, build_sec=build_sec, stage_rooflines=stage_rooflines,
         build_stages=dict(pre=res["pre_time"], knn=res["knn_time"], index=res["index_time"], refine=res["refine_time"],
                           detail={**res["pre_stages"], **res["build_stages"]}),
         nnd_iterations=nnd_iters, nnd_offers=res["nnd_stats"][0], nnd_offers_dropped=res["nnd_stats"][1],
@@ -207,7 +229,8 @@ def run_workload(args, workload, torch, want_cpu):
         qps=nq * args.steps / (wall_ms * 1e-3), ms_per_step=ms_per_step, kernel_ms=kernel_ms,
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=MEASURED_TRAFFIC_BYTES.get((workload, chosen["beam"])),
-                      kernel="search_kernel<%d,%d,%d>" % (64 if degree <= 64 else 128, 64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256,
+                      kernel="search_kernel<%d,%d,%d>" % (64 if degree <= 64 else 128 if degree <= 128 else 256,
+                                                          64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256 if chosen["beam"] <= 256 else 512,
                                                           1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8),
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )
@@ -310,14 +333,14 @@ def main():
         "device": info["name"],
     }
     for k in ("build_sec", "build_stages", "graph_recall_at_32", "graph_recall_at_32_global", "recall_at_10", "recall_target_met",
-              "empty_slots_fraction", "sweep", "kernel_ms", "nnd_offers", "nnd_offers_dropped", "roofline"):
+              "empty_slots_fraction", "sweep", "kernel_ms", "nnd_offers", "nnd_offers_dropped", "stage_rooflines", "roofline"):
         line[k] = main_res[k]
     if "cpu_baseline" in main_res:
         line["cpu_baseline"] = main_res["cpu_baseline"]
     if args.workload == "cfg1" and not args.no_navigable:
         nav = run_workload(args, "cfg1-navigable", torch, want_cpu=False)
         line["navigable_variant"] = {k: nav[k] for k in ("workload", "build_sec", "build_stages", "graph_recall_at_32", "beam", "recall_at_10",
-                                                         "recall_target_met", "qps", "kernel_ms", "sweep", "roofline")}
+                                                         "recall_target_met", "qps", "kernel_ms", "sweep", "stage_rooflines", "roofline")}
     print(json.dumps(line, default=float))
 
 
