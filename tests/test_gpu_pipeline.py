@@ -4,10 +4,13 @@ configurations (clipped mixture L2 with k=64, normalised mixture cosine with 96 
 The two pipelines share the centroids and the entry points, so the partitioning is the same; the kNN graphs come
 from different NN-descent runs, so the comparison is statistical:
   * kNN-graph recall@k against exact neighbours inside each partition: GPU >= CPU - 0.005,
-  * search recall@10 at equal beam, mean over three NN-descent seeds on each side: GPU >= CPU - tolerance.
-On the mixture data the finished index depends strongly on which residual random edges the kNN graph still holds
-(an exact kNN graph has no edge between mixture components): one CPU pipeline differs from the next by up to
-0.12 in recall@10 from the NN-descent seed alone, so the tolerance on the mean is 0.06 for the clipped mixture and 0.015 elsewhere.
+  * search recall@10 at equal beam, mean over several NN-descent seeds on each side: GPU >= CPU - tolerance.
+On the mixture data the finished index depends strongly on which residual far edges the kNN graph still holds (an
+exact kNN graph has no edge between mixture components, so search only crosses components over edges NN-descent has
+not yet replaced).  Measured over 12 seeds on this case: recall@10 varies from seed to seed with sigma 0.05 (beam 32)
+to 0.07 (beam 128) on both sides; the means are 0.611 (GPU) and 0.615 (CPU) at beam 32, 0.780 and 0.823 at beam 128,
+the GPU's lists holding 16 % fewer edges longer than 500 at equal recall@32 (recall@64: 0.861 against 0.866).  Eight seeds and a tolerance of 0.12 on the mean keep this case from failing by chance while a broken
+stage (recall 0.17 against 0.63 was one) still fails; elsewhere three seeds and 0.015.
 With the GPU's kNN graph as input, the later stages are deterministic and the finished graph must be bit-identical.
 """
 import numpy as np
@@ -46,11 +49,10 @@ def _graph_recall(D, knn, truth, k):
 
 CASES = [
     # name, generator, num, dim, partitions, graph degree, knn degree, NN-descent iterations, metric, queries
-    ("clipped-mixture-k64", "gmm_clipped", 20_000, 128, 4, 32, 64, 8, 0, 1000, 0.06),
+    ("clipped-mixture-k64", "gmm_clipped", 20_000, 128, 4, 32, 64, 8, 0, 1000, 0.12),
     ("normalised-mixture-cosine", "gmm_normalized", 20_000, 96, 4, 32, 32, 10, 1, 1000, 0.015),
     ("beta-960-degree64", "beta_scaled", 6_000, 960, 3, 64, 64, 8, 0, 300, 0.015),
 ]
-SEEDS = (0, 1, 2)
 
 
 @pytest.mark.parametrize("name,gen,num,dim,parts,degree,knn_degree,iters,metric,nq,tol", CASES, ids=[c[0] for c in CASES])
@@ -60,6 +62,7 @@ def test_pipeline_matches_cpu_pipeline(hip, name, gen, num, dim, parts, degree, 
     data = getattr(D, gen)(num, dim, seed=1234)
     queries = getattr(D, gen)(nq, dim, seed=4321)
     print("case", name, data.shape, flush=True)
+    SEEDS = tuple(range(8)) if gen == "gmm_clipped" else (0, 1, 2)
 
     # ---- GPU pipeline
     d_data = hip.DeviceArray.from_numpy(data)
@@ -119,6 +122,14 @@ def test_pipeline_matches_cpu_pipeline(hip, name, gen, num, dim, parts, degree, 
     r_gpu, r_cpu = _graph_recall(D, knn_gpu, truth, k_eval), _graph_recall(D, knn_cpu, truth, k_eval)
     print("graph recall@%d gpu %.4f cpu %.4f" % (k_eval, r_gpu, r_cpu), flush=True)
     assert r_gpu >= r_cpu - 0.005
+    if knn_degree > k_eval:
+        # The whole list, not only its better half.  Its tail is far from converged after 8 rounds (0.85-0.87) and the
+        # GPU build trails the CPU restatement there by 0.1-0.5 points on the mixture and 1.4-1.8 points on the 960-d
+        # data (not an effect of offers lost to full inboxes: keeping the nearer offer on overflow changes nothing).
+        truth_k = _exact_knn_in_partitions(O, rdata, seg_start, seg_len, knn_degree, metric)
+        rk_gpu, rk_cpu = _graph_recall(D, knn_gpu, truth_k, knn_degree), _graph_recall(D, knn_cpu, truth_k, knn_degree)
+        print("graph recall@%d gpu %.4f cpu %.4f" % (knn_degree, rk_gpu, rk_cpu), flush=True)
+        assert rk_gpu >= rk_cpu - 0.03
 
     # ---- search recall@10 at equal beam, mean over the seeds; seed 0 of the GPU side runs on the GPU
     gt, _ = O.bruteforce_knn(data, queries, 10, metric)
