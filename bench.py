@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE, KiB per dispatch) and scaled by what the same counters report for copy_kernel moving exactly 1 GiB
 # (--copy-calibration: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Keyed by (workload, beam); other combinations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg1", 256): 6_371_900 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
+    ("cfg1", 256): 6_337_000 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
     ("cfg1-navigable", 32): 2_451_000 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
 }
 
@@ -203,7 +203,10 @@ def run_workload(args, workload, torch, want_cpu):
 
     def hbm_stage(seconds, nbytes):
         gbs = nbytes / seconds / 1e9 if seconds > 0 else 0.0
-        return dict(bound="hbm", seconds=seconds, algorithmic_bytes=int(nbytes), achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS)
+        out = dict(bound="hbm", seconds=seconds, algorithmic_bytes=int(nbytes), achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS)
+        if gbs > HBM_PEAK_GBS:   # rows are scored again and again inside one partition (32 MB at cfg1): most gathers hit L2 / the memory-side cache
+            out["note"] = "algorithmic bytes exceed what HBM can deliver: the stage is served from cache, see the FETCH_SIZE counters"
+        return out
 
     stage_rooflines = {}
     assign_flops = 2.0 * num * parts * dim
