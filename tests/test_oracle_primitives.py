@@ -235,3 +235,37 @@ def test_sort_for_beam_merges_to_the_smallest(max_beam, beam, degree):
         assert got == [(float(np.float32(k)), v) for k, v in truth], (rnd, max_beam, beam, degree)
         for j in range(len(truth), beam):
             assert bd[_swz(j)] >= np.float32(3e38)
+
+
+def test_sort_of_32_slots_on_the_64_network_equals_the_32_network():
+    """With at most 32 candidate slots in use, the reference's strided load (search_kernel.cuh:9-37) puts them on the
+    even elements of the 64-element network and +inf on the odd ones.  The sorted sequence, ties included, is the one
+    the 32-element network gives on the slots alone, provided every +inf key carries the invalid id; the GPU code
+    relies on this.  A real id with an +inf key is the exception (shown too)."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(3)
+    fmax = np.finfo(np.float32).max
+    exception_seen = False
+    for trial in range(3000):
+        used = int(rng.integers(1, 33))
+        keys = np.full(32, fmax, np.float32)
+        vals = np.full(32, 0xFFFFFFFF, np.uint32)
+        keys[:used] = rng.integers(0, rng.integers(1, 7), used).astype(np.float32)      # many equal keys
+        vals[:used] = rng.permutation(100000)[:used].astype(np.uint32)
+        dead = rng.random(32) < rng.random() * 0.5                                       # visited / empty graph slots
+        keys[dead], vals[dead] = fmax, 0xFFFFFFFF
+        k64, v64 = np.full(64, fmax, np.float32), np.full(64, 0xFFFFFFFF, np.uint32)
+        k64[0::2], v64[0::2] = keys, vals
+        a_k, a_v = O.bitonic_warp_sort(k64, v64)
+        b_k, b_v = O.bitonic_warp_sort(keys, vals)
+        assert np.array_equal(a_k[:32], b_k) and np.array_equal(a_v[:32], b_v), trial
+        assert (a_k[32:] == fmax).all() and (a_v[32:] == 0xFFFFFFFF).all()
+        # a real id under an +inf key may end up anywhere among the +inf keys of the larger network
+        keys2, vals2 = keys.copy(), vals.copy()
+        j = int(rng.integers(0, 32))
+        keys2[j], vals2[j] = fmax, 77
+        k64[0::2], v64[0::2] = keys2, vals2
+        a_k, a_v = O.bitonic_warp_sort(k64, v64)
+        b_k, b_v = O.bitonic_warp_sort(keys2, vals2)
+        exception_seen |= not np.array_equal(a_v[:32], b_v)
+    assert exception_seen
