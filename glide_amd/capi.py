@@ -291,6 +291,15 @@ def kmeans_workspace_bytes(cluster_num, dim):
     return int(_size_fn("glide_hip_kmeans_workspace_bytes")(u32(cluster_num), u32(dim)))
 
 
+def kmeans_seed_workspace_bytes(sample_num):
+    return int(_size_fn("glide_hip_kmeans_seed_workspace_bytes")(u32(sample_num)))
+
+
+def kmeans_seed(sample, sample_num, dim, cluster_num, seed, centroids, workspace, workspace_bytes, chosen_rows=None, stream=None):
+    check(lib().glide_hip_kmeans_seed(_ptr(sample), u32(sample_num), u32(dim), u32(cluster_num), u32(seed), _ptr(centroids),
+                                      _ptr(chosen_rows), _ptr(workspace), C.c_size_t(workspace_bytes), vp(stream)), "glide_hip_kmeans_seed")
+
+
 def kmeans_fit(sample, sample_num, dim, cluster_num, iterations, centroids, workspace, workspace_bytes, stream=None):
     check(lib().glide_hip_kmeans_fit(_ptr(sample), u32(sample_num), u32(dim), u32(cluster_num), u32(iterations),
                                      _ptr(centroids), _ptr(workspace), C.c_size_t(workspace_bytes), vp(stream)),

@@ -341,6 +341,192 @@ __global__ __launch_bounds__(256) void row_norms_kernel(const float* rows, uint3
     if (lane == 0) norms[i] = acc;
 }
 
+// ---- greedy k-means++ seeding (cuvs::cluster::kmeans::fit initialises with its k-means++ family by default) ----
+// Step s draws 2 + floor(ln k) candidate rows with probability min_dist[i] / sum (uniformly for s = 0) and keeps the
+// one that leaves the smallest potential sum_i min(min_dist[i], |x_i - candidate|^2); the distance kernel then lowers
+// min_dist with the distances to the winner.  Draw j of step s is a counter-based hash of (seed, 16 s + j), so a run
+// is reproducible and a CPU restatement can follow it.
+constexpr uint32_t kSeedTrials = 8;        // most candidates per step
+constexpr uint32_t kSeedPoints = 64;       // sample rows per workgroup of the trial kernel
+
+__host__ __device__ inline uint32_t seed_trials(uint32_t k) {
+    uint32_t t = 2;
+    for (uint32_t v = k; v >= 3; v = static_cast<uint32_t>(v / 2.718281828459045)) t++;
+    return t > kSeedTrials ? kSeedTrials : t;
+}
+__device__ __forceinline__ uint32_t seed_hash(uint32_t seed, uint32_t step) {
+    uint32_t x = seed * 0x9E3779B9u + step * 0x85EBCA6Bu + 0x6A09E667u;
+    x ^= x >> 16; x *= 0x7FEB352Du; x ^= x >> 15; x *= 0x846CA68Bu; x ^= x >> 16;
+    return x;
+}
+__device__ __forceinline__ double shfl_up_f64(double v, int delta) { return __shfl_up(v, delta); }
+__device__ __forceinline__ double shfl_f64(double v, int src) { return __shfl(v, src); }
+
+// One wavefront: first index i in [0, len) with load(i) > 0 whose running sum (entries 0..i) exceeds target, and the
+// sum of the entries before it; the last positive entry if no running sum gets there (rounding at the upper end).
+template <class Load>
+__device__ __forceinline__ uint32_t wave_locate(Load load, uint32_t len, double target, double& before, int lane) {
+    const uint32_t seg = (len + 63) / 64;
+    const uint32_t lo = lane * seg < len ? lane * seg : len, hi = lo + seg < len ? lo + seg : len;
+    double local = 0.0;
+    for (uint32_t i = lo; i < hi; i++) local += load(i);
+    double incl = local;
+    for (int off = 1; off < 64; off <<= 1) {
+        const double t = shfl_up_f64(incl, off);
+        if (lane >= off) incl += t;
+    }
+    double run = incl - local;
+    uint32_t found = 0xffffffffu, last = 0xffffffffu;
+    double run_found = 0.0, run_last = 0.0;
+    for (uint32_t i = lo; i < hi; i++) {
+        const double v = load(i);
+        if (v > 0.0) {
+            last = i;
+            run_last = run;
+            if (found == 0xffffffffu && run + v > target) { found = i; run_found = run; }
+        }
+        run += v;
+    }
+    const uint64_t hit = ballot(found != 0xffffffffu);
+    if (hit) {
+        const int src = __builtin_ctzll(hit);
+        before = shfl_f64(run_found, src);
+        return static_cast<uint32_t>(__shfl(static_cast<int>(found), src));
+    }
+    const uint64_t any = ballot(last != 0xffffffffu);
+    if (!any) { before = 0.0; return 0; }
+    const int src = 63 - __builtin_clzll(any);
+    before = shfl_f64(run_last, src);
+    return static_cast<uint32_t>(__shfl(static_cast<int>(last), src));
+}
+
+// one workgroup of 16 wavefronts: chunk sums of min_dist, then wavefront j draws candidate j
+__global__ __launch_bounds__(1024) void kmeanspp_pick_kernel(uint32_t n, const float* min_dist, uint32_t seed, uint32_t step, uint32_t trials,
+                                                            uint32_t* candidates) {
+    __shared__ double part[1024];
+    const uint32_t t = threadIdx.x;
+    const int lane = lane_id();
+    const uint32_t wave = t >> 6;
+    if (step == 0) {
+        if (t < trials) candidates[t] = seed_hash(seed, 0) % n;
+        return;
+    }
+    const uint32_t chunk = (n + 1023) / 1024;
+    {
+        const uint32_t lo = t * chunk < n ? t * chunk : n, hi = lo + chunk < n ? lo + chunk : n;
+        double acc = 0.0;
+        for (uint32_t i = lo; i < hi; i++) acc += static_cast<double>(min_dist[i]);
+        part[t] = acc;
+    }
+    __syncthreads();
+    if (wave >= trials) return;
+    double total = 0.0;
+    for (uint32_t i = lane * 16; i < lane * 16 + 16; i++) total += part[i];
+    for (int off = 32; off >= 1; off >>= 1) total += __shfl_xor(total, off);
+    uint32_t cand = seed_hash(seed, 16 * step) % n;      // every row already coincides with a centroid
+    if (total > 0.0) {
+        const uint32_t h = seed_hash(seed, 16 * step + wave);
+        const double target = static_cast<double>(h >> 8) * (1.0 / 16777216.0) * total;
+        double before = 0.0, unused = 0.0;
+        const double* pp = part;
+        const uint32_t c = wave_locate([pp](uint32_t i) { return pp[i]; }, 1024, target, before, lane);
+        const uint32_t base = c * chunk, len = (base + chunk < n ? base + chunk : n) - base;
+        const float* md = min_dist + base;
+        cand = base + wave_locate([md](uint32_t i) { return static_cast<double>(md[i]); }, len, target - before, unused, lane);
+    }
+    if (lane == 0) candidates[wave] = cand;
+}
+
+// 64 sample rows per workgroup, 16 per wavefront: potential of every candidate over these rows, in double
+__global__ __launch_bounds__(256) void kmeanspp_trial_kernel(const float* sample, uint32_t n, uint32_t dim, const float* min_dist,
+                                                             const uint32_t* candidates, uint32_t trials, double* partial) {
+    __shared__ double wave_pot[4][kSeedTrials];
+    const int lane = lane_id();
+    const uint32_t wave = threadIdx.x >> 6;
+    double pot[kSeedTrials];
+#pragma unroll
+    for (uint32_t j = 0; j < kSeedTrials; j++) pot[j] = 0.0;
+    for (uint32_t r = 0; r < kSeedPoints / 4; r++) {
+        const uint32_t i = blockIdx.x * kSeedPoints + wave * (kSeedPoints / 4) + r;
+        if (i >= n) break;
+        const float* x = sample + static_cast<size_t>(i) * dim;
+        const float md = min_dist[i];
+#pragma unroll
+        for (uint32_t j = 0; j < kSeedTrials; j++) {
+            if (j >= trials) break;
+            const float* c = sample + static_cast<size_t>(candidates[j]) * dim;
+            float acc = 0.f;
+            for (uint32_t d0 = lane * 4; d0 < dim; d0 += 256) {
+                const float4 a = *reinterpret_cast<const float4*>(x + d0);
+                const float4 b = *reinterpret_cast<const float4*>(c + d0);
+                const float dx = a.x - b.x, dy = a.y - b.y, dz = a.z - b.z, dw = a.w - b.w;
+                acc = fmaf(dx, dx, acc);
+                acc = fmaf(dy, dy, acc);
+                acc = fmaf(dz, dz, acc);
+                acc = fmaf(dw, dw, acc);
+            }
+            acc = wave_sum(acc);
+            pot[j] += static_cast<double>(fminf(md, acc));
+        }
+    }
+    if (lane == 0)
+        for (uint32_t j = 0; j < kSeedTrials; j++) wave_pot[wave][j] = pot[j];
+    __syncthreads();
+    if (threadIdx.x < kSeedTrials)
+        partial[static_cast<size_t>(blockIdx.x) * kSeedTrials + threadIdx.x] =
+            wave_pot[0][threadIdx.x] + wave_pot[1][threadIdx.x] + wave_pot[2][threadIdx.x] + wave_pot[3][threadIdx.x];
+}
+
+// one workgroup: potentials summed over the trial kernel's workgroups, the smallest wins (the first on a tie); its row
+// becomes centroid `step`
+__global__ __launch_bounds__(256) void kmeanspp_choose_kernel(const float* sample, uint32_t dim, const double* partial, uint32_t blocks,
+                                                              const uint32_t* candidates, uint32_t trials, uint32_t step, float* centroids,
+                                                              uint32_t* chosen_rows) {
+    __shared__ double slice[kSeedTrials][32];
+    __shared__ uint32_t winner;
+    const uint32_t j = threadIdx.x >> 5, sl = threadIdx.x & 31;
+    double acc = 0.0;
+    if (step > 0 && j < trials)
+        for (uint32_t b = sl; b < blocks; b += 32) acc += partial[static_cast<size_t>(b) * kSeedTrials + j];
+    slice[j][sl] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t best = 0;
+        double best_pot = 0.0;
+        for (uint32_t c = 0; c < (step > 0 ? trials : 1u); c++) {
+            double p = 0.0;
+            for (uint32_t q = 0; q < 32; q++) p += slice[c][q];
+            if (c == 0 || p < best_pot) { best_pot = p; best = c; }
+        }
+        winner = candidates[best];
+        if (chosen_rows) chosen_rows[step] = winner;
+    }
+    __syncthreads();
+    const float* src = sample + static_cast<size_t>(winner) * dim;
+    for (uint32_t d = threadIdx.x; d < dim; d += 256) centroids[static_cast<size_t>(step) * dim + d] = src[d];
+}
+
+// one wavefront per sample row: min_dist[i] = min(min_dist[i], |x_i - c|^2) (set on the first step)
+__global__ __launch_bounds__(256) void kmeanspp_distance_kernel(const float* sample, uint32_t n, uint32_t dim, const float* centroid, float* min_dist,
+                                                                int first) {
+    const int lane = lane_id();
+    const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (i >= n) return;
+    const float* x = sample + static_cast<size_t>(i) * dim;
+    float acc = 0.f;
+    for (uint32_t d0 = lane * 4; d0 < dim; d0 += 256) {
+        const float4 a = *reinterpret_cast<const float4*>(x + d0);
+        const float4 b = *reinterpret_cast<const float4*>(centroid + d0);
+        const float dx = a.x - b.x, dy = a.y - b.y, dz = a.z - b.z, dw = a.w - b.w;
+        acc = fmaf(dx, dx, acc);
+        acc = fmaf(dy, dy, acc);
+        acc = fmaf(dz, dz, acc);
+        acc = fmaf(dw, dw, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) min_dist[i] = first ? acc : fminf(min_dist[i], acc);
+}
+
 // ---- Lloyd k-means on a sample (stand-in for cuvs::cluster::kmeans::fit, reference partition.cuh:48-54) ----
 // one wavefront per sample point: nearest centroid by direct distances, then atomic accumulation
 __global__ __launch_bounds__(256) void kmeans_accumulate_kernel(const float* sample, uint32_t n, uint32_t dim, const float* centroids,
@@ -377,6 +563,10 @@ size_t assign_lds_bytes(int cb, uint32_t centroid_num) {
 }  // namespace glide
 
 using namespace glide;
+
+namespace {
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+}  // namespace
 
 extern "C" {
 
@@ -443,6 +633,37 @@ int glide_hip_sample_rows(const float* data, uint32_t dim, const uint32_t* sampl
 
 size_t glide_hip_kmeans_workspace_bytes(uint32_t cluster_num, uint32_t dim) {
     return static_cast<size_t>(cluster_num) * dim * 4 + static_cast<size_t>(cluster_num) * 4 + 256;
+}
+
+size_t glide_hip_kmeans_seed_workspace_bytes(uint32_t sample_num) {
+    // min_dist (f32 per row) | candidates (8 u32) | per-workgroup potentials of the trial kernel (8 f64 each)
+    return align_up(static_cast<size_t>(sample_num) * 4, 256) + 256 + static_cast<size_t>(ceil_div(sample_num, kSeedPoints)) * kSeedTrials * 8;
+}
+
+int glide_hip_kmeans_seed(const float* sample, uint32_t sample_num, uint32_t dim, uint32_t cluster_num, uint32_t seed, float* centroids,
+                          uint32_t* chosen_rows, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!sample || !centroids || !workspace || dim == 0 || cluster_num == 0 || sample_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    if (workspace_bytes < glide_hip_kmeans_seed_workspace_bytes(sample_num) || reinterpret_cast<uintptr_t>(workspace) % 8)
+        return GLIDE_ERR_BAD_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(sample) % 16 || reinterpret_cast<uintptr_t>(centroids) % 16) return GLIDE_ERR_BAD_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    unsigned char* w = static_cast<unsigned char*>(workspace);
+    float* min_dist = reinterpret_cast<float*>(w);
+    uint32_t* candidates = reinterpret_cast<uint32_t*>(w + align_up(static_cast<size_t>(sample_num) * 4, 256));
+    double* partial = reinterpret_cast<double*>(w + align_up(static_cast<size_t>(sample_num) * 4, 256) + 256);
+    const uint32_t trials = seed_trials(cluster_num), blocks = ceil_div(sample_num, kSeedPoints);
+    for (uint32_t step = 0; step < cluster_num; step++) {
+        hipLaunchKernelGGL(kmeanspp_pick_kernel, dim3(1), dim3(1024), 0, s, sample_num, min_dist, seed, step, trials, candidates);
+        if (step > 0)
+            hipLaunchKernelGGL(kmeanspp_trial_kernel, dim3(blocks), dim3(256), 0, s, sample, sample_num, dim, min_dist, candidates, trials, partial);
+        hipLaunchKernelGGL(kmeanspp_choose_kernel, dim3(1), dim3(256), 0, s, sample, dim, partial, blocks, candidates, trials, step, centroids,
+                           chosen_rows);
+        if (step + 1 < cluster_num)
+            hipLaunchKernelGGL(kmeanspp_distance_kernel, dim3(ceil_div(sample_num, 4)), dim3(256), 0, s, sample, sample_num, dim,
+                               centroids + static_cast<size_t>(step) * dim, min_dist, step == 0 ? 1 : 0);
+    }
+    return launch_status();
 }
 
 int glide_hip_kmeans_fit(const float* sample, uint32_t sample_num, uint32_t dim, uint32_t cluster_num, uint32_t iterations,

@@ -15,7 +15,7 @@
 namespace glide {
 
 // get_centroids (partition.cuh:8-59): shuffle ids, gather a sample, cluster it.  The reference calls
-// cuvs::cluster::kmeans::fit; here the first centroid_num sampled rows seed Lloyd iterations.
+// cuvs::cluster::kmeans::fit; here greedy k-means++ seeding, then Lloyd iterations.
 template <typename Data_t, typename Index_t>
 void get_centroids(device_resources& handle, device_matrix_view<Data_t, Index_t> d_data_view, device_matrix_view<float> d_centroid_view,
                    const PartitionParameter& param, float& build_time) {
@@ -28,18 +28,15 @@ void get_centroids(device_resources& handle, device_matrix_view<Data_t, Index_t>
     device_vector<uint32_t> d_indices(sample_num);
     copy_to_device(d_indices.data_handle(), indices.data(), sample_num);
     device_matrix<float> d_sample(sample_num, dim);
-    std::vector<uint32_t> first(c);
-    for (uint32_t i = 0; i < c; i++) first[i] = i % sample_num;
-    device_vector<uint32_t> d_first(c);
-    copy_to_device(d_first.data_handle(), first.data(), c);
-    const size_t wb = glide_hip_kmeans_workspace_bytes(c, dim);
-    device_buffer ws(wb);
+    const size_t wb = glide_hip_kmeans_workspace_bytes(c, dim), sb = glide_hip_kmeans_seed_workspace_bytes(sample_num);
+    device_buffer ws(wb), seed_ws(sb);
     gpu_timer timer;
     timer.start();
     hip_try(glide_hip_sample_rows(d_data_view.data_handle(), dim, d_indices.data_handle(), sample_num, d_sample.data_handle(), handle.stream()),
             "glide_hip_sample_rows");
-    hip_try(glide_hip_sample_rows(d_sample.data_handle(), dim, d_first.data_handle(), c, d_centroid_view.data_handle(), handle.stream()),
-            "glide_hip_sample_rows");
+    hip_try(glide_hip_kmeans_seed(d_sample.data_handle(), sample_num, dim, c, param.seed, d_centroid_view.data_handle(), nullptr, seed_ws.get(), sb,
+                                  handle.stream()),
+            "glide_hip_kmeans_seed");
     hip_try(glide_hip_kmeans_fit(d_sample.data_handle(), sample_num, dim, c, param.kmeans_iterations, d_centroid_view.data_handle(), ws.get(), wb,
                                  handle.stream()),
             "glide_hip_kmeans_fit");

@@ -42,11 +42,13 @@ float get_centroids_for_large(device_resources& handle, const PartitionParameter
     for (uint32_t i = 0; i < sample_num; i++) std::copy_n(h_data.row(indices[i]), dim, &h_sample(i, 0));   // widens uint8 rows
     device_matrix<float> d_sample(sample_num, dim);
     copy_to_device(d_sample.data_handle(), h_sample.data_handle(), h_sample.size());
-    copy_to_device(d_centroid_view.data_handle(), h_sample.data_handle(), static_cast<size_t>(std::min(c, sample_num)) * dim);
-    const size_t wb = glide_hip_kmeans_workspace_bytes(c, dim);
-    device_buffer ws(wb);
+    const size_t wb = glide_hip_kmeans_workspace_bytes(c, dim), sb = glide_hip_kmeans_seed_workspace_bytes(sample_num);
+    device_buffer ws(wb), seed_ws(sb);
     gpu_timer timer;
     timer.start();
+    hip_try(glide_hip_kmeans_seed(d_sample.data_handle(), sample_num, dim, c, param.seed, d_centroid_view.data_handle(), nullptr, seed_ws.get(), sb,
+                                  handle.stream()),
+            "glide_hip_kmeans_seed");
     hip_try(glide_hip_kmeans_fit(d_sample.data_handle(), sample_num, dim, c, param.kmeans_iterations, d_centroid_view.data_handle(), ws.get(), wb,
                                  handle.stream()),
             "glide_hip_kmeans_fit");

@@ -31,7 +31,7 @@ class PartitionParameter:          # params.cuh:10-15
     boundary_factor: float = 1.05
     sample_factor: float = 0.01
     metric: int = Metric.Euclidean
-    kmeans_iterations: int = 20     # cuVS kmeans is replaced by Lloyd steps; count and seed are explicit here
+    kmeans_iterations: int = 20     # cuVS kmeans is replaced by greedy k-means++ seeding + Lloyd steps; count and seed are explicit here
     seed: int = 7
 
 
@@ -156,9 +156,11 @@ def preprocess(param, d_data, result=None):
     d_centroids = capi.DeviceArray((c, dim), np.float32)
     wb = capi.kmeans_workspace_bytes(c, dim)
     ws = capi.DeviceArray(wb // 4 + 1, np.uint32)
+    sb = capi.kmeans_seed_workspace_bytes(sample_num)
+    seed_ws = capi.DeviceArray(sb // 8 + 1, np.uint64)
     with _Timer() as t:
         capi.sample_rows(d_data, dim, d_ids, sample_num, d_sample)
-        capi.sample_rows(d_sample, dim, capi.DeviceArray.from_numpy(np.arange(c, dtype=np.uint32) % sample_num), c, d_centroids)
+        capi.kmeans_seed(d_sample, sample_num, dim, c, param.seed, d_centroids, seed_ws, sb)
         capi.kmeans_fit(d_sample, sample_num, dim, c, param.kmeans_iterations, d_centroids, ws, wb)
     times["centroids"] = t.seconds
     # define_partition (partition.cuh:61-116)

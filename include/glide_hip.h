@@ -104,8 +104,16 @@ int glide_hip_reorder_batch(const float *data, uint32_t num, uint32_t dim, const
 int glide_hip_sample_rows(const float *data, uint32_t dim, const uint32_t *sample_ids, uint32_t sample_num,
                           float *sample, void *stream);
 
-/* Stands in for cuvs::cluster::kmeans::fit (third-party; call site partition.cuh:48-54): `iterations` Lloyd
- * steps from the centroids passed in (the caller seeds them, e.g. with sampled rows). */
+/* Stands in for cuvs::cluster::kmeans::fit (third-party, rapidsai/cuvs 24.08; call site partition.cuh:48-54) in two
+ * calls.  glide_hip_kmeans_seed: greedy k-means++ seeding.  Every further centroid is the best of 2 + floor(ln k)
+ * sample rows drawn with probability proportional to their squared distance from the nearest centroid chosen so
+ * far, best = smallest remaining potential (cuVS initialises with its k-means++ family by default).  The draws are a
+ * hash of (seed, step, trial), so a run is reproducible.  chosen_rows (nullable, cluster_num u32) receives the sample
+ * rows taken.  workspace: 8-byte aligned.  glide_hip_kmeans_fit: `iterations` Lloyd steps from the centroids passed in. */
+size_t glide_hip_kmeans_seed_workspace_bytes(uint32_t sample_num);
+int glide_hip_kmeans_seed(const float *sample, uint32_t sample_num, uint32_t dim, uint32_t cluster_num, uint32_t seed,
+                          float *centroids, uint32_t *chosen_rows, void *workspace, size_t workspace_bytes,
+                          void *stream);
 size_t glide_hip_kmeans_workspace_bytes(uint32_t cluster_num, uint32_t dim);
 int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim, uint32_t cluster_num,
                          uint32_t iterations, float *centroids, void *workspace, size_t workspace_bytes,

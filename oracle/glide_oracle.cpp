@@ -1133,6 +1133,90 @@ void go_bruteforce_knn(const float *data, uint32_t num, uint32_t dim, const floa
     }
 }
 
+// Greedy k-means++ seeding as the HIP library's glide_hip_kmeans_seed does it (no counterpart in the reference tree:
+// the reference calls cuvs::cluster::kmeans::fit, whose default initialisation is of the k-means++ family).  Every
+// step draws 2 + floor(ln k) candidate rows with probability min_dist[i] / sum (the sum taken over 1024 chunks in
+// double; draw j of step s is a hash of (seed, 16 s + j)) and keeps the candidate that leaves the smallest potential
+// sum_i min(min_dist[i], |x_i - candidate|^2), the first one on a tie.
+static uint32_t seed_hash(uint32_t seed, uint32_t step) {
+    uint32_t x = seed * 0x9E3779B9u + step * 0x85EBCA6Bu + 0x6A09E667u;
+    x ^= x >> 16; x *= 0x7FEB352Du; x ^= x >> 15; x *= 0x846CA68Bu; x ^= x >> 16;
+    return x;
+}
+static uint32_t kmeans_trials(uint32_t k) {
+    uint32_t t = 2;
+    for (uint32_t v = k; v >= 3; v = static_cast<uint32_t>(v / 2.718281828459045)) t++;   // 2 + floor(ln k) for k >= 1
+    return t > 8 ? 8 : t;
+}
+// first index whose running sum of the positive entries exceeds target; the last positive entry if none does
+static uint32_t locate(const double *v, uint32_t len, double target, double *before) {
+    double run = 0.0;
+    uint32_t last = 0;
+    for (uint32_t i = 0; i < len; i++) {
+        if (v[i] > 0.0) {
+            last = i;
+            if (run + v[i] > target) { *before = run; return i; }
+        }
+        run += v[i];
+    }
+    double r = 0.0;
+    for (uint32_t i = 0; i < last; i++) r += v[i];
+    *before = r;
+    return last;
+}
+
+void go_kmeans_seed(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32_t seed, float *centroids,
+                    uint32_t *chosen_out) {
+    std::vector<float> min_dist(n, FLT_MAX);
+    const uint32_t chunk = (n + 1023) / 1024, trials = kmeans_trials(k);
+    auto dist_to = [&](uint32_t row, uint32_t i) {
+        float acc = 0.0f;
+        for (uint32_t t = 0; t < dim; t++) {
+            const float diff = sample[static_cast<size_t>(i) * dim + t] - sample[static_cast<size_t>(row) * dim + t];
+            acc += diff * diff;
+        }
+        return acc;
+    };
+    for (uint32_t step = 0; step < k; step++) {
+        uint32_t chosen = seed_hash(seed, 16 * step) % n;
+        if (step > 0) {
+            std::vector<double> part(1024, 0.0);
+            double total = 0.0;
+            for (uint32_t t = 0; t < 1024; t++) {
+                const uint64_t lo = std::min<uint64_t>(static_cast<uint64_t>(t) * chunk, n), hi = std::min<uint64_t>(lo + chunk, n);
+                for (uint64_t i = lo; i < hi; i++) part[t] += static_cast<double>(min_dist[i]);
+            }
+            for (uint32_t t = 0; t < 1024; t++) total += part[t];
+            if (total > 0.0) {
+                double best_pot = 0.0;
+                for (uint32_t j = 0; j < trials; j++) {
+                    const uint32_t h = seed_hash(seed, 16 * step + j);
+                    const double target = static_cast<double>(h >> 8) * (1.0 / 16777216.0) * total;
+                    double before = 0.0;
+                    const uint32_t c = locate(part.data(), 1024, target, &before);
+                    const uint32_t base = c * chunk, len = static_cast<uint32_t>(std::min<uint64_t>(static_cast<uint64_t>(base) + chunk, n) - base);
+                    std::vector<double> seg(len);
+                    for (uint32_t i = 0; i < len; i++) seg[i] = static_cast<double>(min_dist[base + i]);
+                    double b2 = 0.0;
+                    const uint32_t cand = base + locate(seg.data(), len, target - before, &b2);
+                    double pot = 0.0;
+                    for (uint32_t i = 0; i < n; i++) pot += static_cast<double>(std::min(min_dist[i], dist_to(cand, i)));
+                    if (j == 0 || pot < best_pot) { best_pot = pot; chosen = cand; }
+                }
+            }
+        }
+        if (chosen_out) chosen_out[step] = chosen;
+        std::memcpy(centroids + static_cast<size_t>(step) * dim, sample + static_cast<size_t>(chosen) * dim, dim * sizeof(float));
+        for (uint32_t i = 0; i < n; i++) {
+            const float d = dist_to(chosen, i);
+            min_dist[i] = step == 0 ? d : std::min(min_dist[i], d);
+        }
+    }
+}
+
+// Lloyd steps from the centroids passed in (init != 0) or from k rows of a shuffle of the sample (init == 0)
+void go_kmeans_from(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32_t iterations, float *centroids);
+
 void go_kmeans(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32_t iterations, uint32_t seed,
                float *centroids) {
     std::mt19937 gen(seed);
@@ -1141,6 +1225,10 @@ void go_kmeans(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32
     std::shuffle(perm.begin(), perm.end(), gen);
     for (uint32_t c = 0; c < k; c++)
         std::memcpy(centroids + static_cast<size_t>(c) * dim, sample + static_cast<size_t>(perm[c % n]) * dim, dim * sizeof(float));
+    go_kmeans_from(sample, n, dim, k, iterations, centroids);
+}
+
+void go_kmeans_from(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32_t iterations, float *centroids) {
     std::vector<double> sums(static_cast<size_t>(k) * dim);
     std::vector<uint32_t> counts(k);
     for (uint32_t it = 0; it < iterations; it++) {

@@ -23,7 +23,9 @@
  *   beam search            recall vs exact brute force; bit-exactness is GPU-vs-oracle only
  *   NN-descent             parity unpinned bit-wise (the reference is unseeded and racy);
  *                          statistical: graph recall vs exact kNN
- *   k-means (cuVS)         parity unpinned (third-party, absent from the reference tree)
+ *   k-means (cuVS)         parity unpinned (third-party, absent from the reference tree); the stand-in
+ *                          (greedy k-means++ seeding + Lloyd) is held to scikit-learn's inertia through
+ *                          the fixture tests/golden/kmeans_sklearn.json
  */
 #pragma once
 #include <stdint.h>
@@ -151,6 +153,9 @@ int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, uint32_t di
 void go_bruteforce_knn(const float *data, uint32_t num, uint32_t dim, const float *queries, uint32_t query_num,
                        uint32_t k, int metric, int exclude_self, uint32_t *ids, float *dists, int threads);
 /* Lloyd k-means (stand-in for cuvs::cluster::kmeans::fit, partition.cuh:48-54) */
+void go_kmeans_seed(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32_t seed, float *centroids,
+                    uint32_t *chosen_out);
+void go_kmeans_from(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32_t iterations, float *centroids);
 void go_kmeans(const float *sample, uint32_t n, uint32_t dim, uint32_t k, uint32_t iterations, uint32_t seed,
                float *centroids);
 

@@ -336,6 +336,21 @@ def kmeans(sample, k, iterations=20, seed=7):
     return cent
 
 
+def kmeans_seed(sample, k, seed=7):
+    """k-means++ seeding with the HIP library's draws; returns (centroids, chosen sample rows)."""
+    sample = _f32(sample)
+    cent = np.empty((k, sample.shape[1]), dtype=np.float32)
+    chosen = np.empty(k, dtype=np.uint32)
+    lib().go_kmeans_seed(_p(sample), u32(sample.shape[0]), u32(sample.shape[1]), u32(k), u32(seed), _p(cent), _p(chosen))
+    return cent, chosen
+
+
+def kmeans_from(sample, centroids, iterations=20):
+    sample, cent = _f32(sample), _f32(centroids).copy()
+    lib().go_kmeans_from(_p(sample), u32(sample.shape[0]), u32(sample.shape[1]), u32(cent.shape[0]), u32(iterations), _p(cent))
+    return cent
+
+
 def build_index(data, centroid_num, graph_degree=32, knn_degree=32, boundary_factor=1.04, relaxant=1.05,
                 build_beam=64, refine_beam=128, nnd_iterations=8, metric=EUCLIDEAN, seed=11, sample_factor=0.01,
                 centroids=None, threads=0):
