@@ -40,6 +40,7 @@ def parse():
     ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg1-navigable", "cfg2", "cfg3"])
     ap.add_argument("--nnd-iterations", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--knn-only", action="store_true", help="partition + NN-descent kNN graph of the workload only (for kernel profiles)")
     ap.add_argument("--no-navigable", action="store_true", help="skip the extra navigable-data variant")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel on 1 GiB x steps (yardstick for rocprofv3 byte counters) and exit")
@@ -322,6 +323,21 @@ def main():
         print(json.dumps({"stage": "partition assign (assign + scan + slot kernels)", "rows": num, "dim": dim, "centroids": c, "ms": ms,
                           "algorithmic_GBps": (num * dim * 4 + num * 12) / ms / 1e6, "algorithmic_TFLOPs": 2.0 * num * c * dim / ms / 1e9,
                           "fp32_mfma_peak_TFLOPs": 157.3}))
+        return
+
+    if args.knn_only:
+        from glide_amd import index as G
+        num, parts, knn_degree, nnd_iters, nq, desc, dim, metric, degree = WORKLOADS[args.workload]
+        data, _ = make_data(args.workload, num, nq)
+        d_data = capi.DeviceArray.from_numpy(data)
+        res = {}
+        pp = G.PartitionParameter(centroid_num=parts, boundary_factor=1.04, sample_factor=0.01, metric=metric)
+        d_re, d_map, h_start, h_len, d_cent = G.preprocess(pp, d_data, res)
+        nn = G.NNDescentParameter(graph_degree=knn_degree, max_iterations=args.nnd_iterations or nnd_iters)
+        G.build_nnd(nn, d_re, h_start, h_len, res, stats=True)
+        print(json.dumps({"stage": "NN-descent kNN graph", "workload": desc, "rows": int(h_len.sum()), "dim": dim, "k": knn_degree,
+                          "iterations_allowed": nn.max_iterations, "knn_sec": res["knn_time"], "offers": res["nnd_stats"][0],
+                          "offers_beyond_inbox": res["nnd_stats"][1]}))
         return
 
     main_res = run_workload(args, args.workload, torch, want_cpu=not args.no_cpu)

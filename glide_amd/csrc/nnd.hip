@@ -13,6 +13,7 @@
 // in the list instead of a host-side Bloom filter.  All ids are partition-local.
 #include "common.hpp"
 #include "host_util.hpp"
+#include <vector>
 
 namespace glide {
 
@@ -886,6 +887,17 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
         if ((rc = nnd_join(c)) != GLIDE_OK) return rc;
         if ((rc = nnd_merge(c, stats_out != nullptr)) != GLIDE_OK) return rc;
         if ((rc = nnd_converge(c, dim, termination_threshold)) != GLIDE_OK) return rc;
+        // GNND::build leaves its loop when the update count falls below the limit (nn_descent.cuh:1270-1284).  Here the
+        // partitions rest one by one on the device; once none is active the remaining rounds would only launch kernels
+        // that return at once, so the states are read back (a few hundred bytes) and the loop ends.
+        if (termination_threshold > 0.f && it >= 2 && it + 1 < iterations) {
+            std::vector<uint32_t> states(segment_num);
+            GLIDE_HIP_TRY(hipMemcpyAsync(states.data(), c.segs.state, sizeof(uint32_t) * segment_num, hipMemcpyDeviceToHost, c.s));
+            GLIDE_HIP_TRY(hipStreamSynchronize(c.s));
+            bool any_active = false;
+            for (uint32_t st : states) any_active |= st != kDone;
+            if (!any_active) break;
+        }
     }
     return nnd_finalize(c, knn_degree, knn_graph, stats_out);
 }

@@ -129,7 +129,9 @@ int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim,
  * epilogue, one offer per row/column) -> merge are run; lists, flags and samples stay in `workspace`.
  * termination_threshold (NNDescentParameter::termination_threshold, params.cuh:21; 0 disables): a partition whose
  * list insertions on every 100th row fall below termination_threshold * reorder_num * dim / 100 in a round
- * (nn_descent.cuh:1123,1280) runs one more round and is then left alone.  At most 2048 partitions.
+ * (nn_descent.cuh:1123,1280) runs one more round and is then left alone; from the third round on the partition
+ * states are read back after each round (the call then waits on `stream`) and the loop ends once every partition
+ * rests.  At most 2048 partitions.
  * stats_out (nullable, 2 device u64): offers received by the merge step, offers dropped by a full inbox.
  * Limits: knn_degree <= 65 (list width round_up32(1.3 * knn_degree) <= 96, Bloom filter <= 2048 bits), dim % 4 == 0. */
 size_t glide_hip_nnd_workspace_bytes(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree);
