@@ -513,23 +513,15 @@ __device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane
 //   the list and this round's offers are sorted together by (distance, id); of the distinct offered ids only the
 //   best 32 count (the rest are dropped, as the 32-wide device list drops them); those not yet in the list enter it;
 //   new samples = those of the best 32 that the Bloom filter has not seen; the ones entering the list are flagged old.
+// The sort network is sized by what the node holds this round (list + offers received): the keys are distinct up to
+// identical copies, so every size gives the same sorted sequence, and most nodes need far less than the largest one.
 template <int M>
-__global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t num,
-                                                        uint32_t width, uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new,
-                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats, Segments segs) {
+__device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t width,
+                                           uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new, uint32_t* fwd_old,
+                                           uint32_t* counts, unsigned long long* stats, Segments segs, uint32_t node, uint32_t seg, uint32_t raw,
+                                           uint32_t* filter, int lane) {
     constexpr int NR = M / 64;
-    __shared__ uint32_t filter_lds[4][64];
-    const int lane = lane_id();
-    const int wave = threadIdx.x >> 6;
-    const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (node >= num) return;
-    uint32_t seg_start, seg_len;
-    const uint32_t seg = locate_uniform(segs, node, seg_start, seg_len);
-    if (segs.state[seg] == kDone) return;
-    uint32_t* filter = filter_lds[wave];
     const uint32_t bloom_words = bloom_sets * 16;
-    if (static_cast<uint32_t>(lane) < bloom_words) filter[lane] = bloom[static_cast<size_t>(node) * bloom_words + lane];
-    const uint32_t raw = inbox_counts[node];
     const uint32_t n_in = raw < inbox_cap ? raw : inbox_cap;
     unsigned long long k[NR];
     uint32_t v[NR];
@@ -665,6 +657,34 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
             if (raw > inbox_cap) atomicAdd(&slot[1], static_cast<unsigned long long>(raw - inbox_cap));
         }
     }
+}
+
+template <int MMAX>
+__global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t num,
+                                                        uint32_t width, uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new,
+                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats, Segments segs) {
+    __shared__ uint32_t filter_lds[4][64];
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (node >= num) return;
+    uint32_t seg_start, seg_len;
+    const uint32_t seg = locate_uniform(segs, node, seg_start, seg_len);
+    if (segs.state[seg] == kDone) return;
+    uint32_t* filter = filter_lds[wave];
+    const uint32_t bloom_words = bloom_sets * 16;
+    if (static_cast<uint32_t>(lane) < bloom_words) filter[lane] = bloom[static_cast<size_t>(node) * bloom_words + lane];
+    const uint32_t raw = inbox_counts[node];
+    const uint32_t held = width + (raw < inbox_cap ? raw : inbox_cap);   // the same for every lane of the wavefront
+    if (held <= 64)
+        merge_node<64>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
+                       seg, raw, filter, lane);
+    else if (MMAX == 128 || held <= 128)
+        merge_node<128>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
+                        seg, raw, filter, lane);
+    else
+        merge_node<256>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
+                        seg, raw, filter, lane);
 }
 
 // Termination test of GNND::build's update_and_sample (nn_descent.cuh:1270-1284): a partition whose sampled update
