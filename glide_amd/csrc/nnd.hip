@@ -242,23 +242,20 @@ __device__ __forceinline__ void mfma_chunk(float16v& acc, const _Float16 (*A)[kR
 }
 
 // Nearest partner of one row (BY_ROW) or one column of the distance tile (get_min_item, nn_descent.cuh:581-623):
-// four adjacent lanes scan 16 entries each, then combine (smaller distance, then smaller index).
-// Thread t handles line t/4; `skip(idx)` excludes entries (the line's own id).
-template <bool BY_ROW, class SkipFn>
-__device__ __forceinline__ void line_argmin(const float (*dist)[kDStride], uint32_t line, uint32_t part, uint32_t count, SkipFn skip,
-                                            float& best, uint32_t& best_idx) {
+// four adjacent lanes scan 16 entries each, then combine (smaller distance, then smaller index).  Thread t handles
+// line t/4.  Entries that must not win (outside the lists, the line's own id) hold FLT_MAX in the tile.
+template <bool BY_ROW>
+__device__ __forceinline__ void line_argmin(const float (*dist)[kDStride], uint32_t line, uint32_t part, float& best, uint32_t& best_idx) {
     best = FLT_MAX;
     best_idx = kInvalid;
     const uint32_t first = part * 16;
-#pragma unroll 4
+#pragma unroll
     for (uint32_t k = 0; k < 16; k++) {
         const uint32_t idx = first + k;
-        if (idx < count) {
-            const float d = BY_ROW ? dist[line][idx] : dist[idx][line];
-            if (d < best && !skip(idx)) {
-                best = d;
-                best_idx = idx;
-            }
+        const float d = BY_ROW ? dist[line][idx] : dist[idx][line];
+        if (d < best) {
+            best = d;
+            best_idx = idx;
         }
     }
 #pragma unroll
@@ -369,7 +366,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     for (int r = 0; r < 16; r++) {
         const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
         float d = FLT_MAX;
-        if (i < n_new && j < n_new) d = fmaxf((L.new_norms[i] + L.new_norms[j]) - 2.f * acc_nn[r], 0.f);
+        if (i < n_new && j < n_new && i != j) d = fmaxf((L.new_norms[i] + L.new_norms[j]) - 2.f * acc_nn[r], 0.f);
         L.dist[i][j] = d;
     }
     __syncthreads();
@@ -379,7 +376,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     {
         float best;
         uint32_t bj;
-        line_argmin<true>(L.dist, line, part, n_new, [line](uint32_t j) { return j == line; }, best, bj);
+        line_argmin<true>(L.dist, line, part, best, bj);
         if (part == 0 && line < n_new && bj != kInvalid) {
             off_target[0] = L.new_ids[line];
             off_cand[0] = L.new_ids[bj];
@@ -389,11 +386,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     if (n_old != 0) {
         // ---- phase 2: new x old (rows: new, columns: old)
         __syncthreads();
+        const uint32_t col_id = cb * 32 + t < n_old ? L.old_ids[cb * 32 + t] : kInvalid;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
-            float d = FLT_MAX;
-            if (i < n_new && j < n_old) d = fmaxf((L.new_norms[i] + L.old_norms[j]) - 2.f * acc_no[r], 0.f);
+            float d = FLT_MAX;   // also where the same point sits in both lists: it is no partner of itself
+            if (i < n_new && j < n_old && L.new_ids[i] != col_id) d = fmaxf((L.new_norms[i] + L.old_norms[j]) - 2.f * acc_no[r], 0.f);
             L.dist[i][j] = d;
         }
         __syncthreads();
@@ -401,8 +399,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
             float best;
             uint32_t bj;
             const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
-            const uint32_t* old_ids = L.old_ids;
-            line_argmin<true>(L.dist, line, part, n_old, [old_ids, me](uint32_t j) { return old_ids[j] == me; }, best, bj);
+            line_argmin<true>(L.dist, line, part, best, bj);
             if (part == 0 && line < n_new && bj != kInvalid) {
                 off_target[1] = me;
                 off_cand[1] = L.old_ids[bj];
@@ -413,8 +410,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
             float best;
             uint32_t bi;
             const uint32_t me = line < n_old ? L.old_ids[line] : kInvalid;
-            const uint32_t* new_ids = L.new_ids;
-            line_argmin<false>(L.dist, line, part, n_new, [new_ids, me](uint32_t i) { return new_ids[i] == me; }, best, bi);
+            line_argmin<false>(L.dist, line, part, best, bi);
             if (part == 0 && line < n_old && bi != kInvalid) {
                 off_target[2] = me;
                 off_cand[2] = L.new_ids[bi];
