@@ -192,7 +192,7 @@ struct JoinArgs {
     const uint32_t* fwd_old;
     const uint32_t* rev_new;
     const uint32_t* rev_old;
-    const uint32_t* counts;
+    uint32_t* counts;           // num x 4: forward new / old, reverse new / old
     uint32_t* inbox_counts;
     uint2* inbox;               // num x inbox_cap (dist bits, id)
     unsigned long long* stats;  // [0] offers emitted, [1] offers dropped by a full inbox (nullable)
@@ -294,8 +294,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     if (a.segs.state[seg] == kDone) return;
     const uint32_t c_fn = c4.x, c_fo = c4.y;
     const uint32_t c_rn = c4.z < kSamples ? c4.z : kSamples, c_ro = c4.w < kSamples ? c4.w : kSamples;
+    __syncthreads();   // every thread holds the counts
+    // this list's reverse samples are consumed here and now: the counts restart for the scatter that follows the join
+    if (tid == 0) *reinterpret_cast<uint2*>(a.counts + static_cast<size_t>(node) * 4 + 2) = make_uint2(0u, 0u);
     if (c_fn + c_rn == 0) return;
-    __syncthreads();
     // forward then reverse samples, duplicates removed with an LDS hash set (reference: sort + binary search, :625-666)
     if (tid < 128) {
         const bool is_old = tid >= 64;
@@ -509,13 +511,20 @@ __device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane
 //   the list and this round's offers are sorted together by (distance, id); of the distinct offered ids only the
 //   best 32 count (the rest are dropped, as the 32-wide device list drops them); those not yet in the list enter it;
 //   new samples = those of the best 32 that the Bloom filter has not seen; the ones entering the list are flagged old.
+// add_rev_edges_kernel (:490-507) for one sample: list `node` appends itself to the reverse list of sample `id`
+__device__ __forceinline__ void reverse_append(uint32_t* counts, uint32_t* rev, uint32_t seg_start, uint32_t id, uint32_t which, uint32_t node) {
+    const uint32_t target = seg_start + id;
+    const uint32_t pos = atomicAdd(&counts[static_cast<size_t>(target) * 4 + which], 1u);
+    if (pos < kSamples) rev[static_cast<size_t>(target) * kSamples + pos] = node - seg_start;
+}
+
 // The sort network is sized by what the node holds this round (list + offers received): the keys are distinct up to
 // identical copies, so every size gives the same sorted sequence, and most nodes need far less than the largest one.
 template <int M>
 __device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t width,
                                            uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new, uint32_t* fwd_old,
                                            uint32_t* counts, unsigned long long* stats, Segments segs, uint32_t node, uint32_t seg, uint32_t raw,
-                                           uint32_t* filter, int lane) {
+                                           uint32_t* filter, int lane, uint32_t seg_start, uint32_t* rev_new, uint32_t* rev_old) {
     constexpr int NR = M / 64;
     const uint32_t bloom_words = bloom_sets * 16;
     const uint32_t n_in = raw < inbox_cap ? raw : inbox_cap;
@@ -548,7 +557,11 @@ __device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists
 #pragma unroll
         for (int r = 0; r < NR; r++) {
             if (k[r] != ~0ull && !(k[r] & 1ull) && (v[r] & kOld)) {
-                if (rank < kSamples) fwd_old[static_cast<size_t>(node) * kSamples + rank] = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+                if (rank < kSamples) {
+                    const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+                    fwd_old[static_cast<size_t>(node) * kSamples + rank] = id;
+                    if (rev_old) reverse_append(counts, rev_old, seg_start, id, 3, node);
+                }
                 rank++;
             }
         }
@@ -607,6 +620,7 @@ __device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists
         uint32_t flag = v[r];
         if (fresh[r]) {   // at most 32 of them: all become samples
             fwd_new[static_cast<size_t>(node) * kSamples + nrank] = id;
+            if (rev_new) reverse_append(counts, rev_new, seg_start, id, 2, node);
             nrank++;
             flag = kOld;
             const uint32_t base = (id % bloom_sets) * 512;
@@ -645,8 +659,10 @@ __device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists
         inbox_counts[node] = 0;
         counts[static_cast<size_t>(node) * 4 + 0] = total_new;
         counts[static_cast<size_t>(node) * 4 + 1] = total_old < kSamples ? total_old : kSamples;
-        counts[static_cast<size_t>(node) * 4 + 2] = 0;
-        counts[static_cast<size_t>(node) * 4 + 3] = 0;
+        if (!rev_new) {   // with the scatter fused in, other wavefronts are adding to these two right now; the join clears them
+            counts[static_cast<size_t>(node) * 4 + 2] = 0;
+            counts[static_cast<size_t>(node) * 4 + 3] = 0;
+        }
         if (stats) {   // striped over 1024 slots: one shared address would serialise every wavefront of the launch
             unsigned long long* slot = stats + 2 * (blockIdx.x & 1023u);
             atomicAdd(&slot[0], static_cast<unsigned long long>(raw));
@@ -658,7 +674,8 @@ __device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists
 template <int MMAX>
 __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t num,
                                                         uint32_t width, uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new,
-                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats, Segments segs) {
+                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats, Segments segs, uint32_t* rev_new,
+                                                        uint32_t* rev_old) {
     __shared__ uint32_t filter_lds[4][64];
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
@@ -674,13 +691,13 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, floa
     const uint32_t held = width + (raw < inbox_cap ? raw : inbox_cap);   // the same for every lane of the wavefront
     if (held <= 64)
         merge_node<64>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
-                       seg, raw, filter, lane);
+                       seg, raw, filter, lane, seg_start, rev_new, rev_old);
     else if (MMAX == 128 || held <= 128)
         merge_node<128>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
-                        seg, raw, filter, lane);
+                        seg, raw, filter, lane, seg_start, rev_new, rev_old);
     else
         merge_node<256>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
-                        seg, raw, filter, lane);
+                        seg, raw, filter, lane, seg_start, rev_new, rev_old);
 }
 
 // Termination test of GNND::build's update_and_sample (nn_descent.cuh:1270-1284): a partition whose sampled update
@@ -860,15 +877,19 @@ int nnd_join(const NndCtx& c) {
     return launch_status();
 }
 
-int nnd_merge(const NndCtx& c, bool with_stats) {
+// scatter_reverse: the new and old samples a node draws are appended to the reverse lists of their targets right away
+// (what the next round's nnd_reverse would do), while the sort of other nodes keeps the vector ALU busy
+int nnd_merge(const NndCtx& c, bool with_stats, bool scatter_reverse = false) {
     unsigned long long* stats = with_stats ? c.stats : nullptr;
+    uint32_t* rev_new = scatter_reverse ? c.rev_new : nullptr;
+    uint32_t* rev_old = scatter_reverse ? c.rev_old : nullptr;
     const uint32_t m = c.l.width + c.l.cap;
     if (m <= 128) {
         hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
-                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs);
+                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs, rev_new, rev_old);
     } else {
         hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
-                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs);
+                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs, rev_new, rev_old);
     }
     return launch_status();
 }
@@ -899,9 +920,9 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
     if (rc != GLIDE_OK) return rc;
     if ((rc = nnd_prepare(c, reorder_data, dim, seed)) != GLIDE_OK) return rc;
     for (uint32_t it = 0; it < iterations; it++) {
-        if ((rc = nnd_reverse(c)) != GLIDE_OK) return rc;
+        if (it == 0 && (rc = nnd_reverse(c)) != GLIDE_OK) return rc;   // later rounds: the merge of the round before has done it
         if ((rc = nnd_join(c)) != GLIDE_OK) return rc;
-        if ((rc = nnd_merge(c, stats_out != nullptr)) != GLIDE_OK) return rc;
+        if ((rc = nnd_merge(c, stats_out != nullptr, it + 1 < iterations)) != GLIDE_OK) return rc;
         if ((rc = nnd_converge(c, dim, termination_threshold)) != GLIDE_OK) return rc;
         // GNND::build leaves its loop when the update count falls below the limit (nn_descent.cuh:1270-1284).  Here the
         // partitions rest one by one on the device; once none is active the remaining rounds would only launch kernels
