@@ -1,5 +1,7 @@
 // class GLIDE_large: data, graph and map live in pinned host memory; one partition at a time is staged through the
 // GPU.  Reference: glide_large.cuh:14-212, glide_large_impl.cuh:14-507 (instantiated there for uint8 rows; uint8 or float here).
+// On a GPU that holds the whole index (rows as fp32 + graph + map; 32 GB for 50M x 128) search() uploads it once and
+// searches the partitions in place; the staged search is kept for indexes that do not fit.
 // Partitions are independent on this path (no boundary list, no cross-partition merge), so build -> reverse edges ->
 // refine run back to back on a staged partition instead of in three passes over the host arrays, and the copy of
 // the next partition overlaps the kernels of the current one.
@@ -9,6 +11,8 @@
 // merged index is searched like a small index: rows and graph resident in HBM, one kernel, no staging per query batch.
 #pragma once
 #include <cfloat>
+#include <cstdlib>
+#include <cstring>
 #include <fstream>
 #include <iostream>
 #include <optional>
@@ -247,6 +251,22 @@ public:
             search_merged(param, d_query_view, h_result_ids_view, h_result_distances_view, result_file);
             return;
         }
+        // 288 GB of HBM hold what the reference has to stage for every query batch (50M x 128 fp32 rows + graph = 32 GB):
+        // when the whole index fits it is uploaded once and the partitions are searched in place; the staged path below
+        // remains for indexes that do not fit (or when GLIDE_LARGE_STAGED is set).
+        if (!std::getenv("GLIDE_LARGE_STAGED") && !resident_failed) {
+            bool first_use = false;
+            try {
+                first_use = make_resident();
+            } catch (const hip_error&) {
+                r_data.reset(); r_graph.reset(); r_centroids.reset(); r_start_points.reset(); r_map.reset();
+                resident_failed = true;
+            }
+            if (!resident_failed) {
+                search_resident(param, min_segment_num, boundary_factor, d_query_view, h_result_ids_view, h_result_distances_view, result_file, first_use);
+                return;
+            }
+        }
         const uint32_t query_number = d_query_view.extent(0), top_k = param.top_k, deg = graph_degree(), c = centroids_num();
         device_matrix<uint32_t> d_final_ids(query_number, top_k), d_segment_ids(query_number, c);
         device_matrix<float> d_final_dists(query_number, top_k), d_centroids(c, dim());
@@ -365,6 +385,58 @@ public:
         }
     }
 
+    // The per-partition search of glide_large_impl.cuh:347-507 on an index that is resident in device memory: the same
+    // kernels on the same partitions in the same order as the staged path, without the copies.
+    void search_resident(SearchParameter& param, uint32_t min_segment_num, float boundary_factor, device_matrix_view<Data_t> d_query_view,
+                         host_matrix_view<uint32_t> h_result_ids_view, host_matrix_view<float> h_result_distances_view, std::string& result_file,
+                         bool first_use) {
+        const uint32_t query_number = d_query_view.extent(0), top_k = param.top_k, deg = graph_degree(), c = centroids_num();
+        device_matrix<uint32_t> d_final_ids(query_number, top_k), d_segment_ids(query_number, c);
+        device_matrix<float> d_final_dists(query_number, top_k);
+        device_matrix<float> d_query_f32(sizeof(Data_t) == 1 ? query_number : 0, dim());
+        const int mc = metric_code(metric);
+        void* cs = handle.stream();
+        const float fmax = FLT_MAX;
+        uint32_t fmax_bits;
+        std::memcpy(&fmax_bits, &fmax, 4);
+        auto run = [&](uint32_t queries) {
+            hip_try(glide_hip_fill_u32(d_final_ids.data_handle(), 0xffffffffu, d_final_ids.size(), cs), "glide_hip_fill_u32");
+            hip_try(glide_hip_fill_u32(reinterpret_cast<uint32_t*>(d_final_dists.data_handle()), fmax_bits, d_final_dists.size(), cs), "glide_hip_fill_u32");
+            const float* d_queries = reinterpret_cast<const float*>(d_query_view.data_handle());
+            if (sizeof(Data_t) == 1) {
+                hip_try(glide_hip_widen_u8(reinterpret_cast<const unsigned char*>(d_query_view.data_handle()), static_cast<size_t>(queries) * dim(),
+                                           d_query_f32.data_handle(), cs),
+                        "glide_hip_widen_u8");
+                d_queries = d_query_f32.data_handle();
+            }
+            hip_try(glide_hip_select_segments(d_queries, queries, dim(), r_centroids->data_handle(), c, min_segment_num, boundary_factor, mc,
+                                              d_segment_ids.data_handle(), cs),
+                    "glide_hip_select_segments");
+            for (uint32_t s = 0; s < segment_num(); s++) {
+                const size_t start = h_segment_start(s);
+                if (h_segment_length(s) == 0) continue;
+                hip_try(glide_hip_search_sub(r_data->data_handle() + start * dim(), dim(), r_graph->data_handle() + start * deg, deg,
+                                             r_map->data_handle() + start, d_queries, queries, d_segment_ids.data_handle(), c, s, h_start_point(s),
+                                             top_k, param.beam, param.max_iterations, param.min_iterations, param.hash_bit, param.hash_reset_interval,
+                                             mc, d_final_ids.data_handle(), d_final_dists.data_handle(), nullptr, cs),
+                        "glide_hip_search_sub");
+            }
+        };
+        if (first_use && query_number) run(1);   // part of bringing the index up: the first launch of a kernel loads its code
+        gpu_timer timer;
+        timer.start();
+        run(query_number);
+        const float search_time = timer.stop();
+        std::cout << "query time: " << search_time << " s" << "   " << "QPS: " << static_cast<float>(query_number) / search_time << std::endl;
+        std::ofstream result;
+        result.setf(std::ios::fixed);
+        result.open(result_file, std::ios::app);
+        result << search_time << "," << static_cast<float>(query_number) / search_time << ",";
+        result.close();
+        copy_to_host(h_result_ids_view.data_handle(), d_final_ids.data_handle(), d_final_ids.size());
+        copy_to_host(h_result_distances_view.data_handle(), d_final_dists.data_handle(), d_final_dists.size());
+    }
+
 private:
     static uint32_t upload_piece(uint32_t n) { return std::min<uint32_t>(n, 1u << 20); }
 
@@ -386,7 +458,7 @@ private:
         }
     }
 
-    // one-time upload of a merged index
+    // one-time upload of the index (rows as fp32, graph, centroids, entry points, and the map for the per-partition search)
     bool make_resident() {
         if (r_data) return false;
         const uint32_t n = point_num(), c = centroids_num(), deg = graph_degree();
@@ -406,6 +478,10 @@ private:
         for (uint32_t s = 0; s < c; s++) entry[s] = h_segment_start(s) + h_start_point(s);
         r_start_points.emplace(c);
         copy_to_device(r_start_points->data_handle(), entry.data(), c);
+        if (!merged()) {   // the per-partition search writes input row numbers itself
+            r_map.emplace(n);
+            copy_to_device(r_map->data_handle(), h_map.data_handle(), n);
+        }
         std::cout << "index upload time: " << timer.stop() << " s" << std::endl;
         return true;
     }
@@ -413,7 +489,8 @@ private:
     std::optional<device_matrix<float>> r_data;
     std::optional<device_matrix<uint32_t>> r_graph;
     std::optional<device_matrix<float>> r_centroids;
-    std::optional<device_vector<uint32_t>> r_start_points;
+    std::optional<device_vector<uint32_t>> r_start_points, r_map;
+    bool resident_failed = false;
     device_resources& handle;
     Metric metric;
     pinned_matrix<Data_t> h_data;

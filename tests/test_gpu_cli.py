@@ -11,8 +11,8 @@ pytestmark = pytest.mark.gpu
 BIN = os.path.join(ROOT, "glide_amd", "bin")
 
 
-def run(*args):
-    r = subprocess.run([str(a) for a in args], capture_output=True, text=True, timeout=300)
+def run(*args, env=None):
+    r = subprocess.run([str(a) for a in args], capture_output=True, text=True, timeout=300, env=None if env is None else {**os.environ, **env})
     assert r.returncode == 0, r.stdout + r.stderr
     return r.stdout
 
@@ -136,8 +136,14 @@ def test_large_pipeline_cli(tmp_path):
     for i, (s, l) in enumerate(zip(starts.tolist(), lengths.tolist())):
         O.search_sub(rdata[s:s + l], graph[s:s + l], mp[s:s + l], queries, seg_ids, i, int(sp[i]), 10, spp, e_ids, e_d)
     assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= 0.9
+    assert "index upload time" in out        # the index fits the GPU: uploaded once, partitions searched in place
     row = open(result).read().strip().splitlines()[1].split(",")
     assert len(row) == 8
+    # the staged search (every partition copied from host memory for the batch, as the reference does) gives the same answer
+    out2 = run(os.path.join(BIN, "large_search"), pre, f("query.fbin"), f("truth"), graph_base, f("result2.csv"), "Euclidean", 10, 50, 2, 1.1,
+               env={"GLIDE_LARGE_STAGED": "1"})
+    assert "index upload time" not in out2
+    assert float(out2.split("total_recall:")[1].split()[0]) == recall
 
 
 def test_large_merged_pipeline_cli(tmp_path):
