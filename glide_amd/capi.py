@@ -410,6 +410,24 @@ def select_segments(queries, query_num, dim, centroids, centroid_num, min_segmen
                                           _ptr(segment_ids), vp(stream)), "glide_hip_select_segments")
 
 
+def group_queries(segment_ids, query_num, centroid_num, counts, offsets, lists, stream=None):
+    wb = int(_size_fn("glide_hip_group_queries_workspace_bytes")(u32(centroid_num)))
+    ws = DeviceArray(wb // 4 + 1, np.uint32)
+    check(lib().glide_hip_group_queries(_ptr(segment_ids), u32(query_num), u32(centroid_num), _ptr(counts), _ptr(offsets), _ptr(lists),
+                                        _ptr(ws), C.c_size_t(wb), vp(stream)), "glide_hip_group_queries")
+    synchronize(stream)      # the workspace is released on return
+
+
+def search_sub_listed(segment_data, dim, segment_graph, graph_degree, segment_map, queries, query_num, query_list, list_len,
+                      segment_id, start_point, top_k, beam, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric,
+                      final_ids, final_dists, counters=None, stream=None):
+    check(lib().glide_hip_search_sub_listed(_ptr(segment_data), u32(dim), _ptr(segment_graph), u32(graph_degree), _ptr(segment_map),
+                                            _ptr(queries), u32(query_num), _ptr(query_list), u32(list_len), u32(segment_id),
+                                            u32(start_point), u32(top_k), u32(beam), u32(max_iterations), u32(min_iterations),
+                                            u32(hash_bit), u32(hash_reset_interval), C.c_int(metric), _ptr(final_ids), _ptr(final_dists),
+                                            _ptr(counters), vp(stream)), "glide_hip_search_sub_listed")
+
+
 def search_sub(segment_data, dim, segment_graph, graph_degree, segment_map, queries, query_num, segment_ids,
                centroid_num, segment_id, start_point, top_k, beam, max_iterations, min_iterations, hash_bit,
                hash_reset_interval, metric, final_ids, final_dists, counters=None, stream=None):

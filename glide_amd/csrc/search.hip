@@ -142,16 +142,44 @@ __global__ __launch_bounds__(64) void select_segments_kernel(SelectArgs a) {
     }
 }
 
+// Queries grouped by the partitions they selected: counts, then offsets, then the lists.  With them a partition's
+// search launches one wavefront per query that wants it instead of one per query of the batch.
+__global__ __launch_bounds__(256) void group_count_kernel(const uint32_t* segment_ids, uint32_t total, uint32_t centroid_num, uint32_t* counts) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t s = segment_ids[i];
+    if (s < centroid_num) atomicAdd(&counts[s], 1u);
+}
+__global__ __launch_bounds__(256) void group_scan_kernel(uint32_t* counts, uint32_t centroid_num, uint32_t* offsets, uint32_t* cursor) {
+    if (threadIdx.x == 0) {
+        uint32_t run = 0;
+        for (uint32_t s = 0; s < centroid_num; s++) {
+            offsets[s] = run;
+            cursor[s] = run;
+            run += counts[s];
+        }
+        offsets[centroid_num] = run;
+    }
+}
+__global__ __launch_bounds__(256) void group_fill_kernel(const uint32_t* segment_ids, uint32_t total, uint32_t centroid_num, uint32_t* cursor,
+                                                         uint32_t* lists) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t s = segment_ids[i];
+    if (s < centroid_num) lists[atomicAdd(&cursor[s], 1u)] = i / centroid_num;
+}
+
 struct SubArgs {
     const float* data;          // the staged partition
     const uint32_t* graph;      // partition-local ids
     const uint32_t* map;        // local id -> original id
     const float* queries;
     const uint32_t* segment_ids;
+    const uint32_t* query_list;   // nullable: the queries that selected this partition (then segment_ids is not read)
     uint32_t* final_ids;
     float* final_dists;
     unsigned long long* counters;
-    uint32_t query_num, centroid_num, segment_id, start_point, top_k, max_topk;
+    uint32_t query_num, centroid_num, segment_id, start_point, top_k, max_topk, list_len;
     BeamParams p;
 };
 
@@ -196,15 +224,20 @@ __global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
     float* head_dist = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>));   // beam head staged for the merge (128 pairs)
     uint32_t* head_id = reinterpret_cast<uint32_t*>(head_dist + 128);
     uint32_t* hash = head_id + 128;
-    const uint32_t qid = blockIdx.x;
-    if (qid >= a.query_num) return;
-    bool is_search = false;   // wave-uniform scan of this query's partition list
-    for (uint32_t i = 0; i < a.centroid_num; i++) {
-        const uint32_t s = a.segment_ids[static_cast<size_t>(qid) * a.centroid_num + i];
-        if (s == a.segment_id) { is_search = true; break; }
-        if (s == kInvalid) break;
+    uint32_t qid = blockIdx.x;
+    if (a.query_list) {
+        if (qid >= a.list_len) return;
+        qid = a.query_list[qid];
+    } else {
+        if (qid >= a.query_num) return;
+        bool is_search = false;   // wave-uniform scan of this query's partition list
+        for (uint32_t i = 0; i < a.centroid_num; i++) {
+            const uint32_t s = a.segment_ids[static_cast<size_t>(qid) * a.centroid_num + i];
+            if (s == a.segment_id) { is_search = true; break; }
+            if (s == kInvalid) break;
+        }
+        if (!is_search) return;
     }
-    if (!is_search) return;
 
     Beam<MAX_CAND, MAX_BEAM, DIMV> b;
     b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
@@ -377,15 +410,17 @@ extern "C" int glide_hip_select_segments(const float* queries, uint32_t query_nu
     return launch_status();
 }
 
-extern "C" int glide_hip_search_sub(const float* segment_data, uint32_t dim, const uint32_t* segment_graph, uint32_t graph_degree,
-                                    const uint32_t* segment_map, const float* queries, uint32_t query_num, const uint32_t* segment_ids,
-                                    uint32_t centroid_num, uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam,
-                                    uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
-                                    int metric, uint32_t* final_ids, float* final_dists, unsigned long long* counters, void* stream) {
-    if (!segment_data || !segment_graph || !segment_map || !queries || !segment_ids || !final_ids || !final_dists) return GLIDE_ERR_BAD_ARGUMENT;
+namespace {
+int launch_search_sub(const float* segment_data, uint32_t dim, const uint32_t* segment_graph, uint32_t graph_degree, const uint32_t* segment_map,
+                      const float* queries, uint32_t query_num, const uint32_t* segment_ids, const uint32_t* query_list, uint32_t list_len,
+                      uint32_t centroid_num, uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam, uint32_t max_iterations,
+                      uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, int metric, uint32_t* final_ids,
+                      float* final_dists, unsigned long long* counters, void* stream) {
+    if (!segment_data || !segment_graph || !segment_map || !queries || (!segment_ids && !query_list) || !final_ids || !final_dists)
+        return GLIDE_ERR_BAD_ARGUMENT;
     if (dim == 0 || graph_degree == 0 || centroid_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
-    if (query_num == 0) return GLIDE_OK;
+    if (query_num == 0 || (query_list && list_len == 0)) return GLIDE_OK;
     if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 1024 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;   // top_k buckets: kernel_config.cuh:312-323
     SubArgs a;
@@ -394,6 +429,8 @@ extern "C" int glide_hip_search_sub(const float* segment_data, uint32_t dim, con
     a.map = segment_map;
     a.queries = queries;
     a.segment_ids = segment_ids;
+    a.query_list = query_list;
+    a.list_len = list_len;
     a.final_ids = final_ids;
     a.final_dists = final_dists;
     a.counters = counters;
@@ -407,6 +444,47 @@ extern "C" int glide_hip_search_sub(const float* segment_data, uint32_t dim, con
     sub_fn fn = graph_degree <= 64 ? pick_sub_beam<64>(beam, dim) : graph_degree <= 128 ? pick_sub_beam<128>(beam, dim) : pick_sub_beam<256>(beam, dim);
     const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-    hipLaunchKernelGGL(fn, dim3(query_num), dim3(64), lds_bytes, as_stream(stream), a);
+    hipLaunchKernelGGL(fn, dim3(query_list ? list_len : query_num), dim3(64), lds_bytes, as_stream(stream), a);
+    return launch_status();
+}
+}  // namespace
+
+extern "C" int glide_hip_search_sub(const float* segment_data, uint32_t dim, const uint32_t* segment_graph, uint32_t graph_degree,
+                                    const uint32_t* segment_map, const float* queries, uint32_t query_num, const uint32_t* segment_ids,
+                                    uint32_t centroid_num, uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam,
+                                    uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
+                                    int metric, uint32_t* final_ids, float* final_dists, unsigned long long* counters, void* stream) {
+    if (!segment_ids) return GLIDE_ERR_BAD_ARGUMENT;
+    return launch_search_sub(segment_data, dim, segment_graph, graph_degree, segment_map, queries, query_num, segment_ids, nullptr, 0, centroid_num,
+                             segment_id, start_point, top_k, beam, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric, final_ids,
+                             final_dists, counters, stream);
+}
+
+extern "C" int glide_hip_search_sub_listed(const float* segment_data, uint32_t dim, const uint32_t* segment_graph, uint32_t graph_degree,
+                                           const uint32_t* segment_map, const float* queries, uint32_t query_num, const uint32_t* query_list,
+                                           uint32_t list_len, uint32_t segment_id, uint32_t start_point, uint32_t top_k, uint32_t beam,
+                                           uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
+                                           int metric, uint32_t* final_ids, float* final_dists, unsigned long long* counters, void* stream) {
+    if (!query_list && list_len) return GLIDE_ERR_BAD_ARGUMENT;
+    if (list_len == 0) return GLIDE_OK;
+    return launch_search_sub(segment_data, dim, segment_graph, graph_degree, segment_map, queries, query_num, nullptr, query_list, list_len, 1,
+                             segment_id, start_point, top_k, beam, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric, final_ids,
+                             final_dists, counters, stream);
+}
+
+extern "C" size_t glide_hip_group_queries_workspace_bytes(uint32_t centroid_num) { return (static_cast<size_t>(centroid_num) + 1) * 4 + 256; }
+
+extern "C" int glide_hip_group_queries(const uint32_t* segment_ids, uint32_t query_num, uint32_t centroid_num, uint32_t* counts, uint32_t* offsets,
+                                       uint32_t* lists, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!segment_ids || !counts || !offsets || !lists || !workspace || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (workspace_bytes < glide_hip_group_queries_workspace_bytes(centroid_num)) return GLIDE_ERR_BAD_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    int rc = glide_hip_fill_u32(counts, 0u, centroid_num, stream);
+    if (rc != GLIDE_OK) return rc;
+    const uint32_t total = query_num * centroid_num;
+    uint32_t* cursor = static_cast<uint32_t*>(workspace);
+    if (total) hipLaunchKernelGGL(group_count_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s, segment_ids, total, centroid_num, counts);
+    hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(256), 0, s, counts, centroid_num, offsets, cursor);
+    if (total) hipLaunchKernelGGL(group_fill_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s, segment_ids, total, centroid_num, cursor, lists);
     return launch_status();
 }

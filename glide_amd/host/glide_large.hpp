@@ -394,6 +394,11 @@ public:
         device_matrix<uint32_t> d_final_ids(query_number, top_k), d_segment_ids(query_number, c);
         device_matrix<float> d_final_dists(query_number, top_k);
         device_matrix<float> d_query_f32(sizeof(Data_t) == 1 ? query_number : 0, dim());
+        device_vector<uint32_t> d_counts(c), d_offsets(c + 1);
+        device_matrix<uint32_t> d_lists(query_number ? query_number : 1, c);
+        const size_t gwb = glide_hip_group_queries_workspace_bytes(c);
+        device_buffer group_ws(gwb);
+        std::vector<uint32_t> offsets(c + 1);
         const int mc = metric_code(metric);
         void* cs = handle.stream();
         const float fmax = FLT_MAX;
@@ -412,14 +417,20 @@ public:
             hip_try(glide_hip_select_segments(d_queries, queries, dim(), r_centroids->data_handle(), c, min_segment_num, boundary_factor, mc,
                                               d_segment_ids.data_handle(), cs),
                     "glide_hip_select_segments");
+            // the queries of each partition, so that a partition launches one wavefront per query that selected it
+            hip_try(glide_hip_group_queries(d_segment_ids.data_handle(), queries, c, d_counts.data_handle(), d_offsets.data_handle(),
+                                            d_lists.data_handle(), group_ws.get(), gwb, cs),
+                    "glide_hip_group_queries");
+            hip_try(glide_hip_memcpy_d2h(offsets.data(), d_offsets.data_handle(), (c + 1) * sizeof(uint32_t), cs), "glide_hip_memcpy_d2h");
             for (uint32_t s = 0; s < segment_num(); s++) {
                 const size_t start = h_segment_start(s);
-                if (h_segment_length(s) == 0) continue;
-                hip_try(glide_hip_search_sub(r_data->data_handle() + start * dim(), dim(), r_graph->data_handle() + start * deg, deg,
-                                             r_map->data_handle() + start, d_queries, queries, d_segment_ids.data_handle(), c, s, h_start_point(s),
-                                             top_k, param.beam, param.max_iterations, param.min_iterations, param.hash_bit, param.hash_reset_interval,
-                                             mc, d_final_ids.data_handle(), d_final_dists.data_handle(), nullptr, cs),
-                        "glide_hip_search_sub");
+                const uint32_t wanted = offsets[s + 1] - offsets[s];
+                if (h_segment_length(s) == 0 || wanted == 0) continue;
+                hip_try(glide_hip_search_sub_listed(r_data->data_handle() + start * dim(), dim(), r_graph->data_handle() + start * deg, deg,
+                                                    r_map->data_handle() + start, d_queries, queries, d_lists.data_handle() + offsets[s], wanted, s,
+                                                    h_start_point(s), top_k, param.beam, param.max_iterations, param.min_iterations, param.hash_bit,
+                                                    param.hash_reset_interval, mc, d_final_ids.data_handle(), d_final_dists.data_handle(), nullptr, cs),
+                        "glide_hip_search_sub_listed");
             }
         };
         if (first_use && query_number) run(1);   // part of bringing the index up: the first launch of a kernel loads its code

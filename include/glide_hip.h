@@ -245,6 +245,23 @@ int glide_hip_refine(const float *data, uint32_t num, uint32_t dim, const uint32
  * partition-local); the caller stages them (the reference copies each partition from host memory,
  * glide_large_impl.cuh:109-166).  Data type: float (the reference's large executables instantiate uint8). */
 
+/* Queries grouped by the partitions they selected (no counterpart in the reference, whose search_on_sub_kernel starts
+ * one block per query of the batch for every partition and lets the blocks of other partitions return at once).
+ * segment_ids: query_num x centroid_num from glide_hip_select_segments.  counts (centroid_num u32) and offsets
+ * (centroid_num + 1 u32) describe lists (at most query_num x centroid_num u32): the queries that selected partition
+ * s are lists[offsets[s] .. offsets[s + 1]), in no particular order.  All device arrays. */
+size_t glide_hip_group_queries_workspace_bytes(uint32_t centroid_num);
+int glide_hip_group_queries(const uint32_t *segment_ids, uint32_t query_num, uint32_t centroid_num, uint32_t *counts,
+                            uint32_t *offsets, uint32_t *lists, void *workspace, size_t workspace_bytes, void *stream);
+
+/* glide_hip_search_sub for the queries named in query_list (list_len of them) instead of a scan of segment_ids. */
+int glide_hip_search_sub_listed(const float *segment_data, uint32_t dim, const uint32_t *segment_graph,
+                                uint32_t graph_degree, const uint32_t *segment_map, const float *queries,
+                                uint32_t query_num, const uint32_t *query_list, uint32_t list_len, uint32_t segment_id,
+                                uint32_t start_point, uint32_t top_k, uint32_t beam, uint32_t max_iterations,
+                                uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, int metric,
+                                uint32_t *final_ids, float *final_dists, unsigned long long *counters, void *stream);
+
 /* ---- merged large build (GLIDE_large::build_with_merge, declared at glide_large.cuh:89-97 without a definition) --
  * The merged graph lives in device memory in reorder-id space: row r belongs to reorder row r (r < num) and holds
  * reorder ids.  The two passes below are the large-path forms of map_to_graph (graph_kernel.cuh:145-150) and

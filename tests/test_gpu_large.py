@@ -98,6 +98,22 @@ def test_search_over_partitions_bit_exact(hip, large_index, top_k, beam):
         assert np.array_equal(g_d.numpy(), e_d), s
     gt, _ = O.bruteforce_knn(L["data"], L["queries"], 10)
     assert recall(e_ids[:, :10], gt, 10) >= 0.9          # two partitions per query
+    # the same through the grouped form: each partition launches only the queries that selected it
+    c = 3
+    counts, offsets, lists = hip.DeviceArray(c, np.uint32), hip.DeviceArray(c + 1, np.uint32), hip.DeviceArray(nq * c, np.uint32)
+    hip.group_queries(d_seg, nq, c, counts, offsets, lists)
+    h_counts, h_off, h_lists = counts.numpy(), offsets.numpy(), lists.numpy()
+    assert np.array_equal(h_counts, [(seg_ids == s).sum() for s in range(c)]) and np.array_equal(h_off, np.concatenate([[0], np.cumsum(h_counts)]))
+    for s in range(c):
+        assert np.array_equal(np.sort(h_lists[h_off[s]:h_off[s + 1]]), np.flatnonzero((seg_ids == s).any(axis=1)))
+    l_ids = hip.DeviceArray.from_numpy(np.full((nq, top_k), INV, np.uint32))
+    l_d = hip.DeviceArray.from_numpy(np.full((nq, top_k), np.finfo(np.float32).max, np.float32))
+    for s, seg in enumerate(L["segs"]):
+        d_data, d_graph, d_map = hip.DeviceArray.from_numpy(seg["data"]), hip.DeviceArray.from_numpy(seg["graph"]), hip.DeviceArray.from_numpy(seg["map"])
+        hip.search_sub_listed(d_data, 128, d_graph, 32, d_map, d_q, nq, lists.ptr + 4 * int(h_off[s]), int(h_counts[s]), s, int(L["start_points"][s]),
+                              top_k, sp["beam"], sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 0, l_ids, l_d)
+        hip.synchronize()
+    assert np.array_equal(l_ids.numpy(), e_ids) and np.array_equal(l_d.numpy(), e_d)
 
 
 def test_place_and_merge_boundary_bit_exact(hip):
