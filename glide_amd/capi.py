@@ -428,6 +428,19 @@ def search_sub_listed(segment_data, dim, segment_graph, graph_degree, segment_ma
                                             _ptr(counters), vp(stream)), "glide_hip_search_sub_listed")
 
 
+def search_partitions(data, dim, graph, graph_degree, mp, segment_starts, segment_start_points, segment_num, queries, query_num,
+                      segment_ids, top_k, beam, max_iterations, min_iterations, hash_bit, hash_reset_interval, metric, final_ids,
+                      final_dists, counters=None, stream=None):
+    wb = int(_size_fn("glide_hip_search_partitions_workspace_bytes")(u32(query_num), u32(segment_num), u32(top_k)))
+    ws = DeviceArray(wb // 8 + 1, np.uint64)
+    check(lib().glide_hip_search_partitions(_ptr(data), u32(dim), _ptr(graph), u32(graph_degree), _ptr(mp), _ptr(segment_starts),
+                                            _ptr(segment_start_points), u32(segment_num), _ptr(queries), u32(query_num), _ptr(segment_ids),
+                                            u32(top_k), u32(beam), u32(max_iterations), u32(min_iterations), u32(hash_bit),
+                                            u32(hash_reset_interval), C.c_int(metric), _ptr(final_ids), _ptr(final_dists), _ptr(ws),
+                                            C.c_size_t(wb), _ptr(counters), vp(stream)), "glide_hip_search_partitions")
+    synchronize(stream)      # the workspace is released on return
+
+
 def search_sub(segment_data, dim, segment_graph, graph_degree, segment_map, queries, query_num, segment_ids,
                centroid_num, segment_id, start_point, top_k, beam, max_iterations, min_iterations, hash_bit,
                hash_reset_interval, metric, final_ids, final_dists, counters=None, stream=None):

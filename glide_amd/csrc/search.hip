@@ -162,11 +162,94 @@ __global__ __launch_bounds__(256) void group_scan_kernel(uint32_t* counts, uint3
     }
 }
 __global__ __launch_bounds__(256) void group_fill_kernel(const uint32_t* segment_ids, uint32_t total, uint32_t centroid_num, uint32_t* cursor,
-                                                         uint32_t* lists) {
+                                                         uint32_t* lists, uint32_t* pair_segment, uint32_t* pair_index) {
     const uint32_t i = blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const uint32_t s = segment_ids[i];
-    if (s < centroid_num) lists[atomicAdd(&cursor[s], 1u)] = i / centroid_num;
+    uint32_t pos = kInvalid;
+    if (s < centroid_num) {
+        pos = atomicAdd(&cursor[s], 1u);
+        lists[pos] = i / centroid_num;
+        if (pair_segment) pair_segment[pos] = s;
+    }
+    if (pair_index) pair_index[i] = pos;
+}
+
+// Per query: the heads its pairs left behind are merged in ascending partition order, the order in which the
+// partition-by-partition search merges them (result_merge, search_kernel.cuh:609-651), so the result is the same.
+template <int MAX_TOPK>
+__device__ __forceinline__ void merge_pairs(const uint32_t* segment_ids, const uint32_t* pair_index, const float* pair_dists, const uint32_t* pair_ids,
+                                            uint32_t centroid_num, uint32_t top_k, float* final_dists, uint32_t* final_ids, int lane) {
+    constexpr int NR = WaveNet<MAX_TOPK>::NR;
+    const bool live = MAX_TOPK >= 64 || lane < 32;
+    float k[NR];
+    uint32_t v[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        k[r] = FLT_MAX;
+        v[r] = kInvalid;
+    }
+    uint32_t last = kInvalid;   // partition merged last; the first pass takes the smallest id
+    for (;;) {
+        uint32_t best = kInvalid, best_slot = 0;
+        for (uint32_t i = lane; i < centroid_num; i += 64) {
+            const uint32_t s = segment_ids[i];
+            if (s != kInvalid && (last == kInvalid || s > last) && s < best) { best = s; best_slot = i; }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const uint32_t ob = __shfl_xor(best, off), os = __shfl_xor(best_slot, off);
+            if (ob < best) { best = ob; best_slot = os; }
+        }
+        if (best == kInvalid) break;
+        last = best;
+        const uint32_t p = pair_index[best_slot];
+        const float* bd = pair_dists + static_cast<size_t>(p) * top_k;
+        const uint32_t* bi = pair_ids + static_cast<size_t>(p) * top_k;
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            const uint32_t e = NR * lane + r;
+            const uint32_t kk = MAX_TOPK - 1 - e;
+            if (live && kk < top_k) {
+                const float rk = bd[kk];
+                if (k[r] > rk) {
+                    k[r] = rk;
+                    v[r] = bi[kk];
+                }
+            }
+        }
+        WaveNet<MAX_TOPK>::merge(k, v, lane);
+#pragma unroll
+        for (int r = 0; r < NR; r++) {   // what the stored running result holds between two merges: top_k entries
+            const uint32_t e = NR * lane + r;
+            if (!(live && e < top_k)) { k[r] = FLT_MAX; v[r] = kInvalid; }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        if (live && e < top_k) {
+            final_dists[e] = k[r];
+            final_ids[e] = v[r];
+        }
+    }
+}
+
+__global__ __launch_bounds__(64) void merge_pairs_kernel(const uint32_t* segment_ids, const uint32_t* pair_index, const float* pair_dists,
+                                                         const uint32_t* pair_ids, uint32_t query_num, uint32_t centroid_num, uint32_t top_k,
+                                                         uint32_t max_topk, float* final_dists, uint32_t* final_ids) {
+    const uint32_t q = blockIdx.x;
+    if (q >= query_num) return;
+    const int lane = lane_id();
+    const uint32_t* seg = segment_ids + static_cast<size_t>(q) * centroid_num;
+    const uint32_t* idx = pair_index + static_cast<size_t>(q) * centroid_num;
+    float* fd = final_dists + static_cast<size_t>(q) * top_k;
+    uint32_t* fi = final_ids + static_cast<size_t>(q) * top_k;
+    switch (max_topk) {
+        case 32: merge_pairs<32>(seg, idx, pair_dists, pair_ids, centroid_num, top_k, fd, fi, lane); break;
+        case 64: merge_pairs<64>(seg, idx, pair_dists, pair_ids, centroid_num, top_k, fd, fi, lane); break;
+        default: merge_pairs<128>(seg, idx, pair_dists, pair_ids, centroid_num, top_k, fd, fi, lane); break;
+    }
 }
 
 struct SubArgs {
@@ -176,6 +259,13 @@ struct SubArgs {
     const float* queries;
     const uint32_t* segment_ids;
     const uint32_t* query_list;   // nullable: the queries that selected this partition (then segment_ids is not read)
+    // pair mode (nullable pair_segment): block p searches query query_list[p] in partition pair_segment[p]; data / graph /
+    // map are then the arrays of all partitions, addressed through segment_starts, and the beam head goes to pair_dists / pair_ids
+    const uint32_t* pair_segment;
+    const uint32_t* segment_starts;
+    const uint32_t* segment_start_points;
+    float* pair_dists;
+    uint32_t* pair_ids;
     uint32_t* final_ids;
     float* final_dists;
     unsigned long long* counters;
@@ -225,7 +315,27 @@ __global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
     uint32_t* head_id = reinterpret_cast<uint32_t*>(head_dist + 128);
     uint32_t* hash = head_id + 128;
     uint32_t qid = blockIdx.x;
-    if (a.query_list) {
+    const float* data = a.data;
+    const uint32_t* graph = a.graph;
+    const uint32_t* map = a.map;
+    uint32_t start_point = a.start_point;
+    if (a.pair_segment) {
+        if (qid >= a.list_len) return;
+        const uint32_t seg = a.pair_segment[qid];
+        const size_t start = a.segment_starts[seg];
+        data += start * a.p.dim;
+        graph += start * a.p.degree;
+        map += start;
+        start_point = a.segment_start_points[seg];
+        if (start_point == kInvalid) {   // an empty partition: nothing to find
+            for (uint32_t e = lane_id(); e < a.top_k; e += 64) {
+                a.pair_dists[static_cast<size_t>(blockIdx.x) * a.top_k + e] = FLT_MAX;
+                a.pair_ids[static_cast<size_t>(blockIdx.x) * a.top_k + e] = kInvalid;
+            }
+            return;
+        }
+        qid = a.query_list[qid];
+    } else if (a.query_list) {
         if (qid >= a.list_len) return;
         qid = a.query_list[qid];
     } else {
@@ -241,10 +351,23 @@ __global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
 
     Beam<MAX_CAND, MAX_BEAM, DIMV> b;
     b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
-    b.expand(a.start_point, a.graph, a.data, kInvalid, kInvalid);   // get_init with point_id = 0xffffffff
-    b.run(a.graph, a.data, kInvalid);
+    b.expand(start_point, graph, data, kInvalid, kInvalid);   // get_init with point_id = 0xffffffff
+    b.run(graph, data, kInvalid);
 
     constexpr int NB = MAX_BEAM / 64;
+    if (a.pair_segment) {   // the head of this pair's beam, ids already as input row numbers; merged per query afterwards
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t e = NB * b.lane + r;
+            if (e < a.top_k) {
+                const float d = b.bk[r];
+                a.pair_dists[static_cast<size_t>(blockIdx.x) * a.top_k + e] = d;
+                a.pair_ids[static_cast<size_t>(blockIdx.x) * a.top_k + e] = d < FLT_MAX ? map[b.bv[r] & kClean] : kInvalid;
+            }
+        }
+        b.flush_counters(a.counters);
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < NB; r++) {
         const uint32_t e = NB * b.lane + r;
@@ -257,9 +380,9 @@ __global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
     float* fd = a.final_dists + static_cast<size_t>(qid) * a.top_k;
     uint32_t* fi = a.final_ids + static_cast<size_t>(qid) * a.top_k;
     switch (a.max_topk) {   // kernel_config.cuh:312-323
-        case 32: merge_result<32, MAX_BEAM>(head_dist, head_id, a.map, fd, fi, a.top_k, b.lane); break;
-        case 64: merge_result<64, MAX_BEAM>(head_dist, head_id, a.map, fd, fi, a.top_k, b.lane); break;
-        default: merge_result<128, MAX_BEAM>(head_dist, head_id, a.map, fd, fi, a.top_k, b.lane); break;
+        case 32: merge_result<32, MAX_BEAM>(head_dist, head_id, map, fd, fi, a.top_k, b.lane); break;
+        case 64: merge_result<64, MAX_BEAM>(head_dist, head_id, map, fd, fi, a.top_k, b.lane); break;
+        default: merge_result<128, MAX_BEAM>(head_dist, head_id, map, fd, fi, a.top_k, b.lane); break;
     }
     b.flush_counters(a.counters);
 }
@@ -431,6 +554,11 @@ int launch_search_sub(const float* segment_data, uint32_t dim, const uint32_t* s
     a.segment_ids = segment_ids;
     a.query_list = query_list;
     a.list_len = list_len;
+    a.pair_segment = nullptr;
+    a.segment_starts = nullptr;
+    a.segment_start_points = nullptr;
+    a.pair_dists = nullptr;
+    a.pair_ids = nullptr;
     a.final_ids = final_ids;
     a.final_dists = final_dists;
     a.counters = counters;
@@ -485,6 +613,101 @@ extern "C" int glide_hip_group_queries(const uint32_t* segment_ids, uint32_t que
     uint32_t* cursor = static_cast<uint32_t*>(workspace);
     if (total) hipLaunchKernelGGL(group_count_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s, segment_ids, total, centroid_num, counts);
     hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(256), 0, s, counts, centroid_num, offsets, cursor);
-    if (total) hipLaunchKernelGGL(group_fill_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s, segment_ids, total, centroid_num, cursor, lists);
+    if (total) hipLaunchKernelGGL(group_fill_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s, segment_ids, total, centroid_num, cursor, lists,
+                                  static_cast<uint32_t*>(nullptr), static_cast<uint32_t*>(nullptr));
+    return launch_status();
+}
+
+namespace {
+size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+struct PartitionSearchLayout { size_t counts, offsets, cursor, lists, pair_segment, pair_index, pair_dists, pair_ids, total; };
+PartitionSearchLayout partition_search_layout(uint32_t query_num, uint32_t centroid_num, uint32_t top_k) {
+    PartitionSearchLayout l;
+    const size_t pairs = static_cast<size_t>(query_num) * centroid_num;   // every query could select every partition
+    size_t off = 0;
+    auto take = [&off](size_t bytes) { size_t o = off; off += align256(bytes); return o; };
+    l.counts = take(static_cast<size_t>(centroid_num) * 4);
+    l.offsets = take((static_cast<size_t>(centroid_num) + 1) * 4);
+    l.cursor = take(static_cast<size_t>(centroid_num) * 4);
+    l.lists = take(pairs * 4);
+    l.pair_segment = take(pairs * 4);
+    l.pair_index = take(pairs * 4);
+    l.pair_dists = take(pairs * top_k * 4);
+    l.pair_ids = take(pairs * top_k * 4);
+    l.total = off;
+    return l;
+}
+}  // namespace
+
+extern "C" size_t glide_hip_search_partitions_workspace_bytes(uint32_t query_num, uint32_t centroid_num, uint32_t top_k) {
+    return partition_search_layout(query_num, centroid_num, top_k).total;
+}
+
+extern "C" int glide_hip_search_partitions(const float* data, uint32_t dim, const uint32_t* graph, uint32_t graph_degree, const uint32_t* map,
+                                           const uint32_t* segment_starts, const uint32_t* segment_start_points, uint32_t segment_num,
+                                           const float* queries, uint32_t query_num, const uint32_t* segment_ids, uint32_t top_k, uint32_t beam,
+                                           uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval,
+                                           int metric, uint32_t* final_ids, float* final_dists, void* workspace, size_t workspace_bytes,
+                                           unsigned long long* counters, void* stream) {
+    if (!data || !graph || !map || !segment_starts || !segment_start_points || !queries || !segment_ids || !final_ids || !final_dists || !workspace)
+        return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim == 0 || graph_degree == 0 || segment_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
+    if (query_num == 0) return GLIDE_OK;
+    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 1024 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
+        return GLIDE_ERR_UNSUPPORTED;
+    const PartitionSearchLayout l = partition_search_layout(query_num, segment_num, top_k);
+    if (workspace_bytes < l.total || reinterpret_cast<uintptr_t>(workspace) % 8) return GLIDE_ERR_BAD_ARGUMENT;
+    hipStream_t s = as_stream(stream);
+    unsigned char* w = static_cast<unsigned char*>(workspace);
+    uint32_t* counts = reinterpret_cast<uint32_t*>(w + l.counts);
+    uint32_t* offsets = reinterpret_cast<uint32_t*>(w + l.offsets);
+    uint32_t* cursor = reinterpret_cast<uint32_t*>(w + l.cursor);
+    uint32_t* lists = reinterpret_cast<uint32_t*>(w + l.lists);
+    uint32_t* pair_segment = reinterpret_cast<uint32_t*>(w + l.pair_segment);
+    uint32_t* pair_index = reinterpret_cast<uint32_t*>(w + l.pair_index);
+    float* pair_dists = reinterpret_cast<float*>(w + l.pair_dists);
+    uint32_t* pair_ids = reinterpret_cast<uint32_t*>(w + l.pair_ids);
+    int rc = glide_hip_fill_u32(counts, 0u, segment_num, stream);
+    if (rc != GLIDE_OK) return rc;
+    const uint32_t total = query_num * segment_num;
+    hipLaunchKernelGGL(group_count_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s, segment_ids, total, segment_num, counts);
+    hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(256), 0, s, counts, segment_num, offsets, cursor);
+    hipLaunchKernelGGL(group_fill_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s, segment_ids, total, segment_num, cursor, lists, pair_segment,
+                       pair_index);
+    uint32_t pairs = 0;   // the grid of the search: one wavefront per (query, selected partition)
+    GLIDE_HIP_TRY(hipMemcpyAsync(&pairs, offsets + segment_num, sizeof(uint32_t), hipMemcpyDeviceToHost, s));
+    GLIDE_HIP_TRY(hipStreamSynchronize(s));
+    if (pairs) {
+        SubArgs a;
+        a.data = data;
+        a.graph = graph;
+        a.map = map;
+        a.queries = queries;
+        a.segment_ids = nullptr;
+        a.query_list = lists;
+        a.pair_segment = pair_segment;
+        a.segment_starts = segment_starts;
+        a.segment_start_points = segment_start_points;
+        a.pair_dists = pair_dists;
+        a.pair_ids = pair_ids;
+        a.final_ids = nullptr;
+        a.final_dists = nullptr;
+        a.counters = counters;
+        a.query_num = query_num;
+        a.centroid_num = segment_num;
+        a.segment_id = 0;
+        a.start_point = 0;
+        a.top_k = top_k;
+        a.max_topk = top_k <= 32 ? 32 : (top_k <= 64 ? 64 : 128);
+        a.list_len = pairs;
+        a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
+        sub_fn fn = graph_degree <= 64 ? pick_sub_beam<64>(beam, dim) : graph_degree <= 128 ? pick_sub_beam<128>(beam, dim) : pick_sub_beam<256>(beam, dim);
+        const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+        GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
+        hipLaunchKernelGGL(fn, dim3(pairs), dim3(64), lds_bytes, s, a);
+    }
+    hipLaunchKernelGGL(merge_pairs_kernel, dim3(query_num), dim3(64), 0, s, segment_ids, pair_index, pair_dists, pair_ids, query_num, segment_num, top_k,
+                       top_k <= 32 ? 32u : (top_k <= 64 ? 64u : 128u), final_dists, final_ids);
     return launch_status();
 }

@@ -260,6 +260,7 @@ public:
                 first_use = make_resident();
             } catch (const hip_error&) {
                 r_data.reset(); r_graph.reset(); r_centroids.reset(); r_start_points.reset(); r_map.reset();
+                r_segment_starts.reset(); r_local_start_points.reset();
                 resident_failed = true;
             }
             if (!resident_failed) {
@@ -386,7 +387,8 @@ public:
     }
 
     // The per-partition search of glide_large_impl.cuh:347-507 on an index that is resident in device memory: the same
-    // kernels on the same partitions in the same order as the staged path, without the copies.
+    // searches and the same order of result merges as the staged path, without the copies and in three launches
+    // (queries grouped by partition, one wavefront per query and selected partition, one merge per query).
     void search_resident(SearchParameter& param, uint32_t min_segment_num, float boundary_factor, device_matrix_view<Data_t> d_query_view,
                          host_matrix_view<uint32_t> h_result_ids_view, host_matrix_view<float> h_result_distances_view, std::string& result_file,
                          bool first_use) {
@@ -394,19 +396,11 @@ public:
         device_matrix<uint32_t> d_final_ids(query_number, top_k), d_segment_ids(query_number, c);
         device_matrix<float> d_final_dists(query_number, top_k);
         device_matrix<float> d_query_f32(sizeof(Data_t) == 1 ? query_number : 0, dim());
-        device_vector<uint32_t> d_counts(c), d_offsets(c + 1);
-        device_matrix<uint32_t> d_lists(query_number ? query_number : 1, c);
-        const size_t gwb = glide_hip_group_queries_workspace_bytes(c);
-        device_buffer group_ws(gwb);
-        std::vector<uint32_t> offsets(c + 1);
+        const size_t swb = glide_hip_search_partitions_workspace_bytes(query_number, c, top_k);
+        device_buffer search_ws(swb);
         const int mc = metric_code(metric);
         void* cs = handle.stream();
-        const float fmax = FLT_MAX;
-        uint32_t fmax_bits;
-        std::memcpy(&fmax_bits, &fmax, 4);
         auto run = [&](uint32_t queries) {
-            hip_try(glide_hip_fill_u32(d_final_ids.data_handle(), 0xffffffffu, d_final_ids.size(), cs), "glide_hip_fill_u32");
-            hip_try(glide_hip_fill_u32(reinterpret_cast<uint32_t*>(d_final_dists.data_handle()), fmax_bits, d_final_dists.size(), cs), "glide_hip_fill_u32");
             const float* d_queries = reinterpret_cast<const float*>(d_query_view.data_handle());
             if (sizeof(Data_t) == 1) {
                 hip_try(glide_hip_widen_u8(reinterpret_cast<const unsigned char*>(d_query_view.data_handle()), static_cast<size_t>(queries) * dim(),
@@ -417,21 +411,13 @@ public:
             hip_try(glide_hip_select_segments(d_queries, queries, dim(), r_centroids->data_handle(), c, min_segment_num, boundary_factor, mc,
                                               d_segment_ids.data_handle(), cs),
                     "glide_hip_select_segments");
-            // the queries of each partition, so that a partition launches one wavefront per query that selected it
-            hip_try(glide_hip_group_queries(d_segment_ids.data_handle(), queries, c, d_counts.data_handle(), d_offsets.data_handle(),
-                                            d_lists.data_handle(), group_ws.get(), gwb, cs),
-                    "glide_hip_group_queries");
-            hip_try(glide_hip_memcpy_d2h(offsets.data(), d_offsets.data_handle(), (c + 1) * sizeof(uint32_t), cs), "glide_hip_memcpy_d2h");
-            for (uint32_t s = 0; s < segment_num(); s++) {
-                const size_t start = h_segment_start(s);
-                const uint32_t wanted = offsets[s + 1] - offsets[s];
-                if (h_segment_length(s) == 0 || wanted == 0) continue;
-                hip_try(glide_hip_search_sub_listed(r_data->data_handle() + start * dim(), dim(), r_graph->data_handle() + start * deg, deg,
-                                                    r_map->data_handle() + start, d_queries, queries, d_lists.data_handle() + offsets[s], wanted, s,
-                                                    h_start_point(s), top_k, param.beam, param.max_iterations, param.min_iterations, param.hash_bit,
-                                                    param.hash_reset_interval, mc, d_final_ids.data_handle(), d_final_dists.data_handle(), nullptr, cs),
-                        "glide_hip_search_sub_listed");
-            }
+            // one wavefront per (query, selected partition), the heads merged per query in partition order
+            hip_try(glide_hip_search_partitions(r_data->data_handle(), dim(), r_graph->data_handle(), deg, r_map->data_handle(),
+                                                r_segment_starts->data_handle(), r_local_start_points->data_handle(), c, d_queries, queries,
+                                                d_segment_ids.data_handle(), top_k, param.beam, param.max_iterations, param.min_iterations,
+                                                param.hash_bit, param.hash_reset_interval, mc, d_final_ids.data_handle(),
+                                                d_final_dists.data_handle(), search_ws.get(), swb, nullptr, cs),
+                    "glide_hip_search_partitions");
         };
         if (first_use && query_number) run(1);   // part of bringing the index up: the first launch of a kernel loads its code
         gpu_timer timer;
@@ -489,9 +475,15 @@ private:
         for (uint32_t s = 0; s < c; s++) entry[s] = h_segment_start(s) + h_start_point(s);
         r_start_points.emplace(c);
         copy_to_device(r_start_points->data_handle(), entry.data(), c);
-        if (!merged()) {   // the per-partition search writes input row numbers itself
+        if (!merged()) {   // the per-partition search writes input row numbers itself and addresses the partitions on the device
             r_map.emplace(n);
             copy_to_device(r_map->data_handle(), h_map.data_handle(), n);
+            r_segment_starts.emplace(c);
+            copy_to_device(r_segment_starts->data_handle(), h_segment_start.data_handle(), c);
+            std::vector<uint32_t> local(c);
+            for (uint32_t s = 0; s < c; s++) local[s] = h_segment_length(s) ? h_start_point(s) : 0xffffffffu;   // empty partitions are skipped
+            r_local_start_points.emplace(c);
+            copy_to_device(r_local_start_points->data_handle(), local.data(), c);
         }
         std::cout << "index upload time: " << timer.stop() << " s" << std::endl;
         return true;
@@ -500,7 +492,7 @@ private:
     std::optional<device_matrix<float>> r_data;
     std::optional<device_matrix<uint32_t>> r_graph;
     std::optional<device_matrix<float>> r_centroids;
-    std::optional<device_vector<uint32_t>> r_start_points, r_map;
+    std::optional<device_vector<uint32_t>> r_start_points, r_map, r_segment_starts, r_local_start_points;
     bool resident_failed = false;
     device_resources& handle;
     Metric metric;

@@ -262,6 +262,25 @@ int glide_hip_search_sub_listed(const float *segment_data, uint32_t dim, const u
                                 uint32_t min_iterations, uint32_t hash_bit, uint32_t hash_reset_interval, int metric,
                                 uint32_t *final_ids, float *final_dists, unsigned long long *counters, void *stream);
 
+/* The whole per-partition search of GLIDE_large::search (glide_large_impl.cuh:347-507) on an index resident in device
+ * memory, in three launches instead of one per partition: the queries are grouped by partition, one wavefront per
+ * (query, selected partition) pair runs search_on_sub_kernel's search and leaves the head of its beam, and one
+ * wavefront per query merges its heads in ascending partition order, the order of the partition-by-partition loop,
+ * so ids and distances are the same.  data / graph / map hold all partitions in reorder order (graph ids are
+ * partition-local); segment_starts and segment_start_points (local; 0xffffffff marks an empty partition) are device
+ * arrays of segment_num entries;
+ * segment_ids comes from glide_hip_select_segments with centroid_num = segment_num.  final_ids / final_dists
+ * (query_num x top_k) are overwritten.  The call waits on `stream` once (it reads the number of pairs back).
+ * workspace: glide_hip_search_partitions_workspace_bytes(), sized for every query selecting every partition. */
+size_t glide_hip_search_partitions_workspace_bytes(uint32_t query_num, uint32_t centroid_num, uint32_t top_k);
+int glide_hip_search_partitions(const float *data, uint32_t dim, const uint32_t *graph, uint32_t graph_degree,
+                                const uint32_t *map, const uint32_t *segment_starts,
+                                const uint32_t *segment_start_points, uint32_t segment_num, const float *queries,
+                                uint32_t query_num, const uint32_t *segment_ids, uint32_t top_k, uint32_t beam,
+                                uint32_t max_iterations, uint32_t min_iterations, uint32_t hash_bit,
+                                uint32_t hash_reset_interval, int metric, uint32_t *final_ids, float *final_dists,
+                                void *workspace, size_t workspace_bytes, unsigned long long *counters, void *stream);
+
 /* ---- merged large build (GLIDE_large::build_with_merge, declared at glide_large.cuh:89-97 without a definition) --
  * The merged graph lives in device memory in reorder-id space: row r belongs to reorder row r (r < num) and holds
  * reorder ids.  The two passes below are the large-path forms of map_to_graph (graph_kernel.cuh:145-150) and

@@ -114,6 +114,19 @@ def test_search_over_partitions_bit_exact(hip, large_index, top_k, beam):
                               top_k, sp["beam"], sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 0, l_ids, l_d)
         hip.synchronize()
     assert np.array_equal(l_ids.numpy(), e_ids) and np.array_equal(l_d.numpy(), e_d)
+    # and in three launches over the resident index: one wavefront per (query, partition) pair, heads merged per query
+    all_data = np.concatenate([seg["data"] for seg in L["segs"]])
+    all_graph = np.concatenate([seg["graph"] for seg in L["segs"]])
+    all_map = np.concatenate([seg["map"] for seg in L["segs"]])
+    lens = np.array([seg["data"].shape[0] for seg in L["segs"]], np.uint32)
+    seg_starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.uint32)
+    p_ids, p_d = hip.DeviceArray((nq, top_k), np.uint32), hip.DeviceArray((nq, top_k), np.float32)
+    cnt = hip.new_counters()
+    hip.search_partitions(hip.DeviceArray.from_numpy(all_data), 128, hip.DeviceArray.from_numpy(all_graph), 32, hip.DeviceArray.from_numpy(all_map),
+                          hip.DeviceArray.from_numpy(seg_starts), hip.DeviceArray.from_numpy(L["start_points"].astype(np.uint32)), c, d_q, nq, d_seg,
+                          top_k, sp["beam"], sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"], 0, p_ids, p_d, cnt)
+    assert np.array_equal(p_ids.numpy(), e_ids) and np.array_equal(p_d.numpy(), e_d)
+    assert hip.read_counters(cnt)[0] > 0
 
 
 def test_place_and_merge_boundary_bit_exact(hip):
