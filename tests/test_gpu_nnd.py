@@ -121,3 +121,18 @@ def test_nnd_rejects_unsupported(hip):
     with pytest.raises(hip.GlideHipError) as e:
         hip.nnd_build(d, 8, 128, d, d, 1, 32, 1, 0.0, 0, d, d, 16)      # workspace too small
     assert e.value.code == -2
+
+
+@pytest.mark.parametrize("dim,k", [(4, 8), (36, 16), (100, 32), (132, 48), (260, 64), (1024, 24)])
+def test_nnd_shapes(hip, dim, k):
+    """Dimensions that are not a multiple of the 64-dim chunk of the join (or of 8) and list widths 32, 64 and 96."""
+    data = lowdim_data(3000, dim, latent=min(8, dim), seed=dim)
+    seg_len = np.array([1800, 1200], dtype=np.uint32)
+    seg_start = np.array([0, 1800], dtype=np.uint32)
+    knn, _ = gpu_nnd(hip, data, seg_start, seg_len, k, 12)
+    for s, l in zip(seg_start.tolist(), seg_len.tolist()):
+        rows = knn[s:s + l]
+        assert (rows < l).all() and (rows != np.arange(l, dtype=np.uint32)[:, None]).all()
+    r = partition_recall(knn, data, seg_start, seg_len, k, sample=200)
+    print("graph recall@%d (dim %d): %.4f" % (k, dim, r))
+    assert r >= (0.9 if dim > 4 else 0.6)      # 4 small-integer dimensions are mostly ties
