@@ -823,6 +823,8 @@ int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* s
     if (dim == 0 || segment_num == 0 || knn_degree == 0 || reorder_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (segment_num > kMaxSegments) return GLIDE_ERR_UNSUPPORTED;
     if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // also keeps the Bloom filter within 64 words
+    // one thread per list slot / per sample: the products must fit the 32-bit launch arithmetic (44 M rows at width 96)
+    if (static_cast<unsigned long long>(reorder_num) * nnd_width(knn_degree) >= 0xffffffffull || reorder_num >= (1u << 26)) return GLIDE_ERR_UNSUPPORTED;
     c.l = nnd_layout(reorder_num, dim, knn_degree);
     if (c.l.bloom_sets > 4) return GLIDE_ERR_UNSUPPORTED;
     if (workspace_bytes < c.l.total || reinterpret_cast<uintptr_t>(workspace) % 16) return GLIDE_ERR_BAD_ARGUMENT;

@@ -606,6 +606,7 @@ extern "C" int glide_hip_group_queries(const uint32_t* segment_ids, uint32_t que
                                        uint32_t* lists, void* workspace, size_t workspace_bytes, void* stream) {
     if (!segment_ids || !counts || !offsets || !lists || !workspace || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (workspace_bytes < glide_hip_group_queries_workspace_bytes(centroid_num)) return GLIDE_ERR_BAD_ARGUMENT;
+    if (static_cast<unsigned long long>(query_num) * centroid_num >= 0xffffffffull) return GLIDE_ERR_UNSUPPORTED;
     hipStream_t s = as_stream(stream);
     int rc = glide_hip_fill_u32(counts, 0u, centroid_num, stream);
     if (rc != GLIDE_OK) return rc;
@@ -656,6 +657,7 @@ extern "C" int glide_hip_search_partitions(const float* data, uint32_t dim, cons
     if (query_num == 0) return GLIDE_OK;
     if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 1024 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
+    if (static_cast<unsigned long long>(query_num) * segment_num >= 0xffffffffull) return GLIDE_ERR_UNSUPPORTED;   // pairs are numbered with 32 bits
     const PartitionSearchLayout l = partition_search_layout(query_num, segment_num, top_k);
     if (workspace_bytes < l.total || reinterpret_cast<uintptr_t>(workspace) % 8) return GLIDE_ERR_BAD_ARGUMENT;
     hipStream_t s = as_stream(stream);

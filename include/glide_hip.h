@@ -133,7 +133,8 @@ int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim,
  * states are read back after each round (the call then waits on `stream`) and the loop ends once every partition
  * rests.  At most 2048 partitions.
  * stats_out (nullable, 2 device u64): offers received by the merge step, offers dropped by a full inbox.
- * Limits: knn_degree <= 65 (list width round_up32(1.3 * knn_degree) <= 96, Bloom filter <= 2048 bits), dim % 4 == 0. */
+ * Limits: knn_degree <= 65 (list width round_up32(1.3 * knn_degree) <= 96, Bloom filter <= 2048 bits), dim % 4 == 0,
+ * reorder_num < 2^26 and reorder_num * list width < 2^32 per call (the large path calls it partition by partition). */
 size_t glide_hip_nnd_workspace_bytes(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree);
 int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim,
                         const uint32_t *segment_starts, const uint32_t *segment_lengths, uint32_t segment_num,
