@@ -63,17 +63,7 @@ def make_data(workload, num, nq):
     import numpy as np
     from glide_amd import datasets as D
     if workload == "cfg1-navigable":
-        a = np.random.default_rng(0).standard_normal((12, 128)).astype(np.float32)
-
-        def gen(m, seed):
-            r = np.random.default_rng(seed)
-            out = np.empty((m, 128), dtype=np.float32)
-            for s in range(0, m, 1 << 18):
-                e = min(m, s + (1 << 18))
-                z = r.standard_normal((e - s, 12)).astype(np.float32)
-                out[s:e] = np.rint(np.clip(z @ a * 20 + 128 + r.standard_normal((e - s, 128)).astype(np.float32) * 3, 0, 255))
-            return out
-        return gen(num, 1234), gen(nq, 4321)
+        return D.lowdim_integer(num, 128, seed=1234), D.lowdim_integer(nq, 128, seed=4321)
     if workload == "cfg2":
         return D.gmm_normalized(num, 96, seed=1234), D.gmm_normalized(nq, 96, seed=4321)
     if workload == "cfg3":

@@ -46,6 +46,20 @@ def beta_scaled(num, dim=960, components=128, seed=1234, mixture_seed=97):
     return out
 
 
+def lowdim_integer(num, dim=128, latent=12, spread=20.0, noise=3.0, seed=1234, mixture_seed=0):
+    """A `latent`-dimensional Gaussian cloud mapped linearly into `dim` dimensions around 128, plus a little noise,
+    clipped to [0, 255] and rounded: integer-valued data of low intrinsic dimension, on which graph search navigates
+    well.  The linear map depends only on `mixture_seed`."""
+    a = np.random.default_rng(mixture_seed).standard_normal((latent, dim)).astype(np.float32)
+    r = np.random.default_rng(seed)
+    out = np.empty((num, dim), dtype=np.float32)
+    for s in range(0, num, 1 << 18):
+        e = min(num, s + (1 << 18))
+        z = r.standard_normal((e - s, latent)).astype(np.float32)
+        out[s:e] = np.rint(np.clip(z @ a * spread + 128 + r.standard_normal((e - s, dim)).astype(np.float32) * noise, 0, 255))
+    return out
+
+
 def write_fbin(path, matrix):
     matrix = np.ascontiguousarray(matrix)
     with open(path, "wb") as f:

@@ -1,5 +1,6 @@
 """Whole small-build pipeline on the GPU against the CPU oracle's pipeline, on reduced copies of the benchmark
-configurations (clipped mixture L2 with k=64, normalised mixture cosine with 96 dims, 960 dims with degree 64).
+configurations (clipped mixture L2 with k=64, normalised mixture cosine with 96 dims, 960 dims with degree 64) and
+on integer data of low intrinsic dimension.
 
 The two pipelines share the centroids and the entry points, so the partitioning is the same; the kNN graphs come
 from different NN-descent runs, so the comparison is statistical:
@@ -52,6 +53,8 @@ CASES = [
     ("clipped-mixture-k64", "gmm_clipped", 20_000, 128, 4, 32, 64, 8, 0, 1000, 0.12),
     ("normalised-mixture-cosine", "gmm_normalized", 20_000, 96, 4, 32, 32, 10, 1, 1000, 0.015),
     ("beta-960-degree64", "beta_scaled", 6_000, 960, 3, 64, 64, 8, 0, 300, 0.015),
+    # data of low intrinsic dimension, where search recall does not hang on single edges: the 0.5-point bar applies
+    ("low-dimensional-integer", "lowdim_integer", 20_000, 128, 4, 32, 32, 10, 0, 1000, 0.005),
 ]
 
 
@@ -84,7 +87,7 @@ def test_pipeline_matches_cpu_pipeline(hip, name, gen, num, dim, parts, degree, 
     assert np.array_equal(index.d_start_points.numpy(), start_points)
 
     # ---- CPU pipeline from the same centroids and entry points
-    float_data = gen != "gmm_clipped"
+    float_data = gen not in ("gmm_clipped", "lowdim_integer")
     seg_idx, seg_len_cpu, _ = O.partition_assign(data, centroids, 1.04, metric)
     if float_data:
         # a reassociated float sum can move a point that sits on a partition border or on the boundary-ratio threshold
