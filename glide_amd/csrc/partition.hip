@@ -242,27 +242,194 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
         a.tile_hist[static_cast<size_t>(blockIdx.x) * (a.centroid_num + 1) + i] = hist[i];
 }
 
-// exclusive scan over tiles, one workgroup per bin; also emits the bin totals (segment lengths)
-__global__ __launch_bounds__(256) void tile_scan_kernel(uint32_t* tile_hist, uint32_t tiles, uint32_t bins, uint32_t* totals) {
-    __shared__ uint32_t partial[256];
-    const uint32_t bin = blockIdx.x;
-    const uint32_t per = ceil_div(tiles, 256);
-    const uint32_t begin = threadIdx.x * per, end = begin + per < tiles ? begin + per : tiles;
-    uint32_t sum = 0;
-    for (uint32_t i = begin; i < end; i++) sum += tile_hist[static_cast<size_t>(i) * bins + bin];
-    partial[threadIdx.x] = sum;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t run = 0;
-        for (int i = 0; i < 256; i++) {
-            const uint32_t v = partial[i];
-            partial[i] = run;
-            run += v;
+// Assignment for at most 32 centroids of at most 128 dims, the shape that is bound by reading the points once.
+// NQ = number of 32-dim chunks per row.  The whole centroid matrix sits in LDS for the life of the workgroup, so
+// after the one barrier that publishes it the four wavefronts run without meeting again.  Each wavefront issues
+// the loads of all its 32 points at once (coalesced, 16 KB in flight at 128 dims), passes them chunk by chunk
+// through a private LDS tile into the matrix-instruction operand layout and KEEPS those operand registers, so the
+// exact rescoring of the kTop best centroids reads no point a second time: lane (i, half) rescans its half of
+// row i against centroid rows in LDS and the two halves are added.
+template <int NQ>
+__global__ __launch_bounds__(256) void assign_resident_kernel(AssignArgs a) {
+    extern __shared__ __align__(16) float smem[];
+    constexpr int DP = 32 * NQ;           // padded dims
+    constexpr int CS = DP + 4;            // centroid row stride
+    float* cent = smem;                                            // [32][CS], zero outside centroid_num x dim
+    float* x_tile = cent + 32 * CS;                                // [4 waves][32][kLdsStride]
+    uint32_t* hist = reinterpret_cast<uint32_t*>(x_tile + 4 * 32 * kLdsStride);   // [C + 1]
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int half = lane >> 5, t = lane & 31;
+    const uint32_t wave_base = blockIdx.x * kTilePoints + wave * 32;
+    float* xw = x_tile + wave * 32 * kLdsStride;
+
+    float4 xpre[NQ][4];   // chunk c: 8 lanes x float4 per row, 8 rows per step
+#pragma unroll
+    for (int c = 0; c < NQ; c++)
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const uint32_t p = wave_base + it * 8 + (lane >> 3), d0 = c * 32 + (lane & 7) * 4;
+            xpre[c][it] = (p < a.num && d0 < a.dim) ? *reinterpret_cast<const float4*>(a.data + static_cast<size_t>(p) * a.dim + d0)
+                                                    : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        totals[bin] = run;
+    for (uint32_t idx = threadIdx.x; idx < 32 * (DP / 4); idx += 256) {
+        const uint32_t row = idx / (DP / 4), d0 = (idx % (DP / 4)) * 4;
+        *reinterpret_cast<float4*>(cent + row * CS + d0) =
+            (row < a.centroid_num && d0 < a.dim) ? *reinterpret_cast<const float4*>(a.centroids + static_cast<size_t>(row) * a.dim + d0)
+                                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256) hist[i] = 0;
+    __syncthreads();
+
+    float16v acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    float4 xr[NQ][4];   // this lane's operand share of row t: dims c*32 + q*8 + 4*half .. +3
+#pragma unroll
+    for (int c = 0; c < NQ; c++) {
+#pragma unroll
+        for (int it = 0; it < 4; it++)
+            *reinterpret_cast<float4*>(xw + (it * 8 + (lane >> 3)) * kLdsStride + (lane & 7) * 4) = xpre[c][it];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            xr[c][q] = *reinterpret_cast<const float4*>(xw + t * kLdsStride + q * 8 + 4 * half);
+            const float4 bv = *reinterpret_cast<const float4*>(cent + t * CS + c * 32 + q * 8 + 4 * half);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].x, bv.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].y, bv.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].z, bv.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].w, bv.w, acc, 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // ranking: score = ||c||^2 - 2 x.c through this wave's tile (now free), kTop best per point
+    float* sw = xw;   // [32][33]
+    float best_s[kTop];
+    uint32_t best_c[kTop];
+#pragma unroll
+    for (int k = 0; k < kTop; k++) {
+        best_s[k] = FLT_MAX;
+        best_c[k] = kInvalid;
+    }
+    auto offer = [&](float sc, uint32_t c) {
+#pragma unroll
+        for (int k = 0; k < kTop; k++) {
+            if (sc < best_s[k]) {
+                const float ts = best_s[k];
+                const uint32_t tc = best_c[k];
+                best_s[k] = sc;
+                best_c[k] = c;
+                sc = ts;
+                c = tc;
+            }
+        }
+    };
+    {
+        const uint32_t j = t;
+        const float cn = j < a.centroid_num ? a.centroid_norms[j] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int i = 8 * (r / 4) + 4 * half + (r % 4);   // accumulator layout of the 32x32 tile
+            sw[i * 33 + t] = j < a.centroid_num ? cn - 2.f * acc[r] : FLT_MAX;
+        }
+        __builtin_amdgcn_wave_barrier();
+        // the valid columns are shared out evenly between the two lanes of a point
+        const uint32_t per = (a.centroid_num + 1) / 2, col0 = half * per;
+#pragma unroll 4
+        for (uint32_t jj = 0; jj < per; jj++) offer(sw[t * 33 + col0 + jj], col0 + jj);
+    }
+    {
+        float os[kTop];
+        uint32_t oc[kTop];
+#pragma unroll
+        for (int k = 0; k < kTop; k++) {
+            os[k] = lane_xor<32>(best_s[k]);
+            oc[k] = lane_xor<32>(best_c[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < kTop; k++) offer(os[k], oc[k]);
+    }
+    // Both lanes of a point must rescore the same candidates in the same order: equal scores could have been
+    // ranked differently by the two halves, so the upper half takes the lower half's list.
+#pragma unroll
+    for (int k = 0; k < kTop; k++) best_c[k] = static_cast<uint32_t>(__shfl(static_cast<int>(best_c[k]), t));
+
+    // exact rescoring from the kept registers; smallest two by (distance, centroid id)
+    float d0 = FLT_MAX, d1 = FLT_MAX;
+    uint32_t c0 = kInvalid, c1 = kInvalid;
+#pragma unroll
+    for (int k = 0; k < kTop; k++) {
+        const uint32_t ck = best_c[k];
+        const float* crow = cent + (ck != kInvalid ? ck : 0u) * CS + 4 * half;
+        float part = 0.f;
+#pragma unroll
+        for (int c = 0; c < NQ; c++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) part = sqdist4(xr[c][q], *reinterpret_cast<const float4*>(crow + c * 32 + q * 8), part);
+        const float sq = part + lane_xor<32>(part);
+        const float dk = ck != kInvalid ? finish_distance(sq, a.metric) : FLT_MAX;
+        const bool lt0 = dk < d0 || (dk == d0 && ck < c0);
+        const bool lt1 = dk < d1 || (dk == d1 && ck < c1);
+        if (lt0) {
+            d1 = d0; c1 = c0;
+            d0 = dk; c0 = ck;
+        } else if (lt1) {
+            d1 = dk; c1 = ck;
+        }
+    }
+    (void) c1;
+
+    const uint32_t p = wave_base + lane;
+    if (lane < 32 && p < a.num) {
+        // reference partition_kernel.cuh:55-64: boundary iff a second centroid exists and d(2)/d(1) <= factor
+        const bool boundary = a.centroid_num > 1 && (d1 / d0 <= a.boundary_factor);
+        a.segment_indexes[static_cast<size_t>(p) * 3] = c0;
+        a.segment_indexes[static_cast<size_t>(p) * 3 + 2] = boundary ? 0u : kInvalid;
+        if (a.nearest_dists) {
+            a.nearest_dists[static_cast<size_t>(p) * 2] = d0;
+            a.nearest_dists[static_cast<size_t>(p) * 2 + 1] = d1;
+        }
+        atomicAdd(&hist[c0], 1u);
+        if (boundary) atomicAdd(&hist[a.centroid_num], 1u);
     }
     __syncthreads();
-    uint32_t run = partial[threadIdx.x];
+    for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256)
+        a.tile_hist[static_cast<size_t>(blockIdx.x) * (a.centroid_num + 1) + i] = hist[i];
+}
+
+size_t assign_resident_lds_bytes(int nq, uint32_t centroid_num) {
+    return (static_cast<size_t>(32) * (32 * nq + 4) + 4 * 32 * kLdsStride) * sizeof(float) + (centroid_num + 1) * sizeof(uint32_t);
+}
+
+// exclusive scan over tiles, one workgroup per bin; also emits the bin totals (segment lengths)
+constexpr int kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void tile_scan_kernel(uint32_t* tile_hist, uint32_t tiles, uint32_t bins, uint32_t* totals) {
+    __shared__ uint32_t wave_total[kScanThreads / 64];
+    const uint32_t bin = blockIdx.x;
+    const int lane = lane_id(), wave = threadIdx.x >> 6;
+    const uint32_t per = ceil_div(tiles, static_cast<uint32_t>(kScanThreads));
+    const uint32_t begin = min(threadIdx.x * per, tiles), end = min(begin + per, tiles);
+    uint32_t sum = 0;
+    for (uint32_t i = begin; i < end; i++) sum += tile_hist[static_cast<size_t>(i) * bins + bin];
+    uint32_t inclusive = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t below = static_cast<uint32_t>(__shfl_up(static_cast<int>(inclusive), d));
+        if (lane >= d) inclusive += below;
+    }
+    if (lane == 63) wave_total[wave] = inclusive;
+    __syncthreads();
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kScanThreads / 64; w++) {
+        const uint32_t v = wave_total[w];
+        before += w < wave ? v : 0u;
+        total += v;
+    }
+    if (threadIdx.x == 0) totals[bin] = total;
+    uint32_t run = before + inclusive - sum;
     for (uint32_t i = begin; i < end; i++) {
         const uint32_t v = tile_hist[static_cast<size_t>(i) * bins + bin];
         tile_hist[static_cast<size_t>(i) * bins + bin] = run;
@@ -293,28 +460,45 @@ __global__ __launch_bounds__(kTilePoints) void slot_kernel(uint32_t* segment_ind
     if (my_b != kInvalid) segment_indexes[static_cast<size_t>(p) * 3 + 2] = base[centroid_num] + brank;
 }
 
-// reorder_kernel (partition_kernel.cuh:68-100): one wavefront per point
+// reorder_kernel (partition_kernel.cuh:68-100).  One wavefront moves kReorderRows consecutive points: their source
+// rows are one contiguous piece of memory, read as a flat run of float4 with every lane busy whatever the dimension
+// (several loads in flight per lane); lanes 0..rows-1 hold the destination rows, fetched per element by a lane read.
+constexpr uint32_t kReorderRows = 8;
 __global__ __launch_bounds__(256) void reorder_kernel(const float* data, float* reorder_data, const uint32_t* segment_indexes,
                                                       uint32_t* map, const uint32_t* segment_starts, uint32_t num, uint32_t dim,
                                                       uint32_t point_id_offset) {
     const int lane = lane_id();
-    const uint32_t p = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (p >= num) return;
-    const uint32_t seg = segment_indexes[static_cast<size_t>(p) * 3];
-    const uint32_t slot = segment_indexes[static_cast<size_t>(p) * 3 + 1];
-    const uint32_t bslot = segment_indexes[static_cast<size_t>(p) * 3 + 2];
-    const uint32_t rid = segment_starts[seg] + slot;
-    const float* src = data + static_cast<size_t>(p) * dim;
-    float* dst = reorder_data + static_cast<size_t>(rid) * dim;
-    float* bdst = bslot != kInvalid ? reorder_data + static_cast<size_t>(num + bslot) * dim : nullptr;
-    for (uint32_t d0 = lane * 4; d0 < dim; d0 += 256) {
-        const float4 v = *reinterpret_cast<const float4*>(src + d0);
-        *reinterpret_cast<float4*>(dst + d0) = v;
-        if (bdst) *reinterpret_cast<float4*>(bdst + d0) = v;
+    const uint32_t first = (blockIdx.x * 4 + (threadIdx.x >> 6)) * kReorderRows;
+    if (first >= num) return;
+    const uint32_t rows = min(kReorderRows, num - first);
+    uint32_t rid = 0, brow = kInvalid;
+    if (static_cast<uint32_t>(lane) < rows) {
+        const uint32_t* si = segment_indexes + static_cast<size_t>(first + lane) * 3;
+        rid = segment_starts[si[0]] + si[1];
+        if (si[2] != kInvalid) brow = num + si[2];
+        map[rid] = first + lane + point_id_offset;
+        if (brow != kInvalid) map[brow] = first + lane + point_id_offset;
     }
-    if (lane == 0) {
-        map[rid] = p + point_id_offset;
-        if (bdst) map[num + bslot] = p + point_id_offset;
+    const uint32_t q = dim / 4, total = rows * q;
+    const float4* src = reinterpret_cast<const float4*>(data + static_cast<size_t>(first) * dim);
+    float4* out = reinterpret_cast<float4*>(reorder_data);
+    for (uint32_t e0 = 0; e0 < total; e0 += 256) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t e = e0 + u * 64 + lane;
+            if (e < total) v[u] = src[e];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t e = e0 + u * 64 + lane;
+            const uint32_t row = min(e / q, rows - 1), col = e - row * q;
+            const uint32_t r = __shfl(rid, static_cast<int>(row)), b = __shfl(brow, static_cast<int>(row));
+            if (e < total) {
+                out[static_cast<size_t>(r) * q + col] = v[u];
+                if (b != kInvalid) out[static_cast<size_t>(b) * q + col] = v[u];
+            }
+        }
     }
 }
 
@@ -591,6 +775,19 @@ int glide_hip_partition_assign(const float* data, uint32_t num, uint32_t dim, co
     hipLaunchKernelGGL(row_norms_kernel, dim3(ceil_div(centroid_num, 4)), dim3(256), 0, s, centroids, centroid_num, dim, norms);
     AssignArgs a{data, centroids, norms, segment_indexes, tile_hist, nearest_dists, num, dim, centroid_num, boundary_factor, metric};
     const int cb = centroid_num <= 32 ? 1 : centroid_num <= 64 ? 2 : centroid_num <= 128 ? 4 : 8;
+    if (centroid_num <= 32 && dim <= 128) {
+        const int nq = static_cast<int>(ceil_div(dim, 32u));
+        const size_t rlds = assign_resident_lds_bytes(nq, centroid_num);
+        switch (nq) {
+            case 1: hipLaunchKernelGGL(assign_resident_kernel<1>, dim3(tiles), dim3(256), rlds, s, a); break;
+            case 2: hipLaunchKernelGGL(assign_resident_kernel<2>, dim3(tiles), dim3(256), rlds, s, a); break;
+            case 3: hipLaunchKernelGGL(assign_resident_kernel<3>, dim3(tiles), dim3(256), rlds, s, a); break;
+            default: hipLaunchKernelGGL(assign_resident_kernel<4>, dim3(tiles), dim3(256), rlds, s, a); break;
+        }
+        hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(kScanThreads), 0, s, tile_hist, tiles, centroid_num + 1, segment_lengths);
+        hipLaunchKernelGGL(slot_kernel, dim3(tiles), dim3(kTilePoints), 0, s, segment_indexes, tile_hist, num, centroid_num);
+        return launch_status();
+    }
     const size_t lds = assign_lds_bytes(cb, centroid_num);
     if (lds > 64 * 1024) {
         GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&assign_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -602,7 +799,7 @@ int glide_hip_partition_assign(const float* data, uint32_t num, uint32_t dim, co
         case 4: hipLaunchKernelGGL(assign_kernel<4>, dim3(tiles), dim3(256), lds, s, a); break;
         default: hipLaunchKernelGGL(assign_kernel<8>, dim3(tiles), dim3(256), lds, s, a); break;
     }
-    hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(256), 0, s, tile_hist, tiles, centroid_num + 1, segment_lengths);
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(kScanThreads), 0, s, tile_hist, tiles, centroid_num + 1, segment_lengths);
     hipLaunchKernelGGL(slot_kernel, dim3(tiles), dim3(kTilePoints), 0, s, segment_indexes, tile_hist, num, centroid_num);
     return launch_status();
 }
@@ -612,7 +809,7 @@ int glide_hip_reorder_batch(const float* data, uint32_t num, uint32_t dim, const
     if (!data || !segment_indexes || !segment_starts || !reorder_data || !map || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
     if (num == 0) return GLIDE_OK;
-    hipLaunchKernelGGL(reorder_kernel, dim3(ceil_div(num, 4)), dim3(256), 0, as_stream(stream), data, reorder_data, segment_indexes, map,
+    hipLaunchKernelGGL(reorder_kernel, dim3(ceil_div(num, 4 * kReorderRows)), dim3(256), 0, as_stream(stream), data, reorder_data, segment_indexes, map,
                        segment_starts, num, dim, point_id_offset);
     return launch_status();
 }
