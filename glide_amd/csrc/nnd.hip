@@ -294,7 +294,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     if (a.segs.state[seg] == kDone) return;
     const uint32_t c_fn = c4.x, c_fo = c4.y;
     const uint32_t c_rn = c4.z < kSamples ? c4.z : kSamples, c_ro = c4.w < kSamples ? c4.w : kSamples;
-    __syncthreads();   // every thread holds the counts
+    // The counts must have arrived in every thread before thread 0 restarts them below; the barrier itself waits
+    // for LDS traffic only, so the registers are consumed here.
+    asm volatile("" ::"v"(c4.x), "v"(c4.y), "v"(c4.z), "v"(c4.w));
+    __syncthreads();
     // this list's reverse samples are consumed here and now: the counts restart for the scatter that follows the join
     if (tid == 0) *reinterpret_cast<uint2*>(a.counts + static_cast<size_t>(node) * 4 + 2) = make_uint2(0u, 0u);
     if (c_fn + c_rn == 0) return;
