@@ -1,18 +1,23 @@
-"""The 1M x 128 configuration at its real size: 16 partitions, graph degree 32, 10 000 queries, top-10.
+"""The 1M-point configurations at their real size: 16 partitions, graph degree 32, 10 000 queries, top-10 (128 dims
+Euclidean on the benchmark's mixture and on data of low intrinsic dimension, 96 dims cosine on the normalised mixture).
 
 What the CPU oracle can finish in seconds at this size is compared bit for bit (the sub-graph rows of the first
 points, searches of a sample of the queries on the finished index); everything else is held to properties that do
 not depend on the size: the partition is a partition, reordered rows are the rows they claim to be, every list of
 the kNN graph is a set of local ids without the node itself, graph rows hold distinct ids, a second build from the
 same kNN graph gives the same graph, results are sorted, distinct, carry the exact distance of the id they name and
-do not depend on how the queries are ordered or batched.
+do not depend on how the queries are ordered or batched.  On the float data a reassociated sum can flip a near-tie,
+so "bit for bit" becomes "all but a few rows" there and distances are compared to 1e-5.
 """
 import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
 
-N, DIM, C, D, K, NQ = 1_000_000, 128, 16, 32, 32, 10_000
+N, C, D, K, NQ = 1_000_000, 16, 32, 32, 10_000
+# name: generator, dims, metric, integer-valued (sums exact in fp32)
+CONFIGS = {"lowdim_integer": ("lowdim_integer", 128, 0, True), "gmm_clipped": ("gmm_clipped", 128, 0, True),
+           "gmm_normalized_cosine": ("gmm_normalized", 96, 1, False)}
 INVALID = 0xFFFFFFFF
 
 
@@ -25,31 +30,32 @@ def hip():
 
 # the benchmark's mixture (64 far-apart components: search recall is low by construction) and data of low intrinsic
 # dimension, on which recall is meaningful
-@pytest.fixture(scope="module", params=["lowdim_integer", "gmm_clipped"])
+@pytest.fixture(scope="module", params=list(CONFIGS))
 def world(hip, request):
     """Data, queries, the partitioning, the kNN graph and the finished index, all made on the GPU."""
     from glide_amd import datasets as Ds, index as G
-    gen = getattr(Ds, request.param)
+    gen_name, DIM, metric, exact = CONFIGS[request.param]
+    gen = getattr(Ds, gen_name)
     data, queries = gen(N, DIM, seed=1234), gen(NQ, DIM, seed=4321)
     print("data", request.param, data.shape, flush=True)
     d_data = hip.DeviceArray.from_numpy(data)
-    pp = G.PartitionParameter(centroid_num=C, boundary_factor=1.04, sample_factor=0.01, metric=0)
+    pp = G.PartitionParameter(centroid_num=C, boundary_factor=1.04, sample_factor=0.01, metric=metric)
     d_re, d_map, h_start, h_len, d_cent = G.preprocess(pp, d_data)
     rdata, h_map, centroids = d_re.numpy(), d_map.numpy(), d_cent.numpy()
     d_knn = G.build_nnd(G.NNDescentParameter(graph_degree=K, max_iterations=20), d_re, h_start, h_len)
     knn = d_knn.numpy()
     print("partitioned and kNN built", rdata.shape, knn.shape, flush=True)
-    w = dict(kind=request.param, data=data, queries=queries, rdata=rdata, map=h_map, seg_start=h_start.copy(), seg_len=h_len.copy(), centroids=centroids, knn=knn)
+    w = dict(kind=request.param, metric=metric, exact=exact, data=data, queries=queries, rdata=rdata, map=h_map, seg_start=h_start.copy(), seg_len=h_len.copy(), centroids=centroids, knn=knn)
 
     # the sub-graph stage alone, for the comparison with the oracle
-    index = G.GLIDE(D, d_data, d_cent, 0)
+    index = G.GLIDE(D, d_data, d_cent, metric)
     bp = G.IndexParameter(graph_degree=D, knn_degree=K, relaxant_factor=1.05)
     local_sp, start_points = index.start_point_select(h_start, h_len, h_map, bp.seed)
     sp_b = G.make_search_parameter(64, K)
     d_ss, d_sl, d_lsp = (hip.DeviceArray.from_numpy(np.ascontiguousarray(a, dtype=np.uint32)) for a in (h_start, h_len, local_sp))
     d_sub = hip.DeviceArray.full((N, D), INVALID)
     hip.build_subgraph(d_re, N, DIM, d_knn, K, d_map, d_ss, d_sl, C + 1, d_lsp, D, sp_b.beam, sp_b.max_iterations, sp_b.min_iterations,
-                       sp_b.hash_bit, sp_b.hash_reset_interval, 1.05, 0, d_sub)
+                       sp_b.hash_bit, sp_b.hash_reset_interval, 1.05, metric, d_sub)
     hip.synchronize()
     w.update(sub=d_sub.numpy(), local_sp=local_sp, start_points=start_points, sp_b=sp_b)
     d_sub.free()
@@ -57,7 +63,7 @@ def world(hip, request):
     # two complete builds from the same kNN graph (build() consumes its device inputs, so they are copied first)
     graphs = []
     for _ in range(2):
-        idx = G.GLIDE(D, d_data, d_cent, 0)
+        idx = G.GLIDE(D, d_data, d_cent, metric)
         idx.build(bp, sp_b, G.make_search_parameter(128, K), hip.DeviceArray.from_numpy(knn), h_start, h_len,
                   hip.DeviceArray.from_numpy(h_map), hip.DeviceArray.from_numpy(rdata))
         graphs.append(idx.d_graph.numpy())
@@ -71,7 +77,7 @@ def world(hip, request):
 def _truth(world):
     if "truth" not in world:
         from oracle import oracle as O
-        world["truth"] = O.bruteforce_knn(world["data"], world["queries"][:1000], 10, 0)[0].astype(np.uint32)
+        world["truth"] = O.bruteforce_knn(world["data"], world["queries"][:1000], 10, world["metric"])[0].astype(np.uint32)
     return world["truth"]
 
 
@@ -98,7 +104,9 @@ def test_partition_assignment_on_a_sample(world):
     boundary = np.zeros(N, dtype=bool)
     boundary[mp[N:]] = True
     pick = np.random.default_rng(5).choice(N, 20_000, replace=False)
-    d = np.sqrt(((data[pick, None, :].astype(np.float64) - centroids[None].astype(np.float64)) ** 2).sum(-1))
+    d = ((data[pick, None, :].astype(np.float64) - centroids[None].astype(np.float64)) ** 2).sum(-1)
+    if world["metric"] == 0:
+        d = np.sqrt(d)      # the boundary ratio is one of distances for Euclidean, of squared distances for cosine
     order = np.argsort(d, axis=1)
     d0, d1 = d[np.arange(pick.size), order[:, 0]], d[np.arange(pick.size), order[:, 1]]
     clear = d1 - d0 > 1e-4 * d1          # away from ties between the two nearest centroids
@@ -122,7 +130,7 @@ def test_knn_graph_lists(world):
         srt = np.sort(rows, axis=1)
         assert (np.diff(srt, axis=1) > 0).all(), "no list holds an id twice"
         m = 100
-        ids, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + m], K + 1, 0)
+        ids, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + m], K + 1, world["metric"])
         truth = np.array([[x for x in ids[i].tolist() if x != i][:K] for i in range(m)], dtype=np.uint32)
         recalls.append(Ds.recall(knn[s:s + m], truth, K))
     print("graph recall@%d per partition" % K, np.round(recalls, 4), flush=True)
@@ -137,9 +145,11 @@ def test_subgraph_rows_equal_the_oracle(world):
     assert (sp["beam"], sp["max_iterations"], sp["hash_bit"]) == (world["sp_b"].beam, world["sp_b"].max_iterations, world["sp_b"].hash_bit)
     expect = np.full((N, D), INVALID, dtype=np.uint32)
     O.build_subgraph(world["rdata"], m, world["knn"], world["map"], world["seg_start"], world["seg_len"], world["local_sp"], D, sp, 1.05,
-                     graph=expect)
+                     world["metric"], graph=expect)
     rows = world["map"][:m]
-    assert np.array_equal(world["sub"][rows], expect[rows])
+    same = (world["sub"][rows] == expect[rows]).all(axis=1).mean()
+    print("sub-graph rows identical:", same, flush=True)
+    assert same == 1.0 if world["exact"] else same >= 0.97
     assert (expect[rows] != INVALID).any()
 
 
@@ -169,9 +179,15 @@ def test_search_sample_equals_the_oracle(hip, world, beam):
     ids, dists = world["index"].search(sp, world["d_queries"])
     pick = np.random.default_rng(beam).choice(NQ, 48, replace=False)
     e_ids, e_dists, _ = O.search(world["data"], world["graph"], world["centroids"], world["start_points"], world["queries"][pick], 10,
-                                 sp.beam, sp.max_iterations, sp.min_iterations, sp.hash_bit, sp.hash_reset_interval, 0)
-    assert np.array_equal(ids[pick], e_ids)
-    assert np.array_equal(dists[pick], e_dists)
+                                 sp.beam, sp.max_iterations, sp.min_iterations, sp.hash_bit, sp.hash_reset_interval, world["metric"])
+    if world["exact"]:
+        assert np.array_equal(ids[pick], e_ids)
+        assert np.array_equal(dists[pick], e_dists)
+    else:
+        same = (ids[pick] == e_ids).all(axis=1).mean()
+        print("result rows identical:", same, flush=True)
+        assert same >= 0.9
+        assert np.allclose(dists[pick][:, 0], e_dists[:, 0], rtol=1e-5)
 
 
 @pytest.mark.parametrize("beam", [32, 64])
@@ -185,7 +201,10 @@ def test_search_properties(hip, world, beam):
     assert (np.diff(np.sort(ids.astype(np.int64), axis=1), axis=1) > 0).all(), "a result names a point twice"
     # the distance reported is the distance of the point named: integer data, so the fp32 sum is exact
     sq = ((data[ids.reshape(-1)].astype(np.float64) - np.repeat(queries, 10, axis=0).astype(np.float64)) ** 2).sum(1)
-    assert np.array_equal(dists.reshape(-1), np.sqrt(sq.astype(np.float32)))
+    if world["exact"]:
+        assert np.array_equal(dists.reshape(-1), np.sqrt(sq.astype(np.float32)))
+    else:
+        assert np.allclose(dists.reshape(-1), sq if world["metric"] == 1 else np.sqrt(sq), rtol=1e-5, atol=1e-7)
     # the order and the batching of the queries do not matter
     perm = np.random.default_rng(1).permutation(NQ)
     p_ids, p_dists = world["index"].search(sp, hip.DeviceArray.from_numpy(np.ascontiguousarray(queries[perm])))
