@@ -111,8 +111,9 @@ template <int MAX_CAND, int MAX_BEAM, int DIMV>
 __global__ __launch_bounds__(64) void refine_kernel(RefineArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     auto* lds = reinterpret_cast<BeamLds<MAX_CAND>*>(smem);
-    auto* pl = reinterpret_cast<PruneLds<MAX_BEAM>*>(smem + sizeof(BeamLds<MAX_CAND>));
-    float* cent = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>) + sizeof(PruneLds<MAX_BEAM>));
+    using Prune = PruneLds<MAX_BEAM, (MAX_CAND < 64 ? 64 : MAX_CAND)>;   // the row has at most MAX_CAND slots here
+    auto* pl = reinterpret_cast<Prune*>(smem + sizeof(BeamLds<MAX_CAND>));
+    float* cent = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>) + sizeof(Prune));
     uint32_t* hash = reinterpret_cast<uint32_t*>(cent + round_up32(a.centroid_num));
     if (blockIdx.x >= a.num) return;
     const uint32_t point = a.order ? a.order[blockIdx.x] : blockIdx.x;
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(64) void refine_kernel(RefineArgs a) {
     uint32_t* out_row = a.graph_out + static_cast<size_t>(point) * D;
 
     uint32_t need = 0;
-    for (uint32_t base = 0; base < kMaxDegree; base += 64) {
+    for (uint32_t base = 0; base < Prune::kCap; base += 64) {
         const uint32_t i = base + lane;
         const uint32_t g = i < D ? in_row[i] : kInvalid;
         pl->s_graph[i] = g;
@@ -319,6 +320,15 @@ refine_fn pick_refine_beam(uint32_t beam, uint32_t dim) {
 
 size_t prune_lds_bytes(uint32_t beam) {
     return beam <= 64 ? sizeof(PruneLds<64>) : beam <= 128 ? sizeof(PruneLds<128>) : beam <= 256 ? sizeof(PruneLds<256>) : sizeof(PruneLds<512>);
+}
+// the refine kernel's layout: row arrays sized by the degree bucket instead of the maximum degree
+template <int CAP>
+size_t prune_lds_bytes_cap(uint32_t beam) {
+    return beam <= 64 ? sizeof(PruneLds<64, CAP>) : beam <= 128 ? sizeof(PruneLds<128, CAP>) : beam <= 256 ? sizeof(PruneLds<256, CAP>)
+                                                                                                          : sizeof(PruneLds<512, CAP>);
+}
+size_t prune_lds_bytes_refine(uint32_t beam, uint32_t degree) {
+    return degree <= 64 ? prune_lds_bytes_cap<64>(beam) : degree <= 128 ? prune_lds_bytes_cap<128>(beam) : prune_lds_bytes_cap<256>(beam);
 }
 
 int check_beam_sizes(uint32_t degree, uint32_t graph_degree, uint32_t beam, uint32_t dim, uint32_t hash_bit, int metric) {
@@ -564,7 +574,7 @@ int launch_refine(const float* data, uint32_t num, uint32_t dim, const uint32_t*
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
     refine_fn fn = graph_degree <= 64 ? pick_refine_beam<64>(beam, dim)
                  : graph_degree <= 128 ? pick_refine_beam<128>(beam, dim) : pick_refine_beam<256>(beam, dim);
-    const size_t lds_bytes = beam_lds_bytes(graph_degree) + prune_lds_bytes(beam) + round_up32(centroid_num) * sizeof(float) +
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + prune_lds_bytes_refine(beam, graph_degree) + round_up32(centroid_num) * sizeof(float) +
                              (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(num), dim3(64), lds_bytes, as_stream(stream), a);

@@ -8,21 +8,26 @@ namespace glide {
 
 constexpr uint32_t kMaxDegree = 256;   // largest graph / kNN degree (reference kernel_config.cuh:53-60)
 
-template <int MAX_BEAM>
+// DCAP = capacity of the per-row arrays: a multiple of 64 that is at least round_up32(graph_degree).  The refine kernel
+// sizes it by its degree bucket (less LDS per wavefront, more wavefronts per CU); the build kernels, whose output
+// degree is independent of the degree bucket of the kNN graph they search, keep the maximum.
+template <int MAX_BEAM, int DCAP = static_cast<int>(kMaxDegree)>
 struct PruneLds {
+    static_assert(DCAP % 64 == 0 && DCAP <= static_cast<int>(kMaxDegree), "row capacity");
+    static constexpr uint32_t kCap = DCAP;
     uint32_t pool_id[MAX_BEAM];
     float pool_dist[MAX_BEAM];
     uint32_t keep[MAX_BEAM];
-    uint32_t neighbor[kMaxDegree];   // round_up32(graph_degree) <= kMaxDegree
-    uint32_t s_graph[kMaxDegree];
-    uint32_t fresh[kMaxDegree];
-    uint32_t dup_mask[kMaxDegree / 32];
+    uint32_t neighbor[DCAP];
+    uint32_t s_graph[DCAP];
+    uint32_t fresh[DCAP];
+    uint32_t dup_mask[DCAP / 32];
 };
 
 // Beam registers -> LDS pool in rank order with the explored bit stripped (graph_kernel.cuh:65-67), dropping
 // slots that never held a node (their id would be dereferenced by the reference).  Returns the pool size.
-template <int MAX_CAND, int MAX_BEAM, int DIMV>
-__device__ __forceinline__ uint32_t beam_to_pool(Beam<MAX_CAND, MAX_BEAM, DIMV>& b, PruneLds<MAX_BEAM>* pl) {
+template <int MAX_CAND, int MAX_BEAM, int DIMV, class PL>
+__device__ __forceinline__ uint32_t beam_to_pool(Beam<MAX_CAND, MAX_BEAM, DIMV>& b, PL* pl) {
     constexpr int NB = MAX_BEAM / 64;
     // rank order is e = NB*lane + r; compact register by register would break the order, so stage then compact
 #pragma unroll
@@ -52,8 +57,8 @@ __device__ __forceinline__ uint32_t beam_to_pool(Beam<MAX_CAND, MAX_BEAM, DIMV>&
 }
 
 // stable compaction of the pool by the keep flags of entries [first, pool_size)
-template <int MAX_BEAM>
-__device__ __forceinline__ uint32_t compact_pool(PruneLds<MAX_BEAM>* pl, uint32_t first, uint32_t pool_size, int lane) {
+template <int MAX_BEAM, class PL>
+__device__ __forceinline__ uint32_t compact_pool(PL* pl, uint32_t first, uint32_t pool_size, int lane) {
     uint32_t n = 0;
     for (uint32_t base = 0; base < pool_size; base += 64) {
         const uint32_t i = base + lane;
@@ -74,11 +79,11 @@ __device__ __forceinline__ uint32_t compact_pool(PruneLds<MAX_BEAM>* pl, uint32_
 }
 
 // sync_prune: returns the neighbour count; pl->neighbor[0..round_up32(D)) holds ids (+segment_start) or invalid
-template <int MAX_BEAM, int DIMV>
-__device__ __forceinline__ uint32_t prune_pool(PruneLds<MAX_BEAM>* pl, uint32_t pool_size, const float* data, uint32_t dim,
+template <int MAX_BEAM, int DIMV, class PL>
+__device__ __forceinline__ uint32_t prune_pool(PL* pl, uint32_t pool_size, const float* data, uint32_t dim,
                                                uint32_t segment_start, uint32_t graph_degree, float relaxant, int metric,
                                                int lane, uint32_t& rows_scored) {
-    for (uint32_t i = lane; i < kMaxDegree; i += 64) pl->neighbor[i] = kInvalid;
+    for (uint32_t i = lane; i < PL::kCap; i += 64) pl->neighbor[i] = kInvalid;
     wave_sync();
     uint32_t nsize = 0;
     while (nsize < graph_degree && pool_size > 0) {
@@ -98,11 +103,11 @@ __device__ __forceinline__ uint32_t prune_pool(PruneLds<MAX_BEAM>* pl, uint32_t 
 }
 
 // sync_prune_refine: heads must be valid, differ from `self` and not already be in the row (pl->s_graph)
-template <int MAX_BEAM, int DIMV>
-__device__ __forceinline__ uint32_t prune_pool_refine(PruneLds<MAX_BEAM>* pl, uint32_t pool_size, const float* data, uint32_t dim,
+template <int MAX_BEAM, int DIMV, class PL>
+__device__ __forceinline__ uint32_t prune_pool_refine(PL* pl, uint32_t pool_size, const float* data, uint32_t dim,
                                                       uint32_t self, uint32_t graph_degree, uint32_t need, float relaxant,
                                                       int metric, int lane, uint32_t& rows_scored) {
-    for (uint32_t i = lane; i < kMaxDegree; i += 64) pl->neighbor[i] = kInvalid;
+    for (uint32_t i = lane; i < PL::kCap; i += 64) pl->neighbor[i] = kInvalid;
     wave_sync();
     uint32_t nsize = 0;
     while (nsize < need && pool_size > 0) {
@@ -135,12 +140,12 @@ __device__ __forceinline__ uint32_t prune_pool_refine(PruneLds<MAX_BEAM>* pl, ui
 }
 
 // map_to_graph_boundary: merge the boundary copy's neighbours (reorder ids in pl->neighbor) into `row`
-template <int MAX_BEAM>
-__device__ __forceinline__ void merge_boundary_row(PruneLds<MAX_BEAM>* pl, uint32_t* row, const uint32_t* map,
+template <int MAX_BEAM, class PL>
+__device__ __forceinline__ void merge_boundary_row(PL* pl, uint32_t* row, const uint32_t* map,
                                                    uint32_t graph_degree, int lane) {
     const uint32_t max_degree = round_up32(graph_degree);
-    for (uint32_t i = lane; i < kMaxDegree; i += 64) pl->s_graph[i] = i < graph_degree ? row[i] : kInvalid;
-    if (lane < static_cast<int>(kMaxDegree / 32)) pl->dup_mask[lane] = 0;
+    for (uint32_t i = lane; i < PL::kCap; i += 64) pl->s_graph[i] = i < graph_degree ? row[i] : kInvalid;
+    if (lane < static_cast<int>(PL::kCap / 32)) pl->dup_mask[lane] = 0;
     wave_sync();
     uint32_t nfresh = 0, ndup = 0;
     for (uint32_t base = 0; base < max_degree; base += 64) {
