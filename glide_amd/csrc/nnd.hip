@@ -462,19 +462,26 @@ struct Net64 {
                 }
             }
         } else {
+            // Two entries with equal keys are copies of one offer (same distance, id, source and flag), so exchanging
+            // them or not gives the same sequence: one compare decides, and the lanes that keep the larger key take the
+            // partner's entry exactly where the others would not (the complement of the compare mask).
             constexpr int LM = J / NR;
-            const bool lower = (lane & LM) == 0;
 #pragma unroll
             for (int r = 0; r < NR; r++) {
-                const int e = NR * lane + r;
-                const bool asc = (K >= M) ? true : ((e & K) == 0);
+                uint64_t keep_min = 0;   // compile-time pattern: lower partner of an ascending pair, upper of a descending one
+                for (int l = 0; l < 64; l++) {
+                    const int e = NR * l + r;
+                    const bool asc = (K >= M) ? true : ((e & K) == 0);
+                    if (((l & LM) == 0) == asc) keep_min |= 1ull << l;
+                }
                 const unsigned long long ok = xor_lane<LM>(k[r]);
                 const uint32_t ov = lane_xor<LM>(v[r]);
-                const bool keep_min = lower == asc;
-                if (keep_min ? (ok < k[r]) : (ok > k[r])) {
-                    k[r] = ok;
-                    v[r] = ov;
-                }
+                const uint64_t less = __builtin_amdgcn_ballot_w64(ok < k[r]);
+                const uint64_t take = less ^ ~keep_min;
+                const uint32_t lo = select_by_mask(static_cast<uint32_t>(k[r]), static_cast<uint32_t>(ok), take);
+                const uint32_t hi = select_by_mask(static_cast<uint32_t>(k[r] >> 32), static_cast<uint32_t>(ok >> 32), take);
+                k[r] = (static_cast<unsigned long long>(hi) << 32) | lo;
+                v[r] = select_by_mask(v[r], ov, take);
             }
         }
     }
