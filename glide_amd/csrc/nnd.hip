@@ -502,15 +502,19 @@ struct Net64 {
 __device__ __forceinline__ uint32_t bloom_h0(uint32_t v) { v *= 1103515245u; v += 12345u; v ^= v << 13; v ^= v >> 17; v ^= v << 5; return v; }
 __device__ __forceinline__ uint32_t bloom_h1(uint32_t v) { v *= 1664525u; v += 1013904223u; v ^= v << 13; v ^= v >> 17; v ^= v << 5; return v; }
 
+// Prefix sum over the 64 lanes without LDS traffic: four shifted adds inside each row of 16 lanes, then lane 15 of a row
+// is added to the next row (rows 1 and 3) and lane 31 to the upper half (rows 2 and 3).  Lanes a step does not feed add 0.
 __device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane, uint32_t& total) {
-    uint32_t incl = value;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const uint32_t o = __shfl_up(incl, off);
-        if (lane >= off) incl += o;
-    }
-    total = __shfl(incl, 63);
-    return incl - value;
+    (void) lane;
+    int x = static_cast<int>(value);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, true);   // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, true);   // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, true);   // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, true);   // row_shr:8
+    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, true);   // row_bcast:15
+    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, true);   // row_bcast:31
+    total = static_cast<uint32_t>(__builtin_amdgcn_readlane(x, 63));
+    return static_cast<uint32_t>(x) - value;
 }
 
 // Merge + resample, one wavefront per node.  The reference keeps, per node and round, a 32-wide sorted "device" list of
@@ -581,7 +585,10 @@ __device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists
     // represents the offer; it is "known" when the list already holds the id.
     bool from_list[NR], first_offer[NR], known[NR];
     uint32_t offer_count = 0;
-    const unsigned long long last_of_prev = __shfl_up(k[NR - 1], 1);
+    // the previous lane's last key (wave_shr:1; lane 0 has no predecessor and is handled as the head below)
+    const unsigned long long last_of_prev =
+        (static_cast<unsigned long long>(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[NR - 1] >> 32), 0x138, 0xf, 0xf, false))) << 32) |
+        static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[NR - 1]), 0x138, 0xf, 0xf, false));
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         const unsigned long long prev = r == 0 ? last_of_prev : k[r - 1];
