@@ -712,9 +712,39 @@ __global__ __launch_bounds__(256) void kmeanspp_distance_kernel(const float* sam
 }
 
 // ---- Lloyd k-means on a sample (stand-in for cuvs::cluster::kmeans::fit, reference partition.cuh:48-54) ----
+// The sums are kept in 64-bit fixed point: integer addition does not depend on the order in which the atomics
+// arrive, so a fit is reproducible bit for bit.  The scale is the largest power of two for which sample_num values of
+// the largest magnitude still fit (2^35 for 500 000 rows of 0..255 data: every value exact; on unit-norm data values
+// below 2^-19 are rounded to 2^-43).
+
+// largest |value| of the sample, as the bit pattern of a non-negative float (which orders like the unsigned integer)
+__global__ __launch_bounds__(256) void kmeans_range_kernel(const float* sample, size_t count, uint32_t* max_bits) {
+    uint32_t m = 0;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += static_cast<size_t>(gridDim.x) * 256) {
+        const uint32_t b = __float_as_uint(sample[i]) & 0x7fffffffu;
+        m = b > m ? b : m;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(m), off));
+        m = o > m ? o : m;
+    }
+    if (lane_id() == 0 && m) atomicMax(max_bits, m);
+}
+
+// scale = 2^e with max|x| * n * 2^e < 2^62
+__device__ __forceinline__ float kmeans_scale(uint32_t max_bits, uint32_t n) {
+    const float bound = fmaxf(__uint_as_float(max_bits), 1e-30f) * static_cast<float>(n);
+    int e = 0;
+    frexpf(bound, &e);           // bound < 2^e
+    e = 62 - e;
+    e = e > 100 ? 100 : e;
+    return ldexpf(1.f, e);
+}
+
 // one wavefront per sample point: nearest centroid by direct distances, then atomic accumulation
 __global__ __launch_bounds__(256) void kmeans_accumulate_kernel(const float* sample, uint32_t n, uint32_t dim, const float* centroids,
-                                                                uint32_t k, float* sums, uint32_t* counts) {
+                                                                uint32_t k, long long* sums, uint32_t* counts, const uint32_t* max_bits) {
     const int lane = lane_id();
     const int half = lane >> 5, t = lane & 31;
     const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -729,15 +759,21 @@ __global__ __launch_bounds__(256) void kmeans_accumulate_kernel(const float* sam
         if (da < best) { best = da; bc = c0; }
         if (c0 + 1 < k && db < best) { best = db; bc = c0 + 1; }
     }
-    for (uint32_t d = lane; d < dim; d += 64) atomicAdd(&sums[static_cast<size_t>(bc) * dim + d], x[d]);
+    const float scale = kmeans_scale(*max_bits, n);
+    for (uint32_t d = lane; d < dim; d += 64)
+        atomicAdd(reinterpret_cast<unsigned long long*>(&sums[static_cast<size_t>(bc) * dim + d]),
+                  static_cast<unsigned long long>(__float2ll_rn(x[d] * scale)));   // two's complement: the wrap-around sum is the signed sum
     if (lane == 0) atomicAdd(&counts[bc], 1u);
 }
 
-__global__ void kmeans_update_kernel(float* centroids, const float* sums, const uint32_t* counts, uint32_t k, uint32_t dim) {
+__global__ void kmeans_update_kernel(float* centroids, const long long* sums, const uint32_t* counts, uint32_t k, uint32_t dim, uint32_t n,
+                                     const uint32_t* max_bits) {
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= k * dim) return;
     const uint32_t c = idx / dim;
-    if (counts[c]) centroids[idx] = sums[idx] / static_cast<float>(counts[c]);   // an empty cluster keeps its centroid
+    if (counts[c])   // an empty cluster keeps its centroid
+        centroids[idx] = static_cast<float>(static_cast<double>(sums[idx]) / static_cast<double>(kmeans_scale(*max_bits, n)) /
+                                            static_cast<double>(counts[c]));
 }
 
 size_t assign_lds_bytes(int cb, uint32_t centroid_num) {
@@ -829,7 +865,8 @@ int glide_hip_sample_rows(const float* data, uint32_t dim, const uint32_t* sampl
 }
 
 size_t glide_hip_kmeans_workspace_bytes(uint32_t cluster_num, uint32_t dim) {
-    return static_cast<size_t>(cluster_num) * dim * 4 + static_cast<size_t>(cluster_num) * 4 + 256;
+    // sums (i64 per centroid component) | counts (u32 per centroid) | the sample's largest magnitude
+    return static_cast<size_t>(cluster_num) * dim * 8 + static_cast<size_t>(cluster_num) * 4 + 256;
 }
 
 size_t glide_hip_kmeans_seed_workspace_bytes(uint32_t sample_num) {
@@ -869,16 +906,23 @@ int glide_hip_kmeans_fit(const float* sample, uint32_t sample_num, uint32_t dim,
     if (dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
     if (workspace_bytes < glide_hip_kmeans_workspace_bytes(cluster_num, dim)) return GLIDE_ERR_BAD_ARGUMENT;
     hipStream_t s = as_stream(stream);
-    float* sums = static_cast<float*>(workspace);
+    if (reinterpret_cast<uintptr_t>(workspace) % 8) return GLIDE_ERR_BAD_ARGUMENT;
+    long long* sums = static_cast<long long*>(workspace);
     uint32_t* counts = reinterpret_cast<uint32_t*>(sums + static_cast<size_t>(cluster_num) * dim);
-    const size_t words = static_cast<size_t>(cluster_num) * dim + cluster_num;
+    uint32_t* max_bits = counts + cluster_num;
+    const size_t words = static_cast<size_t>(cluster_num) * dim * 2 + cluster_num;
+    int rc = glide_hip_fill_u32(max_bits, 0u, 1, stream);
+    if (rc != GLIDE_OK) return rc;
+    const size_t values = static_cast<size_t>(sample_num) * dim;
+    hipLaunchKernelGGL(kmeans_range_kernel, dim3(static_cast<uint32_t>(values / 256 < 4096 ? values / 256 + 1 : 4096)), dim3(256), 0, s, sample,
+                       values, max_bits);
     for (uint32_t it = 0; it < iterations; it++) {
-        int rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(sums), 0u, words, stream);
+        rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(sums), 0u, words, stream);
         if (rc != GLIDE_OK) return rc;
         hipLaunchKernelGGL(kmeans_accumulate_kernel, dim3(ceil_div(sample_num, 4)), dim3(256), 0, s, sample, sample_num, dim, centroids,
-                           cluster_num, sums, counts);
+                           cluster_num, sums, counts, max_bits);
         hipLaunchKernelGGL(kmeans_update_kernel, dim3(ceil_div(cluster_num * dim, 256)), dim3(256), 0, s, centroids, sums, counts,
-                           cluster_num, dim);
+                           cluster_num, dim, sample_num, max_bits);
     }
     return launch_status();
 }

@@ -109,7 +109,8 @@ int glide_hip_sample_rows(const float *data, uint32_t dim, const uint32_t *sampl
  * sample rows drawn with probability proportional to their squared distance from the nearest centroid chosen so
  * far, best = smallest remaining potential (cuVS initialises with its k-means++ family by default).  The draws are a
  * hash of (seed, step, trial), so a run is reproducible.  chosen_rows (nullable, cluster_num u32) receives the sample
- * rows taken.  workspace: 8-byte aligned.  glide_hip_kmeans_fit: `iterations` Lloyd steps from the centroids passed in. */
+ * rows taken.  workspace: 8-byte aligned.  glide_hip_kmeans_fit: `iterations` Lloyd steps from the centroids passed in;
+ * the cluster sums are accumulated in 64-bit fixed point, so a fit is reproducible bit for bit (workspace: 8-byte aligned). */
 size_t glide_hip_kmeans_seed_workspace_bytes(uint32_t sample_num);
 int glide_hip_kmeans_seed(const float *sample, uint32_t sample_num, uint32_t dim, uint32_t cluster_num, uint32_t seed,
                           float *centroids, uint32_t *chosen_rows, void *workspace, size_t workspace_bytes,

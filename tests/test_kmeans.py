@@ -91,3 +91,33 @@ def test_gpu_kmeans_against_scikit_learn(case):
         hip.synchronize()
         got.append(inertia(x, cent.numpy()))
     assert np.median(got) <= 1.02 * case["median"], (np.median(got), case["median"])
+
+
+@pytest.mark.gpu
+def test_gpu_kmeans_fit_is_reproducible():
+    """Sums are accumulated in fixed point, so the order in which the atomics arrive cannot change a fit: float data with
+    many clusters, several runs, bit-identical centroids; and they agree with a float64 Lloyd from the same start."""
+    from glide_amd import capi as hip, datasets as D
+    hip.set_device(0)
+    n, dim, k = 60_000, 96, 48
+    x = D.gmm_normalized(n, dim, seed=3)
+    start = x[np.random.default_rng(0).choice(n, k, replace=False)].copy()
+    d_x = hip.DeviceArray.from_numpy(x)
+    wb = hip.kmeans_workspace_bytes(k, dim)
+    ws = hip.DeviceArray(wb // 8 + 1, np.uint64)
+    runs = []
+    for _ in range(4):
+        cent = hip.DeviceArray.from_numpy(start)
+        hip.kmeans_fit(d_x, n, dim, k, 10, cent, ws, wb)
+        hip.synchronize()
+        runs.append(cent.numpy())
+    for r in runs[1:]:
+        assert np.array_equal(r, runs[0])
+    c = start.astype(np.float64)
+    x64 = x.astype(np.float64)
+    for _ in range(10):
+        lab = ((x64 ** 2).sum(1)[:, None] + (c ** 2).sum(1)[None] - 2.0 * x64 @ c.T).argmin(1)
+        for j in range(k):
+            if (lab == j).any():
+                c[j] = x64[lab == j].mean(0)
+    assert np.allclose(runs[0], c, rtol=1e-4, atol=1e-5)
