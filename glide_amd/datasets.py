@@ -47,7 +47,7 @@ def beta_scaled(num, dim=960, components=128, seed=1234, mixture_seed=97):
 
 
 def lowdim_integer(num, dim=128, latent=12, spread=20.0, noise=3.0, seed=1234, mixture_seed=0):
-    """A `latent`-dimensional Gaussian cloud mapped linearly into `dim` dimensions around 128, plus a little noise,
+    """A `latent`-dimensional Gaussian cloud mapped linearly into `dim` dimensions, centred on 128, plus a little noise,
     clipped to [0, 255] and rounded: integer-valued data of low intrinsic dimension, on which graph search navigates
     well.  The linear map depends only on `mixture_seed`."""
     a = np.random.default_rng(mixture_seed).standard_normal((latent, dim)).astype(np.float32)
