@@ -27,8 +27,8 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE, KiB per dispatch) and scaled by what the same counters report for copy_kernel moving exactly 1 GiB
 # (--copy-calibration: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Keyed by (workload, beam); other combinations report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg1", 256): 6_302_400 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
-    ("cfg1-navigable", 32): 2_449_100 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
+    ("cfg1", 256): 6_383_100 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
+    ("cfg1-navigable", 32): 2_449_600 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
 }
 
 
