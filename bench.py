@@ -223,9 +223,10 @@ def run_workload(args, workload, torch, want_cpu):
         qps=nq * args.steps / (wall_ms * 1e-3), ms_per_step=ms_per_step, kernel_ms=kernel_ms,
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=MEASURED_TRAFFIC_BYTES.get((workload, chosen["beam"])),
-                      kernel="search_kernel<%d,%d,%d>" % (64 if degree <= 64 else 128 if degree <= 128 else 256,
-                                                          64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256 if chosen["beam"] <= 256 else 512,
-                                                          1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8),
+                      kernel="%s<%d,%d,%d>" % ("search_kernel_dense" if 128 < chosen["beam"] <= 256 and degree <= 128 and dim <= 512 else "search_kernel",
+                                               64 if degree <= 64 else 128 if degree <= 128 else 256,
+                                               64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256 if chosen["beam"] <= 256 else 512,
+                                               1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8),
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )
 
