@@ -246,24 +246,25 @@ def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt, m
     except Exception:
         pass
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    nq = min(queries.shape[0], 4000)
+    nq = min(queries.shape[0], 10_000)
     t = time.time()
     ids, _, _ = O.search(data, graph, centroids, start_points, queries[:nq], top_k, sp.beam, sp.max_iterations, sp.min_iterations,
                          sp.hash_bit, sp.hash_reset_interval, metric, threads=cores)
     search_s = time.time() - t
-    # NN-descent build of one 30k-point partition-sized sample with the same degree / 10 iterations
-    n_s = min(30_000, data.shape[0])
+    # NN-descent build of one partition-sized sample (1M / 16 points) with the same degree / 10 iterations
+    n_s = min(62_500, data.shape[0])
     t = time.time()
     O.nnd_build(data[:n_s], np.array([0], np.uint32), np.array([n_s], np.uint32), 32, 10, 0, threads=cores)
     nnd_s = time.time() - t
     t = time.time()
-    O.bruteforce_knn(data[:200_000], queries[:200], top_k, metric, threads=cores)
+    n_bf = min(queries.shape[0], 1000)
+    O.bruteforce_knn(data, queries[:n_bf], top_k, metric, threads=cores)
     bf_s = time.time() - t
     return dict(value=nq / search_s, unit="queries/s", cores=cores, kind="port",
                 sample="beam search of the first %d queries (same index, beam %d) with the CPU restatement, %d threads" % (nq, sp.beam, cores),
                 recall_at_10=D.recall(ids, gt[:nq], top_k),
                 nnd_points_per_sec=n_s / nnd_s, nnd_sample="NN-descent k=32 x 10 iterations on the first %d points as one partition" % n_s,
-                bruteforce_qps=200 / bf_s * (200_000 / data.shape[0]), bruteforce_sample="exact top-10 of 200 queries over 200k rows, scaled to the full set")
+                bruteforce_qps=n_bf / bf_s, bruteforce_sample="exact top-%d of the first %d queries over all %d rows" % (top_k, n_bf, data.shape[0]))
 
 
 def main():
