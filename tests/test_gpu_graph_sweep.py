@@ -14,7 +14,7 @@ def _cases():
     degrees = [8, 24, 32, 64, 96, 160]
     beams = [32, 64, 128, 256, 320]
     out = []
-    for i in range(14):
+    for i in range(28):
         out.append((i, int(rng.choice(dims)), int(rng.choice(degrees)), int(rng.choice(degrees)), int(rng.choice(beams)), int(rng.choice(beams)),
                     int(rng.integers(0, 2))))
     return out

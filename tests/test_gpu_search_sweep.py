@@ -13,7 +13,7 @@ def _cases():
     degrees = [8, 16, 24, 32, 40, 64, 72, 96, 128, 160, 256]
     beams = [32, 64, 96, 128, 192, 256, 320, 512]
     out = []
-    for i in range(36):
+    for i in range(72):
         dim, deg, beam = int(rng.choice(dims)), int(rng.choice(degrees)), int(rng.choice(beams))
         top_k = int(rng.integers(1, min(beam, 128) + 1))
         cents = int(rng.choice([1, 2, 7, 32, 33, 64, 100, 200]))
