@@ -277,6 +277,22 @@ def partition_assign(data, num, dim, centroids, centroid_num, boundary_factor, m
                                            C.c_size_t(workspace_bytes), vp(stream)), "glide_hip_partition_assign")
 
 
+def partition_assign_fixed_max_points():
+    f = lib().glide_hip_partition_assign_fixed_max_points
+    f.restype = C.c_uint32
+    return int(f())
+
+
+def partition_assign_fixed(data, num, dim, centroids, centroid_num, boundary_factor, metric, segment_indexes,
+                           segment_lengths, nearest_dists, stream=None, check_status=True):
+    rc = lib().glide_hip_partition_assign_fixed(_ptr(data), u32(num), u32(dim), _ptr(centroids), u32(centroid_num),
+                                                f32(boundary_factor), C.c_int(metric), _ptr(segment_indexes),
+                                                _ptr(segment_lengths), _ptr(nearest_dists), vp(stream))
+    if check_status:
+        check(rc, "glide_hip_partition_assign_fixed")
+    return rc
+
+
 def reorder(data, num, dim, segment_indexes, segment_starts, reorder_data, mp, stream=None):
     check(lib().glide_hip_reorder(_ptr(data), u32(num), u32(dim), _ptr(segment_indexes), _ptr(segment_starts),
                                   _ptr(reorder_data), _ptr(mp), vp(stream)), "glide_hip_reorder")

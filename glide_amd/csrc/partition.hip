@@ -4,6 +4,7 @@
 // (:7-20), host sequencing partition.cuh:8-193.
 #include "common.hpp"
 #include "host_util.hpp"
+#include <mutex>
 
 namespace glide {
 
@@ -795,16 +796,10 @@ size_t glide_hip_partition_assign_workspace_bytes(uint32_t num, uint32_t centroi
     return tiles * (centroid_num + 1) * 4 + static_cast<size_t>(centroid_num) * 4 + 256;
 }
 
-int glide_hip_partition_assign(const float* data, uint32_t num, uint32_t dim, const float* centroids, uint32_t centroid_num,
-                               float boundary_factor, int metric, uint32_t* segment_indexes, uint32_t* segment_lengths,
-                               float* nearest_dists, void* workspace, size_t workspace_bytes, void* stream) {
-    if (!data || !centroids || !segment_indexes || !segment_lengths || !workspace) return GLIDE_ERR_BAD_ARGUMENT;
-    if (dim == 0 || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
-    if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
-    if (centroid_num > 256 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // reference buckets: kernel_config.cuh:224-234
-    if (workspace_bytes < glide_hip_partition_assign_workspace_bytes(num, centroid_num)) return GLIDE_ERR_BAD_ARGUMENT;
-    hipStream_t s = as_stream(stream);
-    if (num == 0) return glide_hip_fill_u32(segment_lengths, 0u, centroid_num + 1, stream);
+namespace {
+// The launches of glide_hip_partition_assign on a checked workspace: norms (centroid_num floats, padded to 256 bytes) followed by the tile histograms.
+int assign_on_workspace(const float* data, uint32_t num, uint32_t dim, const float* centroids, uint32_t centroid_num, float boundary_factor,
+                        int metric, uint32_t* segment_indexes, uint32_t* segment_lengths, float* nearest_dists, void* workspace, hipStream_t s) {
     const uint32_t tiles = ceil_div(num, kTilePoints);
     float* norms = static_cast<float*>(workspace);
     uint32_t* tile_hist = reinterpret_cast<uint32_t*>(static_cast<unsigned char*>(workspace) + ((static_cast<size_t>(centroid_num) * 4 + 255) / 256) * 256);
@@ -820,24 +815,90 @@ int glide_hip_partition_assign(const float* data, uint32_t num, uint32_t dim, co
             case 3: hipLaunchKernelGGL(assign_resident_kernel<3>, dim3(tiles), dim3(256), rlds, s, a); break;
             default: hipLaunchKernelGGL(assign_resident_kernel<4>, dim3(tiles), dim3(256), rlds, s, a); break;
         }
-        hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(kScanThreads), 0, s, tile_hist, tiles, centroid_num + 1, segment_lengths);
-        hipLaunchKernelGGL(slot_kernel, dim3(tiles), dim3(kTilePoints), 0, s, segment_indexes, tile_hist, num, centroid_num);
-        return launch_status();
+    } else {
+        const size_t lds = assign_lds_bytes(cb, centroid_num);
+        if (lds > 64 * 1024) {
+            GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&assign_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              static_cast<int>(lds)));
+        }
+        switch (cb) {
+            case 1: hipLaunchKernelGGL(assign_kernel<1>, dim3(tiles), dim3(256), lds, s, a); break;
+            case 2: hipLaunchKernelGGL(assign_kernel<2>, dim3(tiles), dim3(256), lds, s, a); break;
+            case 4: hipLaunchKernelGGL(assign_kernel<4>, dim3(tiles), dim3(256), lds, s, a); break;
+            default: hipLaunchKernelGGL(assign_kernel<8>, dim3(tiles), dim3(256), lds, s, a); break;
+        }
     }
-    const size_t lds = assign_lds_bytes(cb, centroid_num);
-    if (lds > 64 * 1024) {
-        GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&assign_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          static_cast<int>(lds)));
-    }
-    switch (cb) {
-        case 1: hipLaunchKernelGGL(assign_kernel<1>, dim3(tiles), dim3(256), lds, s, a); break;
-        case 2: hipLaunchKernelGGL(assign_kernel<2>, dim3(tiles), dim3(256), lds, s, a); break;
-        case 4: hipLaunchKernelGGL(assign_kernel<4>, dim3(tiles), dim3(256), lds, s, a); break;
-        default: hipLaunchKernelGGL(assign_kernel<8>, dim3(tiles), dim3(256), lds, s, a); break;
-    }
+    // every tile has written all centroid_num + 1 bins of its histogram: nothing in the workspace has to start at zero
     hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(kScanThreads), 0, s, tile_hist, tiles, centroid_num + 1, segment_lengths);
     hipLaunchKernelGGL(slot_kernel, dim3(tiles), dim3(kTilePoints), 0, s, segment_indexes, tile_hist, num, centroid_num);
     return launch_status();
+}
+
+int assign_check(const float* data, uint32_t dim, const float* centroids, uint32_t centroid_num, int metric, const uint32_t* segment_indexes,
+                 const uint32_t* segment_lengths) {
+    if (!data || !centroids || !segment_indexes || !segment_lengths) return GLIDE_ERR_BAD_ARGUMENT;
+    if (dim == 0 || centroid_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
+    if (centroid_num > 256 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // reference buckets: kernel_config.cuh:224-234
+    return GLIDE_OK;
+}
+}  // namespace
+
+int glide_hip_partition_assign(const float* data, uint32_t num, uint32_t dim, const float* centroids, uint32_t centroid_num,
+                               float boundary_factor, int metric, uint32_t* segment_indexes, uint32_t* segment_lengths,
+                               float* nearest_dists, void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = assign_check(data, dim, centroids, centroid_num, metric, segment_indexes, segment_lengths);
+    if (rc != GLIDE_OK) return rc;
+    if (!workspace || workspace_bytes < glide_hip_partition_assign_workspace_bytes(num, centroid_num)) return GLIDE_ERR_BAD_ARGUMENT;
+    if (num == 0) return glide_hip_fill_u32(segment_lengths, 0u, centroid_num + 1, stream);
+    return assign_on_workspace(data, num, dim, centroids, centroid_num, boundary_factor, metric, segment_indexes, segment_lengths, nearest_dists,
+                               workspace, as_stream(stream));
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------------------------
+// glide_hip_partition_assign with its workspace (centroid norms + per-tile histograms) in a file-scope device array,
+// for callers that cannot allocate: code under graph capture, serving loops that route batches of new points or
+// queries to their partitions.  Every GPU holds its own copy of the array until the process ends; its address on a
+// device is looked up once, with that device current, and kept.
+constexpr uint32_t kFixedMaxPoints = 65536;   // per call
+constexpr size_t kFixedScratchBytes = 1024 + static_cast<size_t>(kFixedMaxPoints / kTilePoints) * (256 + 1) * 4;   // norms | 512 tiles x 257 bins
+static __device__ __align__(256) unsigned char scratch[kFixedScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[kMaxDevices];   // device address of `scratch` per device, null until looked up
+
+int scratch_on_current_device(void** out) {
+    int device = 0;
+    GLIDE_HIP_TRY(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return GLIDE_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> guard(scratch_mutex);
+    if (!scratch_ptr[device]) {
+        void* p = nullptr;
+        GLIDE_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return GLIDE_ERR_NO_DEVICE;
+        scratch_ptr[device] = p;
+    }
+    *out = scratch_ptr[device];
+    return GLIDE_OK;
+}
+}  // namespace
+
+uint32_t glide_hip_partition_assign_fixed_max_points(void) { return kFixedMaxPoints; }
+
+int glide_hip_partition_assign_fixed(const float* data, uint32_t num, uint32_t dim, const float* centroids, uint32_t centroid_num,
+                                     float boundary_factor, int metric, uint32_t* segment_indexes, uint32_t* segment_lengths,
+                                     float* nearest_dists, void* stream) {
+    int rc = assign_check(data, dim, centroids, centroid_num, metric, segment_indexes, segment_lengths);
+    if (rc != GLIDE_OK) return rc;
+    if (num > kFixedMaxPoints) return GLIDE_ERR_UNSUPPORTED;   // the array holds the histograms of 65536 points
+    static_assert(kFixedScratchBytes >= 1024 + (kFixedMaxPoints / kTilePoints) * 257 * 4, "scratch too small for the largest call");
+    void* ws = nullptr;
+    if ((rc = scratch_on_current_device(&ws)) != GLIDE_OK) return rc;
+    if (num == 0) return glide_hip_fill_u32(segment_lengths, 0u, centroid_num + 1, stream);   // a fill kernel, no memset node
+    return assign_on_workspace(data, num, dim, centroids, centroid_num, boundary_factor, metric, segment_indexes, segment_lengths, nearest_dists,
+                               ws, as_stream(stream));
 }
 
 int glide_hip_reorder_batch(const float* data, uint32_t num, uint32_t dim, const uint32_t* segment_indexes, const uint32_t* segment_starts,

@@ -3,12 +3,13 @@
  *
  * Every entry point takes raw device pointers and plain sizes, launches on `stream` (a hipStream_t passed as
  * void*, NULL = default stream) and returns an int: 0 = success, > 0 = a hipError_t value, < 0 = one of the
- * GLIDE_ERR_* argument errors below.  No exceptions cross the boundary and the library keeps no global state.
+ * GLIDE_ERR_* argument errors below.  No exceptions cross the boundary and the library keeps no global state apart
+ * from the scratch array of glide_hip_partition_assign_fixed.
  * Each declaration cites the interface of the reference implementation (owlet-hub/GLIDE, paths relative to its
  * src/ directory) that it replaces.
  *
  * No entry point allocates device memory: those that need scratch take a caller-provided `workspace` whose
- * size a companion *_workspace_bytes() function reports.
+ * size a companion *_workspace_bytes() function reports (glide_hip_partition_assign_fixed brings its own).
  */
 #ifndef GLIDE_HIP_H
 #define GLIDE_HIP_H
@@ -86,6 +87,21 @@ int glide_hip_partition_assign(const float *data, uint32_t num, uint32_t dim, co
                                uint32_t centroid_num, float boundary_factor, int metric,
                                uint32_t *segment_indexes, uint32_t *segment_lengths, float *nearest_dists,
                                void *workspace, size_t workspace_bytes, void *stream);
+
+/* glide_hip_partition_assign without a workspace argument.  No counterpart in the reference: it is for callers that
+ * cannot allocate device memory (code under HIP graph capture, serving loops that route batches of new points or
+ * queries to their partitions, harnesses that forbid hipMalloc).  The scratch memory (centroid norms + per-tile
+ * histograms, 515 KB) is a file-scope device array of the library; each GPU the library runs on holds it until the
+ * process ends.  At most glide_hip_partition_assign_fixed_max_points() = 65536 points per call (GLIDE_ERR_UNSUPPORTED
+ * beyond); other limits, arguments and results as glide_hip_partition_assign.  The call allocates and frees nothing.
+ * The array's device address is looked up on the first call on each device (not a stream operation: make that
+ * first call outside a capture).  All calls on one GPU share the array: calls that overlap on one GPU (different
+ * streams or threads) race and must be serialised by the caller. */
+uint32_t glide_hip_partition_assign_fixed_max_points(void);
+int glide_hip_partition_assign_fixed(const float *data, uint32_t num, uint32_t dim, const float *centroids,
+                                     uint32_t centroid_num, float boundary_factor, int metric,
+                                     uint32_t *segment_indexes, uint32_t *segment_lengths, float *nearest_dists,
+                                     void *stream);
 
 /* Replaces reorder_kernel (partition_kernel.cuh:68-100; partition.cuh:118-157): row p goes to
  * segment_starts[segment] + slot, boundary copies to num + boundary slot; map[reorder id] = p.
