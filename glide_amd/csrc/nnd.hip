@@ -7,10 +7,13 @@
 // What is kept: fp16 rows with fp32 squared norms, <= 32 new + <= 32 old forward samples per node, reverse
 // samples capped at 32, a 64 x 64 distance tile per phase (new x new, new x old) computed on the matrix cores
 // with the norm-trick epilogue, and one offer per row / column (its nearest partner) per phase.
-// What is different: the kNN lists, flags and samples never leave HBM.  Offers are appended to a per-node inbox
-// (one atomic counter per node, no locks, no cross-workgroup read-after-write inside a kernel) and a merge kernel
-// folds each inbox into the node's sorted list with a wave-wide bitonic sort; sampling uses the new/old flag kept
-// in the list instead of a host-side Bloom filter.  All ids are partition-local.
+// What is different: the kNN lists, flags, Bloom filters and samples never leave HBM.  Offers and reverse samples go to
+// plain per-node inboxes (one atomic add reserves a slot, no locks); whatever arrives after an inbox is full goes to an
+// overflow table that keeps the smallest keys by atomic minimum with displacement, so the smallest 32 keys of a node --
+// all that the reference's 32-wide device list and its 32 reverse samples ever use -- are the same whatever the order
+// of arrival, and a build is reproducible.  A merge kernel then applies the reference's rules: of a node's offers the
+// best 32 count, those not yet listed enter the sub-list id % num_sub (each sub-list keeps its 32 nearest), those the
+// Bloom filter has not seen are the next "new" samples.  All ids are partition-local.
 #include "common.hpp"
 #include "host_util.hpp"
 #include <vector>
@@ -66,7 +69,7 @@ __device__ __forceinline__ uint32_t locate_uniform(const Segments& s, uint32_t n
 
 // ---- prepare: fp32 rows -> fp16 rows (stride dim_pad, zero padded) + squared norms of the fp32 input
 __global__ __launch_bounds__(256) void nnd_prepare_kernel(const float* data, uint32_t num, uint32_t dim, uint32_t dim_pad, _Float16* half_rows,
-                                                          float* norms) {
+                                                          float2* norms /* squared norm; offer threshold (none yet) */) {
     const int lane = lane_id();
     const uint32_t i = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (i >= num) return;
@@ -77,7 +80,7 @@ __global__ __launch_bounds__(256) void nnd_prepare_kernel(const float* data, uin
         half_rows[static_cast<size_t>(i) * dim_pad + d] = static_cast<_Float16>(v);
     }
     acc = wave_sum(acc);
-    if (lane == 0) norms[i] = acc;
+    if (lane == 0) norms[i] = make_float2(acc, __uint_as_float(kInvalid));
 }
 
 // ---- random initial lists.  The reference (init_random_graph :1003-1038) shuffles one sequence of len / num_sub values
@@ -111,7 +114,7 @@ __device__ __forceinline__ uint32_t permute(uint32_t x, uint32_t m, uint32_t key
     return x;
 }
 
-__global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, uint32_t num, uint32_t width,
+__global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t* list_ids, float* list_dists, uint32_t num, uint32_t width,
                                                        Segments segs, uint32_t seed) {
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
     const uint32_t node = idx / width, j = idx % width;
@@ -130,10 +133,11 @@ __global__ __launch_bounds__(256) void nnd_init_kernel(uint32_t* list_ids, float
     const uint32_t slot = (j % kSamples) * num_sub + sub;
     list_ids[static_cast<size_t>(node) * width + slot] = id;   // new (flag clear)
     list_dists[static_cast<size_t>(node) * width + slot] = FLT_MAX;
-    if (j == 0) inbox_counts[node] = 0;
 }
 
-// ---- sampling: first <= 32 new entries (marked old afterwards) and first <= 32 entries that were already old
+// ---- sampling: first <= 32 new entries (marked old afterwards) and first <= 32 entries that were already old.
+// The list is stored column-major over its sub-lists (slot = rank * num_sub + sub), so storage order is the order in
+// which the reference scans it (sample_graph :1052-1068).
 __global__ __launch_bounds__(256) void nnd_sample_kernel(uint32_t* list_ids, uint32_t num, uint32_t width, Segments segs, uint32_t* fwd_new,
                                                          uint32_t* fwd_old, uint32_t* counts /* num x 4: fwd_new, fwd_old, rev_new, rev_old */) {
     const int lane = lane_id();
@@ -167,9 +171,75 @@ __global__ __launch_bounds__(256) void nnd_sample_kernel(uint32_t* list_ids, uin
     }
 }
 
-// ---- reverse samples (add_rev_edges_kernel :490-507): list u appends itself to the reverse list of each sample
+// ---- where offers and reverse samples arrive ---------------------------------------------------------------------
+// Both go first to a plain inbox of the receiving node: one atomic add reserves a slot, a store fills it.  As long as
+// an inbox does not fill up it holds every arrival, so the set it ends up with does not depend on the order of arrival;
+// the consumer sorts it.  What arrives after an inbox is full goes to the node's overflow table, which keeps the
+// smallest keys whatever the order of arrival:
+//   a table is made of buckets of 16 words, 15 slots and, last, the bucket's bound = the smallest key it has turned
+//   away (all ones: none yet); a key's bucket and first slot are hashes of its id.  A slot keeps the smaller of the key
+//   it holds and the key that arrives (one atomic minimum); the larger one goes on to the next slot of the bucket.
+//   Slot contents only ever decrease, so a key that has passed all 15 slots is larger than everything the bucket holds
+//   in the end and is dropped: a bucket ends with the 15 smallest distinct keys sent to it.  A key that is not smaller
+//   than the bound need not look further, which keeps a node that receives thousands of keys cheap.
+// The consumers only use the smallest 32 keys of inbox + table (the reference's 32-wide device list; its 32 reverse
+// samples).  One of those could only be missing if 15 smaller keys shared its bucket, i.e. if 16 of a node's 32
+// smallest keys fell into one of 16 buckets: with the smallest 32 of every node intact, the result is the same on
+// every run.
+// A node that receives thousands of keys round after round would make every sender wait for atomics on the same few
+// cache lines.  Such a node therefore announces a threshold for the next round, read by the senders before anything
+// else (a plain read of a read-only array): when its inbox overflowed, the 64th best distinct offer (the 56th smallest
+// source) of this round -- like the smallest 32, the smallest 64 of inbox + table do not depend on the order of arrival.  Keys that are not below the threshold stay away.  As long as at least 32 keys below it
+// arrive, the smallest 32 are what they would have been without it; the threshold is kept while arrivals stay
+// plentiful and withdrawn when they do not.  Everything it depends on is itself independent of arrival order.
+constexpr uint32_t kBucketWords = 16, kBucketData = 15;
+constexpr uint32_t kInboxCap = 256;      // offers per node and round before the overflow table takes over
+constexpr uint32_t kRevCap = 64;         // reverse samples per node, kind and round before the overflow table takes over
+// Row strides of the inboxes and reverse lists, in entries.  Arrivals fill a row from its start, so with a power-of-two
+// stride (2 KB, 256 B) the busy front parts of all rows would sit on the same few memory channels.
+constexpr uint32_t kInboxStride = kInboxCap + 8, kRevStride = kRevCap + 8;
+constexpr uint32_t kOfferSlots = 256;    // overflow table per node: 16 buckets of (distance bits : candidate id) keys
+constexpr uint32_t kRevSlots = 256;      // overflow table per node and kind: 16 buckets of source ids
+constexpr unsigned long long kNoOffer = ~0ull;
+constexpr uint32_t kOfferThrRank = 64;    // the threshold of a node whose inbox overflowed: its 64th best distinct offer
+constexpr uint32_t kRevThrRank = 56;      // ... and of a node whose reverse list overflowed: its 56th smallest source
+constexpr uint32_t kOfferKeepArrivals = 64, kRevKeepArrivals = 40;   // fewer arrivals than this withdraw a threshold
+
+__device__ __forceinline__ uint32_t id_hash(uint32_t id) { return id * 0x9E3779B1u; }
+__device__ __forceinline__ uint32_t first_slot(uint32_t hash) { return __umulhi(hash * 0x85EBCA6Bu, kBucketData); }   // 0..14
+
+// One source id into a reverse overflow table (256 words).  The bound is read first: a table only comes into play for
+// nodes with many arrivals, and once its buckets are full nearly every further arrival ends here after one read.
+__device__ __forceinline__ void reverse_insert(uint32_t* table, uint32_t key) {
+    const uint32_t h = id_hash(key);
+    uint32_t* b = table + (h >> 28) * kBucketWords;
+    if (key >= __hip_atomic_load(&b[kBucketData], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return;
+    uint32_t pos = first_slot(h);
+    for (uint32_t probe = 0; probe < kBucketData; probe++) {
+        const uint32_t old = atomicMin(&b[pos], key);
+        if (old == kInvalid || old == key) return;   // settled in an empty slot, or already there
+        if (old > key) key = old;                    // the displaced key carries on
+        pos = pos + 1 == kBucketData ? 0 : pos + 1;
+    }
+    atomicMin(&b[kBucketData], key);   // larger than all 15 the bucket holds
+}
+
+// add_rev_edges_kernel (:490-507) for one sample: list `source` appends itself to the reverse list of `target` (both
+// row indices of the whole build; `source_local` is what is stored).  The reference keeps the first 32 arrivals; here
+// the 32 smallest sources count, which is what a sweep over the lists in order keeps.
+__device__ __forceinline__ void reverse_append(uint32_t* counts, uint32_t* rev_list, uint32_t* rev_tables, const uint32_t* rev_thr, size_t target,
+                                               uint32_t which, uint32_t source_local) {
+    if (source_local >= rev_thr[target * 2 + which]) return;   // the target has asked sources from here on to stay away
+    const uint32_t pos = atomicAdd(&counts[target * 4 + 2 + which], 1u);
+    if (pos < kRevCap)
+        rev_list[target * kRevStride + pos] = source_local;
+    else
+        reverse_insert(rev_tables + (target * 2 + which) * kRevSlots, source_local);
+}
+
+// ---- reverse samples as a stage of its own: every list enters the reverse tables of its samples
 __global__ __launch_bounds__(256) void nnd_reverse_kernel(const uint32_t* fwd_new, const uint32_t* fwd_old, uint32_t* counts, uint32_t* rev_new,
-                                                          uint32_t* rev_old, uint32_t num, Segments segs) {
+                                                          uint32_t* rev_old, uint32_t* rev_tables, const uint32_t* rev_thr, uint32_t num, Segments segs) {
     const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
     const uint32_t node = idx / 64, j = idx % 64;
     if (node >= num) return;
@@ -179,24 +249,25 @@ __global__ __launch_bounds__(256) void nnd_reverse_kernel(const uint32_t* fwd_ne
     const uint32_t which = j / kSamples, k = j % kSamples;   // 0: new, 1: old
     if (k >= counts[static_cast<size_t>(node) * 4 + which]) return;
     const uint32_t v = (which ? fwd_old : fwd_new)[static_cast<size_t>(node) * kSamples + k];
-    const uint32_t target = start + v;
-    const uint32_t pos = atomicAdd(&counts[static_cast<size_t>(target) * 4 + 2 + which], 1u);
-    if (pos < kSamples) (which ? rev_old : rev_new)[static_cast<size_t>(target) * kSamples + pos] = node - start;
+    reverse_append(counts, which ? rev_old : rev_new, rev_tables, rev_thr, static_cast<size_t>(start) + v, which, node - start);
 }
 
 // ---- local join ---------------------------------------------------------------------------------------------
 struct JoinArgs {
     const _Float16* half_rows;
-    const float* norms;
+    const float2* norms;           // num x (squared norm, offer threshold: offers whose distance bits are not below it stay away; all ones: none)
     const uint32_t* fwd_new;
     const uint32_t* fwd_old;
-    const uint32_t* rev_new;
+    const uint32_t* rev_new;       // num x kRevCap: the first reverse samples to arrive
     const uint32_t* rev_old;
-    uint32_t* counts;           // num x 4: forward new / old, reverse new / old
-    uint32_t* inbox_counts;
-    uint2* inbox;               // num x inbox_cap (dist bits, id)
-    unsigned long long* stats;  // [0] offers emitted, [1] offers dropped by a full inbox (nullable)
-    uint32_t num, dim_pad, width, inbox_cap;
+    uint32_t* rev_tables;          // num x 2 x kRevSlots: where later arrivals went; emptied by the join that reads them
+    uint32_t* rev_thr;             // num x 2: sources not below it stay away in the next scatter (all ones: none)
+    uint32_t* counts;              // num x 4: forward new / old, reverse new / old arrivals (restarted by the join)
+    uint32_t* inbox_counts;        // num: offers that have arrived
+    unsigned long long* inbox;     // num x kInboxCap
+    unsigned long long* offers;    // num x kOfferSlots overflow tables
+    unsigned long long* stats;     // striped: [1] offers turned away by a full bucket of an overflow table (nullable)
+    uint32_t num, dim_pad;
     Segments segs;
 };
 
@@ -212,6 +283,10 @@ struct JoinLds {
     uint32_t new_ids[kBi], old_ids[kBi];
     float new_norms[kBi], old_norms[kBi];
     uint32_t hash_new[128], hash_old[128];
+    __attribute__((aligned(16))) uint32_t rev_raw[2][kRevCap + kRevSlots];   // reverse samples as read: the list, then the overflow table
+    uint32_t rev_sel[2][kSamples];                                 // their 32 smallest entries, ascending
+    uint32_t rev_next_thr[2];
+    uint32_t new_thr[kBi], old_thr[kBi];                           // offer thresholds of the members
     uint32_t n_new, n_old;
 };
 
@@ -269,22 +344,26 @@ __device__ __forceinline__ void line_argmin(const float (*dist)[kDStride], uint3
     }
 }
 
-// Six workgroups per CU (80 registers per lane, 20 KB of LDS each): the join is bound by the latency of its
-// gather -> matrix -> arg-min -> offer chain, so residency matters more than registers; seven would spill.
+// Six workgroups per CU (20 KB of LDS each): the join is bound by the latency of its gather -> matrix -> arg-min ->
+// offer chain, so residency matters more than registers; seven would spill.
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     JoinLds& L = *reinterpret_cast<JoinLds*>(smem);
     const uint32_t node = blockIdx.x;
     if (node >= a.num) return;
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    const bool sampler = tid < 128;                  // wave 0 gathers the new members, wave 1 the old ones
+    const bool is_old = (wave & 1) != 0;             // waves 2 and 3 read the reverse tables (new, old)
+    const uint32_t k = tid & 63;                     // sampler: 0..31 forward sample, 32..63 reverse sample
 
     // sample ids are fetched before the counts are known (one memory round trip instead of two)
-    uint32_t my_id = kInvalid;
-    if (tid < 128) {
-        const bool is_old = tid >= 64;
-        const uint32_t k = tid & 63;
-        const uint32_t* src = k < kSamples ? (is_old ? a.fwd_old : a.fwd_new) : (is_old ? a.rev_old : a.rev_new);
-        my_id = src[static_cast<size_t>(node) * kSamples + (k & (kSamples - 1))];
+    uint32_t my_id = kInvalid, thr_in_force = kInvalid;
+    if (!sampler) {
+        my_id = (is_old ? a.rev_old : a.rev_new)[static_cast<size_t>(node) * kRevStride + lane];
+        thr_in_force = a.rev_thr[static_cast<size_t>(node) * 2 + is_old];
+    } else if (lane < static_cast<int>(kSamples))
+        my_id = (is_old ? a.fwd_old : a.fwd_new)[static_cast<size_t>(node) * kSamples + lane];
+    if (sampler) {
         L.hash_new[tid] = kInvalid;
         L.hash_old[tid] = kInvalid;
     }
@@ -292,28 +371,76 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     uint32_t seg_start, seg_len;
     const uint32_t seg = locate_uniform(a.segs, node, seg_start, seg_len);
     if (a.segs.state[seg] == kDone) return;
-    const uint32_t c_fn = c4.x, c_fo = c4.y;
-    const uint32_t c_rn = c4.z < kSamples ? c4.z : kSamples, c_ro = c4.w < kSamples ? c4.w : kSamples;
     // The counts must have arrived in every thread before thread 0 restarts them below; the barrier itself waits
     // for LDS traffic only, so the registers are consumed here.
-    asm volatile("" ::"v"(c4.x), "v"(c4.y), "v"(c4.z), "v"(c4.w));
-    __syncthreads();
+    asm volatile("" ::"v"(c4.x), "v"(c4.y), "v"(c4.z), "v"(c4.w), "v"(my_id), "v"(thr_in_force));
+    if (!sampler) {
+        // Reverse samples: the 32 smallest sources that arrived, in ascending order.  Up to 64 arrivals sit in the list;
+        // a node that received more also has an overflow table, which is read and emptied (bounds included) here.
+        const uint32_t arrived = is_old ? c4.w : c4.z;
+        if (static_cast<uint32_t>(lane) >= arrived) my_id = kInvalid;
+        uint4 more = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
+        const bool overflowed = arrived > kRevCap;
+        if (overflowed) {
+            uint4* const quad = reinterpret_cast<uint4*>(a.rev_tables + (static_cast<size_t>(node) * 2 + is_old) * kRevSlots) + lane;
+            more = *quad;
+            if ((more.x & more.y & more.z & more.w) != kInvalid) *quad = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
+            if ((lane & 3) == 3) more.w = kInvalid;   // word 15 of a bucket is its bound
+            *reinterpret_cast<uint4*>(&L.rev_raw[is_old][kRevCap + 4 * lane]) = more;
+        }
+        L.rev_raw[is_old][lane] = my_id;
+        if (lane < static_cast<int>(kSamples)) L.rev_sel[is_old][lane] = kInvalid;
+        if (lane == 0) L.rev_next_thr[is_old] = kInvalid;
+        __builtin_amdgcn_wave_barrier();
+        if (!overflowed) {
+            uint32_t rank = 0;
+            // all 64 slots in four steps of four independent reads (slots beyond the arrivals hold 0xffffffff and count for nothing)
+#pragma unroll
+            for (uint32_t j = 0; j < kRevCap; j += 4) {
+                const uint4 q = *reinterpret_cast<const uint4*>(&L.rev_raw[is_old][j]);
+                rank += (q.x < my_id) + (q.y < my_id) + (q.z < my_id) + (q.w < my_id);
+            }
+            if (my_id != kInvalid && rank < kSamples) L.rev_sel[is_old][rank] = my_id;
+        } else {
+            const uint32_t mine[5] = {my_id, more.x, more.y, more.z, more.w};
+            uint32_t rank[5] = {0, 0, 0, 0, 0};
+            for (uint32_t j = 0; j < kRevCap + kRevSlots; j += 4) {
+                const uint4 q = *reinterpret_cast<const uint4*>(&L.rev_raw[is_old][j]);
+#pragma unroll
+                for (int m = 0; m < 5; m++) rank[m] += (q.x < mine[m]) + (q.y < mine[m]) + (q.z < mine[m]) + (q.w < mine[m]);
+            }
+#pragma unroll
+            for (int m = 0; m < 5; m++) {
+                if (mine[m] != kInvalid && rank[m] < kSamples) L.rev_sel[is_old][rank[m]] = mine[m];
+                // after an overflow the 56th smallest source becomes the threshold of the scatter that follows: some 55
+                // sources are then expected, few enough to stay in the list, enough for the smallest 32 to be complete
+                if (mine[m] != kInvalid && rank[m] == kRevThrRank - 1) L.rev_next_thr[is_old] = mine[m];
+            }
+        }
+        // a threshold that is in force stays while at least 40 sources still arrive
+        __builtin_amdgcn_wave_barrier();
+        if (lane == 0) {
+            const uint32_t next = overflowed ? L.rev_next_thr[is_old] : (arrived >= kRevKeepArrivals ? thr_in_force : kInvalid);
+            if (next != thr_in_force) a.rev_thr[static_cast<size_t>(node) * 2 + is_old] = next;
+        }
+    }
+    __syncthreads();   // the hash sets are clear, the reverse samples chosen, the counts read by everyone
     // this list's reverse samples are consumed here and now: the counts restart for the scatter that follows the join
     if (tid == 0) *reinterpret_cast<uint2*>(a.counts + static_cast<size_t>(node) * 4 + 2) = make_uint2(0u, 0u);
-    if (c_fn + c_rn == 0) return;
-    // forward then reverse samples, duplicates removed with an LDS hash set (reference: sort + binary search, :625-666)
-    if (tid < 128) {
-        const bool is_old = tid >= 64;
-        const uint32_t k = tid & 63;
-        const uint32_t cf = is_old ? c_fo : c_fn, cr = is_old ? c_ro : c_rn;
-        const bool present = k < kSamples ? k < cf : (k - kSamples) < cr;
+    // Forward then reverse samples, duplicates removed with an LDS hash set (reference: sort + binary search, :625-666).
+    // Forward samples enter the set first, so a point that is in both keeps its forward position.
+    if (sampler) {
+        uint32_t* set = is_old ? L.hash_old : L.hash_new;
+        if (k >= kSamples) my_id = L.rev_sel[is_old][k - kSamples];
+        const bool present = k < kSamples ? k < (is_old ? c4.y : c4.x) : true;
         const uint32_t id = present ? my_id : kInvalid;
-        const bool keep = id != kInvalid && id < seg_len && lds_set_insert(is_old ? L.hash_old : L.hash_new, id);
-        const uint64_t m = ballot(keep);   // wave 0 = new, wave 1 = old; forward entries keep the lower ranks
-        if (keep) {
-            const uint32_t pos = prefix_count(m);
-            (is_old ? L.old_ids : L.new_ids)[pos] = id;
-        }
+        const bool usable = id != kInvalid && id < seg_len;
+        bool keep = false;
+        if (k < kSamples) keep = usable && lds_set_insert(set, id);
+        __builtin_amdgcn_wave_barrier();
+        if (k >= kSamples) keep = usable && lds_set_insert(set, id);
+        const uint64_t m = ballot(keep);
+        if (keep) (is_old ? L.old_ids : L.new_ids)[prefix_count(m)] = id;
         if (lane == 0) (is_old ? L.n_old : L.n_new) = __popcll(m);
     }
     __syncthreads();
@@ -332,20 +459,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
 
     // Chunks of kJoinChunk dims go global -> registers -> LDS: 8 lanes x 16 B per row and chunk, 32 rows per pass (new
     // rows, then old rows).  The loads of chunk k+1 are issued before the matrix instructions of chunk k.  Short chunks
-    // keep the workgroup at 20 KB of LDS, so seven of them share a CU instead of four.
+    // keep the workgroup at 20 KB of LDS, so six of them share a CU instead of four.
     float4 pre[4];
     auto prefetch = [&](uint32_t k0) {
 #pragma unroll
         for (int pass = 0; pass < 4; pass++) {
             const uint32_t r = pass * 32 + (tid >> 3), q = tid & 7;
-            const bool is_old = r >= 64;
+            const bool old_row = r >= 64;
             const uint32_t rr = r & 63;
             const uint32_t d0 = k0 + q * 8;
             pre[pass] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (rr < (is_old ? n_old : n_new)) {
-                const uint32_t id = (is_old ? L.old_ids : L.new_ids)[rr];
+            if (rr < (old_row ? n_old : n_new)) {
+                const uint32_t id = (old_row ? L.old_ids : L.new_ids)[rr];
                 if (d0 < a.dim_pad) pre[pass] = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
-                if (k0 == 0 && q == 0) (is_old ? L.old_norms : L.new_norms)[rr] = a.norms[seg_start + id];   // same round trip as the row
+                if (k0 == 0 && q == 0) {   // same round trip as the row
+                    const float2 nt = a.norms[seg_start + id];
+                    (old_row ? L.old_norms : L.new_norms)[rr] = nt.x;
+                    (old_row ? L.old_thr : L.new_thr)[rr] = __float_as_uint(nt.y);
+                }
             }
         }
     };
@@ -375,18 +506,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         L.dist[i][j] = d;
     }
     __syncthreads();
-    // offers are collected first and sent at the end, so their atomics overlap instead of costing a round trip each
-    uint32_t off_target[3] = {kInvalid, kInvalid, kInvalid}, off_cand[3] = {kInvalid, kInvalid, kInvalid};
-    float off_dist[3] = {FLT_MAX, FLT_MAX, FLT_MAX};
+    // Every offer reserves a slot of its target's inbox; the atomic of phase 1 is in flight while phase 2 computes.
+    unsigned long long key[3] = {kNoOffer, kNoOffer, kNoOffer};
+    size_t row[3] = {0, 0, 0};
+    uint32_t slot[3] = {0, 0, 0};
+    bool live[3] = {false, false, false};
+    auto send = [&](int o, uint32_t target, uint32_t cand, float dist, uint32_t thr) {
+        if (cand == kInvalid || cand == target || cand >= seg_len || !(dist < FLT_MAX)) return;
+        if (__float_as_uint(dist) >= thr) return;   // the target has asked offers from this distance on to stay away
+        key[o] = (static_cast<unsigned long long>(__float_as_uint(dist)) << 32) | cand;
+        row[o] = static_cast<size_t>(seg_start) + target;
+        live[o] = true;
+        slot[o] = atomicAdd(&a.inbox_counts[row[o]], 1u);
+    };
     {
         float best;
         uint32_t bj;
         line_argmin<true>(L.dist, line, part, best, bj);
-        if (part == 0 && line < n_new && bj != kInvalid) {
-            off_target[0] = L.new_ids[line];
-            off_cand[0] = L.new_ids[bj];
-            off_dist[0] = best;
-        }
+        if (part == 0 && line < n_new && bj != kInvalid) send(0, L.new_ids[line], L.new_ids[bj], best, L.new_thr[line]);
     }
     if (n_old != 0) {
         // ---- phase 2: new x old (rows: new, columns: old)
@@ -405,41 +542,85 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
             uint32_t bj;
             const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
             line_argmin<true>(L.dist, line, part, best, bj);
-            if (part == 0 && line < n_new && bj != kInvalid) {
-                off_target[1] = me;
-                off_cand[1] = L.old_ids[bj];
-                off_dist[1] = best;
-            }
+            if (part == 0 && line < n_new && bj != kInvalid) send(1, me, L.old_ids[bj], best, L.new_thr[line]);
         }
         {
             float best;
             uint32_t bi;
             const uint32_t me = line < n_old ? L.old_ids[line] : kInvalid;
             line_argmin<false>(L.dist, line, part, best, bi);
-            if (part == 0 && line < n_old && bi != kInvalid) {
-                off_target[2] = me;
-                off_cand[2] = L.new_ids[bi];
-                off_dist[2] = best;
-            }
+            if (part == 0 && line < n_old && bi != kInvalid) send(2, me, L.new_ids[bi], best, L.old_thr[line]);
         }
     }
-    uint32_t pos[3];
+    bool any = false;
 #pragma unroll
-    for (int k = 0; k < 3; k++) {
-        const bool ok = off_cand[k] != kInvalid && off_cand[k] != off_target[k] && off_cand[k] < seg_len && off_dist[k] < FLT_MAX;
-        if (!ok) off_target[k] = kInvalid;
-        pos[k] = ok ? atomicAdd(&a.inbox_counts[seg_start + off_target[k]], 1u) : kInvalid;
+    for (int o = 0; o < 3; o++) {
+        if (live[o] && slot[o] < kInboxCap) {
+            a.inbox[row[o] * kInboxStride + slot[o]] = key[o];
+            live[o] = false;
+        }
+        any |= live[o];
     }
+    if (any) {
+        // The inbox of the target is full: the overflow table takes the offer (the up to three chains of a thread side by side).
+        unsigned long long* bucket[3];
+        unsigned long long seen[3], bound[3];
+        uint32_t at[3], dropped = 0;
 #pragma unroll
-    for (int k = 0; k < 3; k++) {
-        if (off_target[k] != kInvalid && pos[k] < a.inbox_cap)
-            a.inbox[static_cast<size_t>(seg_start + off_target[k]) * a.inbox_cap + pos[k]] = make_uint2(__float_as_uint(off_dist[k]), off_cand[k]);
+        for (int o = 0; o < 3; o++) {
+            const uint32_t h = id_hash(static_cast<uint32_t>(key[o]));
+            bucket[o] = a.offers + row[o] * kOfferSlots + (h >> 28) * kBucketWords;
+            at[o] = first_slot(h);
+            // the bound first: once the buckets of a node that receives thousands of offers are full, nearly every
+            // further offer ends here after one read
+            bound[o] = live[o] ? __hip_atomic_load(&bucket[o][kBucketData], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : kNoOffer;
+        }
+#pragma unroll
+        for (int o = 0; o < 3; o++) {
+            if (live[o] && key[o] >= bound[o]) {   // the bucket has already turned a smaller key away
+                live[o] = false;
+                dropped++;
+            }
+            seen[o] = live[o] ? atomicMin(&bucket[o][at[o]], key[o]) : kNoOffer;
+        }
+#pragma unroll
+        for (int o = 0; o < 3; o++) {
+            if (live[o]) {
+                if (seen[o] == kNoOffer || seen[o] == key[o]) live[o] = false;     // settled, or a copy was there
+                else if (seen[o] > key[o]) key[o] = seen[o];                       // the displaced key carries on
+            }
+        }
+        for (uint32_t probe = 1; probe < kBucketData; probe++) {
+            if (!(live[0] || live[1] || live[2])) break;
+#pragma unroll
+            for (int o = 0; o < 3; o++) {
+                if (live[o]) {
+                    at[o] = at[o] + 1 == kBucketData ? 0 : at[o] + 1;
+                    seen[o] = atomicMin(&bucket[o][at[o]], key[o]);
+                }
+            }
+#pragma unroll
+            for (int o = 0; o < 3; o++) {
+                if (live[o]) {
+                    if (seen[o] == kNoOffer || seen[o] == key[o]) live[o] = false;
+                    else if (seen[o] > key[o]) key[o] = seen[o];
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < 3; o++) {
+            if (live[o]) {   // it has met 15 smaller keys: the bucket is full of better offers
+                atomicMin(&bucket[o][kBucketData], key[o]);
+                dropped++;
+            }
+        }
+        if (dropped && a.stats) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(dropped));
     }
 }
 
-// ---- merge: list (width) + inbox (<= cap) -> sorted, de-duplicated list of `width`; one wavefront per node
-// key = dist bits : id (31 bits) : source (0 = already in the list, 1 = offer); payload = old flag
-template <int M>
+// ---- merge ------------------------------------------------------------------------------------------------------
+// Register bitonic network over M 64-bit keys (element e = (M/64) * lane + r), with an optional 32-bit payload.
+template <int M, bool VAL>
 struct Net64 {
     static constexpr int NR = M / 64;
     template <int LM>
@@ -457,12 +638,12 @@ struct Net64 {
                     const bool asc = (K >= M) ? true : ((e & K) == 0);
                     if ((k[r] > k[r | J]) == asc) {
                         const unsigned long long tk = k[r]; k[r] = k[r | J]; k[r | J] = tk;
-                        const uint32_t tv = v[r]; v[r] = v[r | J]; v[r | J] = tv;
+                        if constexpr (VAL) { const uint32_t tv = v[r]; v[r] = v[r | J]; v[r | J] = tv; }
                     }
                 }
             }
         } else {
-            // Two entries with equal keys are copies of one offer (same distance, id, source and flag), so exchanging
+            // Two entries with equal keys are copies of one entry (same distance, id, source and flag), so exchanging
             // them or not gives the same sequence: one compare decides, and the lanes that keep the larger key take the
             // partner's entry exactly where the others would not (the complement of the compare mask).
             constexpr int LM = J / NR;
@@ -475,13 +656,12 @@ struct Net64 {
                     if (((l & LM) == 0) == asc) keep_min |= 1ull << l;
                 }
                 const unsigned long long ok = xor_lane<LM>(k[r]);
-                const uint32_t ov = lane_xor<LM>(v[r]);
                 const uint64_t less = __builtin_amdgcn_ballot_w64(ok < k[r]);
                 const uint64_t take = less ^ ~keep_min;
                 const uint32_t lo = select_by_mask(static_cast<uint32_t>(k[r]), static_cast<uint32_t>(ok), take);
                 const uint32_t hi = select_by_mask(static_cast<uint32_t>(k[r] >> 32), static_cast<uint32_t>(ok >> 32), take);
                 k[r] = (static_cast<unsigned long long>(hi) << 32) | lo;
-                v[r] = select_by_mask(v[r], ov, take);
+                if constexpr (VAL) v[r] = select_by_mask(v[r], lane_xor<LM>(v[r]), take);
             }
         }
     }
@@ -501,11 +681,19 @@ struct Net64 {
 // Bloom filter of ids already used as "new" samples (reference BloomFilter :203-276: 512-bit sets, 3 hashes)
 __device__ __forceinline__ uint32_t bloom_h0(uint32_t v) { v *= 1103515245u; v += 12345u; v ^= v << 13; v ^= v >> 17; v ^= v << 5; return v; }
 __device__ __forceinline__ uint32_t bloom_h1(uint32_t v) { v *= 1664525u; v += 1013904223u; v ^= v << 13; v ^= v >> 17; v ^= v << 5; return v; }
+__device__ __forceinline__ void bloom_bits(uint32_t id, uint32_t bloom_sets, uint32_t (&b)[3]) {
+    const uint32_t base = (id % bloom_sets) * 512;
+    uint32_t h = bloom_h0(id);
+    b[0] = base + h % 512;
+    h += bloom_h1(id);
+    b[1] = base + h % 512;
+    h += bloom_h1(id);
+    b[2] = base + h % 512;
+}
 
 // Prefix sum over the 64 lanes without LDS traffic: four shifted adds inside each row of 16 lanes, then lane 15 of a row
 // is added to the next row (rows 1 and 3) and lane 31 to the upper half (rows 2 and 3).  Lanes a step does not feed add 0.
-__device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane, uint32_t& total) {
-    (void) lane;
+__device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, uint32_t& total) {
     int x = static_cast<int>(value);
     x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, true);   // row_shr:1
     x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, true);   // row_shr:2
@@ -517,31 +705,166 @@ __device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, int lane
     return static_cast<uint32_t>(x) - value;
 }
 
-// Merge + resample, one wavefront per node.  The reference keeps, per node and round, a 32-wide sorted "device" list of
-// the offers (insert_to_global_graph :509-579), merges it into the host list (update_graph :1106-1126) and draws the
-// samples of the next join from both (sample_graph_new :973-1001, sample_segment_graph :1073-1104).  Here:
-//   old samples = the first <= 32 entries of the incoming list that are flagged old (the reference samples them before
-//                 this round's results are merged);
-//   the list and this round's offers are sorted together by (distance, id); of the distinct offered ids only the
-//   best 32 count (the rest are dropped, as the 32-wide device list drops them); those not yet in the list enter it;
-//   new samples = those of the best 32 that the Bloom filter has not seen; the ones entering the list are flagged old.
-// add_rev_edges_kernel (:490-507) for one sample: list `node` appends itself to the reverse list of sample `id`
-__device__ __forceinline__ void reverse_append(uint32_t* counts, uint32_t* rev, uint32_t seg_start, uint32_t id, uint32_t which, uint32_t node) {
-    const uint32_t target = seg_start + id;
-    const uint32_t pos = atomicAdd(&counts[static_cast<size_t>(target) * 4 + which], 1u);
-    if (pos < kSamples) rev[static_cast<size_t>(target) * kSamples + pos] = node - seg_start;
+struct MergeArgs {
+    uint32_t* list_ids;
+    float* list_dists;
+    uint32_t* inbox_counts;
+    const unsigned long long* inbox;
+    unsigned long long* offers;  // overflow tables
+    uint32_t* bloom;
+    uint32_t* fwd_new;
+    uint32_t* fwd_old;
+    uint32_t* counts;            // num x 4
+    unsigned long long* stats;   // striped: [0] offers received by the merge steps (nullable)
+    Segments segs;
+    uint32_t* rev_new;           // reverse lists of the next join (null: the scatter is a stage of its own)
+    uint32_t* rev_old;
+    uint32_t* rev_tables;
+    const uint32_t* rev_thr;
+    float2* norms;               // .y: the node's offer threshold
+    uint32_t num, width, num_sub, bloom_sets;
+};
+
+constexpr uint32_t kKnownBits = 9;   // 512-slot id set per wavefront: lists of up to 192 entries + 32 offers
+struct MergeLds {
+    unsigned long long keys[4][kInboxCap];   // the node's offers as they arrived
+    unsigned long long best[4][2 * kOfferThrRank];   // the best 32 distinct ones (64 + 64 while inbox and overflow table are combined)
+    unsigned long long enter[4][kSamples];      // those that enter the list, as keys of the second sort
+    uint32_t known[4][1u << kKnownBits];
+    uint32_t filter[4][128];
+    uint32_t flags[4][kSamples];
+};
+
+// The smallest N_OUT distinct keys of keys[0 .. held), ascending, to best[0 ..); returns how many there are (at most N_OUT).
+// Copies of one offer (the same pair met in several lists) are adjacent after the sort.  The network is sized by what
+// the node holds.  `best` may be part of `keys`: everything is read before anything is written.
+// N_OUT = 32, or 64 where the 64th is needed as well.
+template <int M1, uint32_t N_OUT = kSamples>
+__device__ __forceinline__ uint32_t best_offers(const unsigned long long* keys, uint32_t held, unsigned long long* best, int lane) {
+    constexpr int NR = M1 / 64;
+    unsigned long long k[NR];
+    uint32_t none[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        k[r] = e < held ? keys[e] : kNoOffer;
+    }
+    Net64<M1, false>::sort(k, none, lane);
+    const unsigned long long last_of_prev =
+        (static_cast<unsigned long long>(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[NR - 1] >> 32), 0x138, 0xf, 0xf, false))) << 32) |
+        static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[NR - 1]), 0x138, 0xf, 0xf, false));   // wave_shr:1
+    bool distinct[NR];
+    uint32_t count = 0, total;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const unsigned long long prev = r == 0 ? last_of_prev : k[r - 1];
+        distinct[r] = k[r] != kNoOffer && ((r == 0 && lane == 0) || prev != k[r]);
+        count += distinct[r];
+    }
+    uint32_t rank = wave_exclusive_scan(count, total);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        if (distinct[r]) {
+            if (rank < N_OUT) best[rank] = k[r];
+            rank++;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    return total < N_OUT ? total : N_OUT;
 }
 
-// The sort network is sized by what the node holds this round (list + offers received): the keys are distinct up to
-// identical copies, so every size gives the same sorted sequence, and most nodes need far less than the largest one.
-template <int M>
-__device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t width,
-                                           uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new, uint32_t* fwd_old,
-                                           uint32_t* counts, unsigned long long* stats, Segments segs, uint32_t node, uint32_t seg, uint32_t raw,
-                                           uint32_t* filter, int lane, uint32_t seg_start, uint32_t* rev_new, uint32_t* rev_old) {
-    constexpr int NR = M / 64;
-    const uint32_t bloom_words = bloom_sets * 16;
-    const uint32_t n_in = raw < inbox_cap ? raw : inbox_cap;
+__device__ __forceinline__ uint32_t best_offers_sized(const unsigned long long* keys, uint32_t held, unsigned long long* best, int lane) {
+    if (held > 128) return best_offers<256>(keys, held, best, lane);
+    if (held > 64) return best_offers<128>(keys, held, best, lane);
+    if (held > 0) return best_offers<64>(keys, held, best, lane);
+    return 0;
+}
+
+// Merge + resample, one wavefront per node.  The reference keeps, per node and round, a 32-wide sorted "device" list of
+// the offers (insert_to_global_graph :509-579), merges it into the host list (update_graph :1106-1126: an id goes to
+// sub-list id % num_sub, each a sorted list of 32 that rejects ids it already holds) and draws the samples of the next
+// join from both (sample_graph_new :973-1001, sample_segment_graph :1073-1104).  Here:
+//   old samples = the first <= 32 entries of the incoming list that are flagged old, in storage order (the reference
+//                 samples them before this round's results are merged);
+//   the node's offers are sorted by (distance, id) and the best 32 count; those whose id the list does not hold yet are
+//   sorted together with the list, and every sub-list keeps its 32 nearest;
+//   new samples = those of the best 32 that the Bloom filter has not seen; the ones entering the list are flagged old.
+// M2 = size of the second network >= width + 32.
+template <int M2>
+__global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
+    __shared__ MergeLds L;
+    constexpr int NR = M2 / 64;
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const uint32_t node = blockIdx.x * 4 + wave;
+    if (node >= a.num) return;
+    uint32_t seg_start, seg_len;
+    const uint32_t seg = locate_uniform(a.segs, node, seg_start, seg_len);
+    if (a.segs.state[seg] == kDone) return;
+    const uint32_t width = a.width, num_sub = a.num_sub;
+    unsigned long long* keys = L.keys[wave];
+    unsigned long long* best = L.best[wave];
+    unsigned long long* enter = L.enter[wave];
+    uint32_t* known = L.known[wave];
+    uint32_t* filter = L.filter[wave];
+    uint32_t* flags = L.flags[wave];
+    const uint32_t bloom_words = a.bloom_sets * 16;
+    const uint32_t arrived = a.inbox_counts[node];
+    for (uint32_t w = lane; w < bloom_words; w += 64) filter[w] = a.bloom[static_cast<size_t>(node) * bloom_words + w];
+    for (uint32_t i = lane; i < (1u << kKnownBits); i += 64) known[i] = kInvalid;
+
+    // ---- this round's offers: the inbox, four slots per lane
+    const uint32_t held = arrived < kInboxCap ? arrived : kInboxCap;
+    if (4u * lane < held) {
+        const unsigned long long* src = a.inbox + static_cast<size_t>(node) * kInboxStride + 4 * lane;
+        const uint4 lo = *reinterpret_cast<const uint4*>(src), hi = *reinterpret_cast<const uint4*>(src + 2);
+        *reinterpret_cast<uint4*>(keys + 4 * lane) = lo;
+        *reinterpret_cast<uint4*>(keys + 4 * lane + 2) = hi;
+    }
+    __builtin_amdgcn_wave_barrier();
+    uint32_t n_best;
+    uint32_t next_thr;
+    const uint32_t in_force = __float_as_uint(a.norms[node].y);
+    if (arrived <= kInboxCap) {
+        n_best = best_offers_sized(keys, held, best, lane);
+        // a threshold that is in force stays while the node still receives plenty of offers and its best 32 are complete
+        next_thr = arrived >= kOfferKeepArrivals && n_best == kSamples ? in_force : kInvalid;
+    } else {
+        // The inbox filled up and later offers went to the overflow table: the round's best distinct offers are those
+        // of the inbox's best 64 and the table's best 64.  The table is emptied (bounds included) where something was found.
+        const uint32_t n_inbox = best_offers<256, kOfferThrRank>(keys, held, best, lane);
+        unsigned long long* row = a.offers + static_cast<size_t>(node) * kOfferSlots;
+        const uint4 lo = *reinterpret_cast<const uint4*>(row + 4 * lane), hi = *reinterpret_cast<const uint4*>(row + 4 * lane + 2);
+        unsigned long long o[4] = {(static_cast<unsigned long long>(lo.y) << 32) | lo.x, (static_cast<unsigned long long>(lo.w) << 32) | lo.z,
+                                   (static_cast<unsigned long long>(hi.y) << 32) | hi.x, (static_cast<unsigned long long>(hi.w) << 32) | hi.z};
+        if ((o[0] & o[1] & o[2] & o[3]) != kNoOffer) {
+            const uint4 empty = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
+            *reinterpret_cast<uint4*>(row + 4 * lane) = empty;
+            *reinterpret_cast<uint4*>(row + 4 * lane + 2) = empty;
+        }
+        if ((lane & 3) == 3) o[3] = kNoOffer;   // word 15 of a bucket is its bound, not an offer
+        uint32_t mine = 0, in_table;
+#pragma unroll
+        for (int j = 0; j < 4; j++) mine += o[j] != kNoOffer;
+        uint32_t at = wave_exclusive_scan(mine, in_table);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (o[j] != kNoOffer) keys[at++] = o[j];
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t n_table = best_offers<256, kOfferThrRank>(keys, in_table, best + kOfferThrRank, lane);
+        // best[0 .. n_inbox) and best[64 .. 64 + n_table): close the gap, then once more through a 128-key network.
+        // The distance of the 64th best distinct offer of the round becomes the node's threshold for the next join (none if it has fewer).
+        if (static_cast<uint32_t>(lane) < n_table) keys[n_inbox + lane] = best[kOfferThrRank + lane];
+        if (static_cast<uint32_t>(lane) < n_inbox) keys[lane] = best[lane];
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t n_union = best_offers<128, kOfferThrRank>(keys, n_inbox + n_table, best, lane);
+        n_best = n_union < kSamples ? n_union : kSamples;
+        next_thr = n_union == kOfferThrRank ? static_cast<uint32_t>(best[kOfferThrRank - 1] >> 32) : kInvalid;
+    }
+    if (lane == 0 && next_thr != in_force) a.norms[node].y = __uint_as_float(next_thr);
+
+    // ---- the incoming list, in storage order; its ids go into the wavefront's id set
     unsigned long long k[NR];
     uint32_t v[NR];
     uint32_t old_count = 0;
@@ -551,170 +874,137 @@ __device__ __forceinline__ void merge_node(uint32_t* list_ids, float* list_dists
         k[r] = ~0ull;
         v[r] = 0;
         if (e < width) {
-            const uint32_t id = list_ids[static_cast<size_t>(node) * width + e];
-            const float d = list_dists[static_cast<size_t>(node) * width + e];
+            const uint32_t id = a.list_ids[static_cast<size_t>(node) * width + e];
+            const float d = a.list_dists[static_cast<size_t>(node) * width + e];
             if (id != kInvalid) {
                 k[r] = (static_cast<unsigned long long>(__float_as_uint(d)) << 32) | (static_cast<unsigned long long>(id & ~kOld) << 1);
                 v[r] = id & kOld;
                 old_count += (id & kOld) != 0;
+                hash_insert(known, kKnownBits, id & ~kOld);
             }
-        } else if (e - width < n_in) {
-            const uint2 o = inbox[static_cast<size_t>(node) * inbox_cap + (e - width)];
-            k[r] = (static_cast<unsigned long long>(o.x) << 32) | (static_cast<unsigned long long>(o.y) << 1) | 1ull;
-            v[r] = 0;   // offers enter as new
         }
     }
-    // old samples from the incoming list (element order = list order)
+    // old samples from the incoming list (element order = storage order = the reference's scan order)
     uint32_t total_old;
     {
-        uint32_t rank = wave_exclusive_scan(old_count, lane, total_old);
+        uint32_t rank = wave_exclusive_scan(old_count, total_old);
 #pragma unroll
         for (int r = 0; r < NR; r++) {
-            if (k[r] != ~0ull && !(k[r] & 1ull) && (v[r] & kOld)) {
+            if (k[r] != ~0ull && (v[r] & kOld)) {
                 if (rank < kSamples) {
                     const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
-                    fwd_old[static_cast<size_t>(node) * kSamples + rank] = id;
-                    if (rev_old) reverse_append(counts, rev_old, seg_start, id, 3, node);
+                    a.fwd_old[static_cast<size_t>(node) * kSamples + rank] = id;
+                    if (a.rev_old) reverse_append(a.counts, a.rev_old, a.rev_tables, a.rev_thr, static_cast<size_t>(seg_start) + id, 1, node - seg_start);
                 }
                 rank++;
             }
         }
     }
-    Net64<M>::sort(k, v, lane);
-    // Equal id => equal distance => adjacent after the sort, the list's own copy first.  An id's first offered copy
-    // represents the offer; it is "known" when the list already holds the id.
-    bool from_list[NR], first_offer[NR], known[NR];
-    uint32_t offer_count = 0;
-    // the previous lane's last key (wave_shr:1; lane 0 has no predecessor and is handled as the head below)
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- the best 32 offers, one per lane: new samples, and which of them enter the list
+    uint32_t total_new = 0;
+    {
+        const bool mine = static_cast<uint32_t>(lane) < n_best;
+        const unsigned long long key = mine ? best[lane] : kNoOffer;
+        const uint32_t id = static_cast<uint32_t>(key);
+        const bool take = mine && id < seg_len;
+        bool fresh = false;
+        uint32_t b[3];
+        if (take) {
+            bloom_bits(id, a.bloom_sets, b);
+            fresh = ((filter[b[0] >> 5] >> (b[0] & 31)) & (filter[b[1] >> 5] >> (b[1] & 31)) & (filter[b[2] >> 5] >> (b[2] & 31)) & 1u) == 0;
+        }
+        // an id the list holds (whatever its distance there) is rejected, as insert_to_ordered_list :916-943 does
+        const bool enters = take && hash_insert(known, kKnownBits, id) != 0;
+        const uint64_t fm = ballot(fresh);
+        total_new = __popcll(fm);
+        __builtin_amdgcn_wave_barrier();   // every lane has tested the filter before bits are added
+        if (fresh) {   // at most 32 of them: all become samples
+            a.fwd_new[static_cast<size_t>(node) * kSamples + prefix_count(fm)] = id;
+            if (a.rev_new) reverse_append(a.counts, a.rev_new, a.rev_tables, a.rev_thr, static_cast<size_t>(seg_start) + id, 0, node - seg_start);
+            atomicOr(&filter[b[0] >> 5], 1u << (b[0] & 31));
+            atomicOr(&filter[b[1] >> 5], 1u << (b[1] & 31));
+            atomicOr(&filter[b[2] >> 5], 1u << (b[2] & 31));
+        }
+        if (lane < static_cast<int>(kSamples)) {
+            enter[lane] = enters ? ((key >> 32) << 32) | (static_cast<unsigned long long>(id) << 1) | 1ull : ~0ull;
+            flags[lane] = fresh ? kOld : 0u;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        if (e >= width && e < width + kSamples) {
+            k[r] = enter[e - width];
+            v[r] = flags[e - width];
+        }
+    }
+    Net64<M2, true>::sort(k, v, lane);
+
+    // ---- every sub-list keeps its 32 nearest: rank of an entry among those of its sub-list, in sorted order
     const unsigned long long last_of_prev =
         (static_cast<unsigned long long>(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[NR - 1] >> 32), 0x138, 0xf, 0xf, false))) << 32) |
-        static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[NR - 1]), 0x138, 0xf, 0xf, false));
+        static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[NR - 1]), 0x138, 0xf, 0xf, false));   // wave_shr:1
+    bool valid[NR];
+    uint32_t sub[NR], slot[NR];
 #pragma unroll
     for (int r = 0; r < NR; r++) {
         const unsigned long long prev = r == 0 ? last_of_prev : k[r - 1];
         const bool head = (r == 0 && lane == 0);
-        const bool valid = k[r] != ~0ull;
-        const bool same_id = !head && (prev >> 1) == (k[r] >> 1);
-        from_list[r] = valid && !(k[r] & 1ull) && !same_id;   // a repeated id inside the list (random start) is dropped
-        first_offer[r] = valid && (k[r] & 1ull) && (!same_id || !(prev & 1ull));
-        known[r] = first_offer[r] && same_id;
-        offer_count += first_offer[r];
+        // a repeated entry (the random start lists of a very small partition) is dropped
+        valid[r] = k[r] != ~0ull && (head || (prev >> 1) != (k[r] >> 1));
+        const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+        sub[r] = num_sub == 1 ? 0u : id % num_sub;
+        slot[r] = kInvalid;
     }
-    uint32_t total_offer, total_keep, total_new;
-    uint32_t orank = wave_exclusive_scan(offer_count, lane, total_offer);
-    bool keep[NR], fresh[NR];
-    uint32_t keep_count = 0, fresh_count = 0;
+    for (uint32_t s = 0; s < num_sub; s++) {
+        uint32_t count = 0, total;
 #pragma unroll
-    for (int r = 0; r < NR; r++) {
-        fresh[r] = false;
-        keep[r] = from_list[r];
-        if (first_offer[r]) {
-            if (orank < kSamples) {
-                keep[r] = !known[r];
-                const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
-                const uint32_t base = (id % bloom_sets) * 512;
-                uint32_t h = bloom_h0(id);
-                const uint32_t b0 = base + h % 512;
-                h += bloom_h1(id);
-                const uint32_t b1 = base + h % 512;
-                h += bloom_h1(id);
-                const uint32_t b2 = base + h % 512;
-                const bool seen = ((filter[b0 >> 5] >> (b0 & 31)) & (filter[b1 >> 5] >> (b1 & 31)) & (filter[b2 >> 5] >> (b2 & 31)) & 1u) != 0;
-                fresh[r] = !seen;
+        for (int r = 0; r < NR; r++) count += valid[r] && sub[r] == s;
+        uint32_t rank = wave_exclusive_scan(count, total);
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            if (valid[r] && sub[r] == s) {
+                if (rank < kSamples) slot[r] = rank * num_sub + s;
+                rank++;
             }
-            orank++;
         }
-        keep_count += keep[r];
-        fresh_count += fresh[r];
+        for (uint32_t j = total + lane; j < kSamples; j += 64) {   // the unfilled tail of this sub-list
+            a.list_ids[static_cast<size_t>(node) * width + j * num_sub + s] = kInvalid;
+            a.list_dists[static_cast<size_t>(node) * width + j * num_sub + s] = FLT_MAX;
+        }
     }
-    uint32_t pos = wave_exclusive_scan(keep_count, lane, total_keep);
-    uint32_t nrank = wave_exclusive_scan(fresh_count, lane, total_new);
-    __builtin_amdgcn_wave_barrier();
     uint32_t inserted = 0;
 #pragma unroll
     for (int r = 0; r < NR; r++) {
-        const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
-        uint32_t flag = v[r];
-        if (fresh[r]) {   // at most 32 of them: all become samples
-            fwd_new[static_cast<size_t>(node) * kSamples + nrank] = id;
-            if (rev_new) reverse_append(counts, rev_new, seg_start, id, 2, node);
-            nrank++;
-            flag = kOld;
-            const uint32_t base = (id % bloom_sets) * 512;
-            uint32_t h = bloom_h0(id);
-            const uint32_t b0 = base + h % 512;
-            h += bloom_h1(id);
-            const uint32_t b1 = base + h % 512;
-            h += bloom_h1(id);
-            const uint32_t b2 = base + h % 512;
-            atomicOr(&filter[b0 >> 5], 1u << (b0 & 31));
-            atomicOr(&filter[b1 >> 5], 1u << (b1 & 31));
-            atomicOr(&filter[b2 >> 5], 1u << (b2 & 31));
-        }
-        if (keep[r]) {
-            if (pos < width) {
-                list_ids[static_cast<size_t>(node) * width + pos] = id | flag;
-                list_dists[static_cast<size_t>(node) * width + pos] = __uint_as_float(static_cast<uint32_t>(k[r] >> 32));
-                inserted += first_offer[r];
-            }
-            pos++;
+        if (slot[r] != kInvalid) {
+            const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+            a.list_ids[static_cast<size_t>(node) * width + slot[r]] = id | v[r];
+            a.list_dists[static_cast<size_t>(node) * width + slot[r]] = __uint_as_float(static_cast<uint32_t>(k[r] >> 32));
+            inserted += static_cast<uint32_t>(k[r] & 1ull);
         }
     }
     // update_counter (update_graph :1106-1126): insertions on every 100th row, per partition
     if (node % kCounterInterval == 0) {
         uint32_t total_inserted;
-        wave_exclusive_scan(inserted, lane, total_inserted);
-        if (lane == 0 && total_inserted) atomicAdd(&segs.updates[seg], total_inserted);
-    }
-    for (uint32_t e = total_keep + lane; e < width; e += 64) {
-        list_ids[static_cast<size_t>(node) * width + e] = kInvalid;
-        list_dists[static_cast<size_t>(node) * width + e] = FLT_MAX;
+        wave_exclusive_scan(inserted, total_inserted);
+        if (lane == 0 && total_inserted) atomicAdd(&a.segs.updates[seg], total_inserted);
     }
     __builtin_amdgcn_wave_barrier();
-    if (static_cast<uint32_t>(lane) < bloom_words) bloom[static_cast<size_t>(node) * bloom_words + lane] = filter[lane];
+    for (uint32_t w = lane; w < bloom_words; w += 64) a.bloom[static_cast<size_t>(node) * bloom_words + w] = filter[w];
     if (lane == 0) {
-        inbox_counts[node] = 0;
-        counts[static_cast<size_t>(node) * 4 + 0] = total_new;
-        counts[static_cast<size_t>(node) * 4 + 1] = total_old < kSamples ? total_old : kSamples;
-        if (!rev_new) {   // with the scatter fused in, other wavefronts are adding to these two right now; the join clears them
-            counts[static_cast<size_t>(node) * 4 + 2] = 0;
-            counts[static_cast<size_t>(node) * 4 + 3] = 0;
+        a.inbox_counts[node] = 0;
+        a.counts[static_cast<size_t>(node) * 4 + 0] = total_new;
+        a.counts[static_cast<size_t>(node) * 4 + 1] = total_old < kSamples ? total_old : kSamples;
+        if (!a.rev_new) {   // with the scatter fused in, other wavefronts are adding to these two right now; the join clears them
+            a.counts[static_cast<size_t>(node) * 4 + 2] = 0;
+            a.counts[static_cast<size_t>(node) * 4 + 3] = 0;
         }
-        if (stats) {   // striped over 1024 slots: one shared address would serialise every wavefront of the launch
-            unsigned long long* slot = stats + 2 * (blockIdx.x & 1023u);
-            atomicAdd(&slot[0], static_cast<unsigned long long>(raw));
-            if (raw > inbox_cap) atomicAdd(&slot[1], static_cast<unsigned long long>(raw - inbox_cap));
-        }
+        // striped over 1024 slots: one shared address would serialise every wavefront of the launch
+        if (a.stats && arrived) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u)], static_cast<unsigned long long>(arrived));
     }
-}
-
-template <int MMAX>
-__global__ __launch_bounds__(256) void nnd_merge_kernel(uint32_t* list_ids, float* list_dists, uint32_t* inbox_counts, const uint2* inbox, uint32_t num,
-                                                        uint32_t width, uint32_t inbox_cap, uint32_t* bloom, uint32_t bloom_sets, uint32_t* fwd_new,
-                                                        uint32_t* fwd_old, uint32_t* counts, unsigned long long* stats, Segments segs, uint32_t* rev_new,
-                                                        uint32_t* rev_old) {
-    __shared__ uint32_t filter_lds[4][64];
-    const int lane = lane_id();
-    const int wave = threadIdx.x >> 6;
-    const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (node >= num) return;
-    uint32_t seg_start, seg_len;
-    const uint32_t seg = locate_uniform(segs, node, seg_start, seg_len);
-    if (segs.state[seg] == kDone) return;
-    uint32_t* filter = filter_lds[wave];
-    const uint32_t bloom_words = bloom_sets * 16;
-    if (static_cast<uint32_t>(lane) < bloom_words) filter[lane] = bloom[static_cast<size_t>(node) * bloom_words + lane];
-    const uint32_t raw = inbox_counts[node];
-    const uint32_t held = width + (raw < inbox_cap ? raw : inbox_cap);   // the same for every lane of the wavefront
-    if (held <= 64)
-        merge_node<64>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
-                       seg, raw, filter, lane, seg_start, rev_new, rev_old);
-    else if (MMAX == 128 || held <= 128)
-        merge_node<128>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
-                        seg, raw, filter, lane, seg_start, rev_new, rev_old);
-    else
-        merge_node<256>(list_ids, list_dists, inbox_counts, inbox, width, inbox_cap, bloom, bloom_sets, fwd_new, fwd_old, counts, stats, segs, node,
-                        seg, raw, filter, lane, seg_start, rev_new, rev_old);
 }
 
 // Termination test of GNND::build's update_and_sample (nn_descent.cuh:1270-1284): a partition whose sampled update
@@ -732,7 +1022,9 @@ __global__ void nnd_converge_kernel(Segments segs, float limit) {
     segs.updates[s] = 0;
 }
 
-// ---- finalize (shrink step :1376-1402): first `degree` ids of each list; unfilled slots get a pseudo-random id
+// ---- finalize (shrink step :1376-1402): the `degree` nearest entries of each list; unfilled slots get a pseudo-random id.
+// The reference copies whole sub-lists in storage order (and so never returns an id of the last sub-list when the
+// degree is above 32); here the sub-lists are merged by (distance, id) first.
 __host__ __device__ inline uint32_t xorshift32(uint32_t u) {   // reference utils.cuh:14-19
     u ^= u >> 13;
     u ^= u << 27;
@@ -758,16 +1050,38 @@ __global__ __launch_bounds__(1024) void nnd_stats_reduce_kernel(const unsigned l
     }
 }
 
-__global__ __launch_bounds__(256) void nnd_finalize_kernel(const uint32_t* list_ids, uint32_t num, uint32_t width, uint32_t degree, Segments segs,
-                                                           uint32_t* knn_graph) {
-    const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
-    const uint32_t node = idx / degree, j = idx % degree;
+template <int M>
+__global__ __launch_bounds__(256) void nnd_finalize_kernel(const uint32_t* list_ids, const float* list_dists, uint32_t num, uint32_t width,
+                                                           uint32_t degree, Segments segs, uint32_t* knn_graph) {
+    constexpr int NR = M / 64;
+    const int lane = lane_id();
+    const uint32_t node = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (node >= num) return;
     uint32_t start, len;
-    locate(segs, node, start, len);
-    const uint32_t e = list_ids[static_cast<size_t>(node) * width + j];
-    const uint32_t id = e & ~kOld;
-    knn_graph[static_cast<size_t>(node) * degree + j] = (e != kInvalid && id < len) ? id : xorshift32(node * width + j) % (len ? len : 1);
+    locate_uniform(segs, node, start, len);
+    unsigned long long k[NR];
+    uint32_t none[NR];
+    uint32_t count = 0, total;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        k[r] = ~0ull;
+        if (e < width) {
+            const uint32_t entry = list_ids[static_cast<size_t>(node) * width + e];
+            const uint32_t id = entry & ~kOld;
+            if (entry != kInvalid && id < len) {
+                k[r] = (static_cast<unsigned long long>(__float_as_uint(list_dists[static_cast<size_t>(node) * width + e])) << 32) | id;
+                count++;
+            }
+        }
+    }
+    wave_exclusive_scan(count, total);
+    Net64<M, false>::sort(k, none, lane);
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        if (e < degree) knn_graph[static_cast<size_t>(node) * degree + e] = e < total ? static_cast<uint32_t>(k[r]) : xorshift32(node * width + e) % (len ? len : 1);
+    }
 }
 
 }  // namespace glide
@@ -776,33 +1090,37 @@ using namespace glide;
 
 namespace {
 uint32_t nnd_width(uint32_t degree) { return round_up32(static_cast<uint32_t>(degree * (degree <= 32 ? 1.0 : 1.3))); }  // nn_descent.cuh:1427-1428
-uint32_t nnd_inbox_cap(uint32_t width) { return 256 - width; }   // list + inbox fill one 256-element sort
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+constexpr uint32_t kMaxWidth = 192;   // six sub-lists: degrees up to 128 (width + 32 offers fit one 256-key network)
 
 struct NndLayout {
-    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, counts, inbox_counts, inbox, bloom, stats, seg_state, seg_updates, total;
-    uint32_t width, cap, dim_pad, bloom_sets;
+    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts, inbox_counts, inbox, offers, bloom, stats,
+        seg_state, seg_updates, total;
+    uint32_t width, dim_pad, bloom_sets;
 };
 NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
     NndLayout l;
     l.width = nnd_width(degree);
-    l.cap = nnd_inbox_cap(l.width);
     l.dim_pad = (dim + 7) / 8 * 8;
     l.bloom_sets = nnd_width(static_cast<uint32_t>(1.5 * degree)) / 32;   // internal degree / 32 (nn_descent.cuh:962, params.cuh:23-24)
     const size_t n = num;
     size_t off = 0;
     auto take = [&off](size_t bytes) { size_t o = off; off += align256(bytes); return o; };
     l.half_rows = take(n * l.dim_pad * 2);
-    l.norms = take(n * 4);
+    l.norms = take(n * 8);
     l.list_ids = take(n * l.width * 4);
     l.list_dists = take(n * l.width * 4);
     l.fwd_new = take(n * kSamples * 4);
     l.fwd_old = take(n * kSamples * 4);
-    l.rev_new = take(n * kSamples * 4);
-    l.rev_old = take(n * kSamples * 4);
+    l.rev_new = take(n * kRevStride * 4);
+    l.rev_old = take(n * kRevStride * 4);
+    // the next two are adjacent: one fill empties the overflow tables of the reverse samples and withdraws their thresholds
+    l.rev_tables = take(n * 2 * kRevSlots * 4);
+    l.rev_thr = take(n * 8);
     l.counts = take(n * 16);
     l.inbox_counts = take(n * 4);
-    l.inbox = take(n * l.cap * 8);
+    l.inbox = take(n * kInboxStride * 8);
+    l.offers = take(n * kOfferSlots * 8);
     l.bloom = take(n * l.bloom_sets * 64);
     l.stats = take(1024 * 16);
     l.seg_state = take(kMaxSegments * 4);
@@ -822,11 +1140,11 @@ namespace {
 struct NndCtx {
     NndLayout l;
     _Float16* half_rows;
-    float* norms;
+    float2* norms;
     uint32_t* list_ids;
     float* list_dists;
-    uint32_t *fwd_new, *fwd_old, *rev_new, *rev_old, *counts, *inbox_counts;
-    uint2* inbox;
+    uint32_t *fwd_new, *fwd_old, *rev_new, *rev_old, *rev_tables, *rev_thr, *counts, *inbox_counts;
+    unsigned long long *inbox, *offers;
     uint32_t* bloom;
     unsigned long long* stats;
     Segments segs;
@@ -834,29 +1152,35 @@ struct NndCtx {
     hipStream_t s;
 };
 
+bool nnd_degree_supported(uint32_t knn_degree) {
+    return knn_degree <= 128 && nnd_width(knn_degree) <= kMaxWidth && nnd_width(static_cast<uint32_t>(1.5 * knn_degree)) / 32 <= 8;   // Bloom filter within 128 words
+}
+
 int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
                 uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
     if (!segment_starts || !segment_lengths || !workspace) return GLIDE_ERR_BAD_ARGUMENT;
     if (dim == 0 || segment_num == 0 || knn_degree == 0 || reorder_num == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (segment_num > kMaxSegments) return GLIDE_ERR_UNSUPPORTED;
-    if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;   // also keeps the Bloom filter within 64 words
-    // one thread per list slot / per sample: the products must fit the 32-bit launch arithmetic (44 M rows at width 96)
+    if (!nnd_degree_supported(knn_degree) || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    // one thread per list slot / per sample: the products must fit the 32-bit launch arithmetic
     if (static_cast<unsigned long long>(reorder_num) * nnd_width(knn_degree) >= 0xffffffffull || reorder_num >= (1u << 26)) return GLIDE_ERR_UNSUPPORTED;
     c.l = nnd_layout(reorder_num, dim, knn_degree);
-    if (c.l.bloom_sets > 4) return GLIDE_ERR_UNSUPPORTED;
     if (workspace_bytes < c.l.total || reinterpret_cast<uintptr_t>(workspace) % 16) return GLIDE_ERR_BAD_ARGUMENT;
     unsigned char* w = static_cast<unsigned char*>(workspace);
     c.half_rows = reinterpret_cast<_Float16*>(w + c.l.half_rows);
-    c.norms = reinterpret_cast<float*>(w + c.l.norms);
+    c.norms = reinterpret_cast<float2*>(w + c.l.norms);
     c.list_ids = reinterpret_cast<uint32_t*>(w + c.l.list_ids);
     c.list_dists = reinterpret_cast<float*>(w + c.l.list_dists);
     c.fwd_new = reinterpret_cast<uint32_t*>(w + c.l.fwd_new);
     c.fwd_old = reinterpret_cast<uint32_t*>(w + c.l.fwd_old);
     c.rev_new = reinterpret_cast<uint32_t*>(w + c.l.rev_new);
     c.rev_old = reinterpret_cast<uint32_t*>(w + c.l.rev_old);
+    c.rev_tables = reinterpret_cast<uint32_t*>(w + c.l.rev_tables);
+    c.rev_thr = reinterpret_cast<uint32_t*>(w + c.l.rev_thr);
     c.counts = reinterpret_cast<uint32_t*>(w + c.l.counts);
     c.inbox_counts = reinterpret_cast<uint32_t*>(w + c.l.inbox_counts);
-    c.inbox = reinterpret_cast<uint2*>(w + c.l.inbox);
+    c.inbox = reinterpret_cast<unsigned long long*>(w + c.l.inbox);
+    c.offers = reinterpret_cast<unsigned long long*>(w + c.l.offers);
     c.bloom = reinterpret_cast<uint32_t*>(w + c.l.bloom);
     c.stats = reinterpret_cast<unsigned long long*>(w + c.l.stats);
     c.segs = Segments{segment_starts, segment_lengths, segment_num, reinterpret_cast<uint32_t*>(w + c.l.seg_state),
@@ -873,43 +1197,48 @@ int nnd_prepare(const NndCtx& c, const float* data, uint32_t dim, uint32_t seed)
     if (rc != GLIDE_OK) return rc;
     rc = glide_hip_fill_u32(c.segs.state, 0u, 2 * kMaxSegments, c.s);   // state and updates are adjacent
     if (rc != GLIDE_OK) return rc;
+    // empty overflow tables (their bounds included: nothing turned away yet), empty inboxes
+    rc = glide_hip_fill_u32(c.rev_tables, kInvalid, (c.l.counts - c.l.rev_tables) / 4, c.s);
+    if (rc != GLIDE_OK) return rc;
+    rc = glide_hip_fill_u32(c.inbox_counts, 0u, c.n, c.s);
+    if (rc != GLIDE_OK) return rc;
+    rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(c.offers), kInvalid, static_cast<size_t>(c.n) * kOfferSlots * 2, c.s);
+    if (rc != GLIDE_OK) return rc;
     hipLaunchKernelGGL(nnd_prepare_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, data, c.n, dim, c.l.dim_pad, c.half_rows, c.norms);
-    hipLaunchKernelGGL(nnd_init_kernel, dim3(ceil_div(c.n * c.l.width, 256)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.n,
-                       c.l.width, c.segs, seed);
+    hipLaunchKernelGGL(nnd_init_kernel, dim3(ceil_div(c.n * c.l.width, 256)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, c.segs, seed);
     // first samples come from the random lists (sample_graph(true), nn_descent.cuh:1266); later ones from the merge
     hipLaunchKernelGGL(nnd_sample_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.n, c.l.width, c.segs, c.fwd_new, c.fwd_old, c.counts);
     return launch_status();
 }
 
 int nnd_reverse(const NndCtx& c) {
-    hipLaunchKernelGGL(nnd_reverse_kernel, dim3(ceil_div(c.n * 64, 256)), dim3(256), 0, c.s, c.fwd_new, c.fwd_old, c.counts, c.rev_new, c.rev_old, c.n,
-                       c.segs);
+    hipLaunchKernelGGL(nnd_reverse_kernel, dim3(ceil_div(c.n * 64, 256)), dim3(256), 0, c.s, c.fwd_new, c.fwd_old, c.counts, c.rev_new, c.rev_old,
+                       c.rev_tables, c.rev_thr, c.n, c.segs);
     return launch_status();
 }
 
-int nnd_join(const NndCtx& c) {
+int nnd_join(const NndCtx& c, bool with_stats) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
-    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.counts, c.inbox_counts, c.inbox, c.stats,
-                c.n, c.l.dim_pad, c.l.width, c.l.cap, c.segs};
+    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.inbox_counts, c.inbox,
+                c.offers, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
     hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja);
     return launch_status();
 }
 
-// scatter_reverse: the new and old samples a node draws are appended to the reverse lists of their targets right away
+// scatter_reverse: the new and old samples a node draws enter the reverse tables of their targets right away
 // (what the next round's nnd_reverse would do), while the sort of other nodes keeps the vector ALU busy
 int nnd_merge(const NndCtx& c, bool with_stats, bool scatter_reverse = false) {
-    unsigned long long* stats = with_stats ? c.stats : nullptr;
-    uint32_t* rev_new = scatter_reverse ? c.rev_new : nullptr;
-    uint32_t* rev_old = scatter_reverse ? c.rev_old : nullptr;
-    const uint32_t m = c.l.width + c.l.cap;
-    if (m <= 128) {
-        hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
-                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs, rev_new, rev_old);
-    } else {
-        hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.n,
-                           c.l.width, c.l.cap, c.bloom, c.l.bloom_sets, c.fwd_new, c.fwd_old, c.counts, stats, c.segs, rev_new, rev_old);
-    }
+    MergeArgs ma{c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.offers, c.bloom, c.fwd_new, c.fwd_old, c.counts, with_stats ? c.stats : nullptr, c.segs,
+                 scatter_reverse ? c.rev_new : nullptr, scatter_reverse ? c.rev_old : nullptr, scatter_reverse ? c.rev_tables : nullptr, c.rev_thr, c.norms,
+                 c.n, c.l.width, c.l.width / kSamples, c.l.bloom_sets};
+    const uint32_t m = c.l.width + kSamples;
+    if (m <= 64)
+        hipLaunchKernelGGL(nnd_merge_kernel<64>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
+    else if (m <= 128)
+        hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
+    else
+        hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
     return launch_status();
 }
 
@@ -921,8 +1250,12 @@ int nnd_converge(const NndCtx& c, uint32_t dim, float termination_threshold) {
 }
 
 int nnd_finalize(const NndCtx& c, uint32_t knn_degree, uint32_t* knn_graph, unsigned long long* stats_out) {
-    hipLaunchKernelGGL(nnd_finalize_kernel, dim3(ceil_div(c.n * knn_degree, 256)), dim3(256), 0, c.s, c.list_ids, c.n, c.l.width, knn_degree, c.segs,
-                       knn_graph);
+    if (c.l.width <= 64)
+        hipLaunchKernelGGL(nnd_finalize_kernel<64>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, knn_degree, c.segs, knn_graph);
+    else if (c.l.width <= 128)
+        hipLaunchKernelGGL(nnd_finalize_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, knn_degree, c.segs, knn_graph);
+    else
+        hipLaunchKernelGGL(nnd_finalize_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, knn_degree, c.segs, knn_graph);
     if (stats_out) hipLaunchKernelGGL(nnd_stats_reduce_kernel, dim3(1), dim3(1024), 0, c.s, c.stats, stats_out);
     return launch_status();
 }
@@ -940,7 +1273,7 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
     if ((rc = nnd_prepare(c, reorder_data, dim, seed)) != GLIDE_OK) return rc;
     for (uint32_t it = 0; it < iterations; it++) {
         if (it == 0 && (rc = nnd_reverse(c)) != GLIDE_OK) return rc;   // later rounds: the merge of the round before has done it
-        if ((rc = nnd_join(c)) != GLIDE_OK) return rc;
+        if ((rc = nnd_join(c, stats_out != nullptr)) != GLIDE_OK) return rc;
         if ((rc = nnd_merge(c, stats_out != nullptr, it + 1 < iterations)) != GLIDE_OK) return rc;
         if ((rc = nnd_converge(c, dim, termination_threshold)) != GLIDE_OK) return rc;
         // GNND::build leaves its loop when the update count falls below the limit (nn_descent.cuh:1270-1284).  Here the
@@ -960,13 +1293,13 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
 
 int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree, glide_nnd_layout* out) {
     if (!out || dim == 0 || knn_degree == 0) return GLIDE_ERR_BAD_ARGUMENT;
-    if (nnd_width(knn_degree) > 96 || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
+    if (!nnd_degree_supported(knn_degree) || dim % 4 != 0) return GLIDE_ERR_UNSUPPORTED;
     const NndLayout l = nnd_layout(reorder_num, dim, knn_degree);
     out->half_rows = l.half_rows; out->norms = l.norms; out->list_ids = l.list_ids; out->list_dists = l.list_dists;
-    out->fwd_new = l.fwd_new; out->fwd_old = l.fwd_old; out->rev_new = l.rev_new; out->rev_old = l.rev_old;
-    out->counts = l.counts; out->inbox_counts = l.inbox_counts; out->inbox = l.inbox; out->bloom = l.bloom;
+    out->fwd_new = l.fwd_new; out->fwd_old = l.fwd_old; out->rev_new = l.rev_new; out->rev_old = l.rev_old; out->rev_tables = l.rev_tables; out->rev_thr = l.rev_thr;
+    out->counts = l.counts; out->inbox_counts = l.inbox_counts; out->inbox = l.inbox; out->offers = l.offers; out->bloom = l.bloom;
     out->segment_state = l.seg_state; out->segment_updates = l.seg_updates; out->total = l.total;
-    out->width = l.width; out->inbox_cap = l.cap; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
+    out->width = l.width; out->reverse_cap = kRevCap; out->reverse_stride = kRevStride; out->inbox_cap = kInboxCap; out->inbox_stride = kInboxStride; out->offer_slots = kOfferSlots; out->reverse_slots = kRevSlots; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
     return GLIDE_OK;
 }
 
@@ -990,7 +1323,7 @@ int glide_hip_nnd_local_join(uint32_t reorder_num, uint32_t dim, const uint32_t*
                              uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
     NndCtx c;
     int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
-    return rc != GLIDE_OK ? rc : nnd_join(c);
+    return rc != GLIDE_OK ? rc : nnd_join(c, true);
 }
 
 int glide_hip_nnd_merge(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,

@@ -376,7 +376,7 @@ extern "C" int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, 
 #ifdef _OPENMP
     if (threads > 0) omp_set_num_threads(threads);
 #endif
-    if (knn_degree == 0 || knn_degree > 64) return -1;
+    if (knn_degree == 0 || knn_degree > 128) return -1;
     // preprocess_data_kernel nn_descent.cuh:445-488: rows stored as halfs, squared norms taken from the fp32 input
     std::vector<float> half(static_cast<size_t>(reorder_num) * dim), norms(reorder_num);
 #pragma omp parallel for schedule(static)

@@ -116,16 +116,17 @@ def test_nnd_termination_threshold(hip):
 def test_nnd_rejects_unsupported(hip):
     d = hip.DeviceArray(1024, np.float32)
     with pytest.raises(hip.GlideHipError) as e:
-        hip.nnd_build(d, 8, 128, d, d, 1, 100, 1, 0.0, 0, d, d, 1 << 30)
+        hip.nnd_build(d, 8, 128, d, d, 1, 129, 1, 0.0, 0, d, d, 1 << 30)      # list width above 192 (six sub-lists)
     assert e.value.code == -1
     with pytest.raises(hip.GlideHipError) as e:
         hip.nnd_build(d, 8, 128, d, d, 1, 32, 1, 0.0, 0, d, d, 16)      # workspace too small
     assert e.value.code == -2
 
 
-@pytest.mark.parametrize("dim,k", [(4, 8), (36, 16), (100, 32), (132, 48), (260, 64), (1024, 24)])
+@pytest.mark.parametrize("dim,k", [(4, 8), (36, 16), (100, 32), (132, 48), (260, 64), (1024, 24), (128, 96), (64, 128)])
 def test_nnd_shapes(hip, dim, k):
-    """Dimensions that are not a multiple of the 64-dim chunk of the join (or of 8) and list widths 32, 64 and 96."""
+    """Dimensions that are not a multiple of the 64-dim chunk of the join (or of 8) and list widths 32, 64, 96, 128 and 192
+    (the reference accepts any degree, nn_descent.cuh:1423-1430; its evaluation runs degree 96)."""
     data = lowdim_data(3000, dim, latent=min(8, dim), seed=dim)
     seg_len = np.array([1800, 1200], dtype=np.uint32)
     seg_start = np.array([0, 1800], dtype=np.uint32)
@@ -135,4 +136,31 @@ def test_nnd_shapes(hip, dim, k):
         assert (rows < l).all() and (rows != np.arange(l, dtype=np.uint32)[:, None]).all()
     r = partition_recall(knn, data, seg_start, seg_len, k, sample=200)
     print("graph recall@%d (dim %d): %.4f" % (k, dim, r))
-    assert r >= (0.9 if dim > 4 else 0.6)      # 4 small-integer dimensions are mostly ties
+    if k > 64:
+        # at most 32 offers a round enter a list of 128 or 192 slots: after 12 rounds the tail is still filling, in
+        # the CPU restatement alike; the bar is the restatement's recall at equal degree and iterations
+        from oracle import oracle as O
+        cpu = O.nnd_build(data, seg_start, seg_len, k, 12).astype(np.uint32)
+        r_cpu = partition_recall(cpu, data, seg_start, seg_len, k, sample=200)
+        print("cpu restatement: %.4f" % r_cpu)
+        assert r >= r_cpu - 0.005
+    else:
+        assert r >= (0.9 if dim > 4 else 0.6)      # 4 small-integer dimensions are mostly ties
+
+
+def test_nnd_same_seed_same_graph(hip):
+    """Nothing in the build depends on the order in which atomic operations arrive: the offer tables keep the smallest
+    keys, the reverse tables the smallest sources, and both are sorted before use.  Mixture data, where a few points
+    receive thousands of offers per round, and a degree with three sub-lists."""
+    from glide_amd import datasets as D
+    data = D.gmm_clipped(24000, 128, seed=7)
+    seg_start, seg_len = np.array([0, 14000], np.uint32), np.array([14000, 10000], np.uint32)
+    for k, rounds in ((32, 6), (64, 4)):
+        a, st_a = gpu_nnd(hip, data, seg_start, seg_len, k, rounds, seed=3)
+        b, st_b = gpu_nnd(hip, data, seg_start, seg_len, k, rounds, seed=3)
+        c, _ = gpu_nnd(hip, data, seg_start, seg_len, k, rounds, seed=4)
+        # st[1] counts arrivals turned away by a full bucket: copies of one offer may be counted once or twice, depending on
+        # whether the second copy still finds the first; what the tables end up holding (st[0]) does not depend on that
+        assert np.array_equal(a, b) and st_a[0] == st_b[0]
+        assert not np.array_equal(a, c)
+        print("degree %d: offers merged %d, dropped by full buckets %d" % (k, st_a[0], st_a[1]))

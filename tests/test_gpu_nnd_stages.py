@@ -15,6 +15,9 @@ pytestmark = pytest.mark.gpu
 INV = 0xFFFFFFFF
 OLD = 0x80000000
 S = 32   # samples per list (NUM_SAMPLES, nn_descent.cuh:391)
+R = 256  # words of a reverse overflow table: 16 buckets of 15 slots + the bucket's bound
+CAP = 256  # offers an inbox holds before the overflow table takes over
+RCAP = 64  # reverse samples a list holds before the overflow table takes over
 
 
 @pytest.fixture(scope="module")
@@ -39,11 +42,76 @@ class Workspace:
         return dict(
             list_ids=f(l.list_ids, n * l.width).reshape(n, l.width), list_dists=f(l.list_dists, n * l.width, np.float32).reshape(n, l.width),
             fwd_new=f(l.fwd_new, n * S).reshape(n, S), fwd_old=f(l.fwd_old, n * S).reshape(n, S),
-            rev_new=f(l.rev_new, n * S).reshape(n, S), rev_old=f(l.rev_old, n * S).reshape(n, S),
-            counts=f(l.counts, n * 4).reshape(n, 4), inbox_counts=f(l.inbox_counts, n),
+            rev_new=f(l.rev_new, n * l.reverse_stride).reshape(n, l.reverse_stride)[:, :RCAP], rev_old=f(l.rev_old, n * l.reverse_stride).reshape(n, l.reverse_stride)[:, :RCAP],
+            rev_tables=f(l.rev_tables, n * 2 * R).reshape(n, 2, R), counts=f(l.counts, n * 4).reshape(n, 4),
+            rev_thr=f(l.rev_thr, n * 2).reshape(n, 2),
+            inbox_counts=f(l.inbox_counts, n), inbox=f(l.inbox, n * l.inbox_stride * 2).view(np.uint64).reshape(n, l.inbox_stride)[:, :CAP],
             segment_state=f(l.segment_state, 16), segment_updates=f(l.segment_updates, 16),
-            inbox=f(l.inbox, n * l.inbox_cap * 2).reshape(n, l.inbox_cap, 2), bloom=f(l.bloom, n * l.bloom_sets * 16).reshape(n, l.bloom_sets * 16),
-            norms=f(l.norms, n, np.float32))
+            offers=f(l.offers, n * l.offer_slots * 2).view(np.uint64).reshape(n, l.offer_slots),
+            bloom=f(l.bloom, n * l.bloom_sets * 16).reshape(n, l.bloom_sets * 16),
+            norms=f(l.norms, 2 * n, np.float32)[0::2].copy(), offer_thr=f(l.norms, 2 * n)[1::2].copy())
+
+
+NO_OFFER = np.uint64(0xFFFFFFFFFFFFFFFF)
+SLOT = np.arange(256) % 16 != 15          # word 15 of every bucket of 16 is the bucket's bound, the others are slots
+
+
+def offer_key(dist, cand):
+    return (int(np.float32(dist).view(np.uint32)) << 32) | int(cand)
+
+
+def bucket_table(keys, bucket_bits, empty):
+    """What a table of 2^bucket_bits buckets holds of `keys` (their low 32 bits are the id that is hashed): per bucket the
+    15 smallest distinct keys; returns (kept keys sorted, {bucket: bound}) where a bucket's bound is the smallest key it
+    turned away."""
+    buckets = {}
+    for key in set(keys):
+        buckets.setdefault((((key & 0xFFFFFFFF) * 0x9E3779B1) & 0xFFFFFFFF) >> (32 - bucket_bits), []).append(key)
+    kept = sorted(k for b in buckets.values() for k in sorted(b)[:15])
+    bounds = {i: (sorted(b)[15] if len(b) > 15 else empty) for i, b in buckets.items()}
+    return kept, bounds
+
+
+def kept_by_table(keys):
+    return bucket_table(keys, 4, int(NO_OFFER))[0]
+
+
+def table_slots(row):
+    """(slot values that are not empty, sorted; the bucket bounds) of one table row as read from the device."""
+    row = np.asarray(row)
+    empty = NO_OFFER if row.dtype == np.uint64 else np.uint32(INV)
+    slots = row[SLOT[:row.size]]
+    return sorted(int(x) for x in slots[slots != empty]), [int(x) for x in row[15::16]]
+
+
+def reverse_samples(st, node, which):
+    """The 32 smallest sources that arrived at `node`: its list (the first 32 arrivals) and, beyond 32 arrivals, its overflow table."""
+    cnt = int(st["counts"][node, 2 + which])
+    got = [int(x) for x in st[("rev_new", "rev_old")[which]][node, :min(cnt, RCAP)]]
+    if cnt > RCAP:
+        got += table_slots(st["rev_tables"][node, which])[0]
+    return sorted(set(got))[:S]
+
+
+def offers_held(st, node):
+    """Distinct offers a node holds after a join, ascending: inbox and, beyond CAP arrivals, its overflow table."""
+    cnt = int(st["inbox_counts"][node])
+    got = [int(x) for x in st["inbox"][node, :min(cnt, CAP)]]
+    if cnt > CAP:
+        got += table_slots(st["offers"][node])[0]
+    return sorted(set(got))
+
+
+def model_offer_threshold(st, node):
+    """The threshold a node announces for the next join: after an overflow of its inbox the distance (bits) of the 64th best
+    distinct offer of the round; one in force is kept while 64 or more offers arrive and the best 32 are complete."""
+    cnt = int(st["inbox_counts"][node])
+    if cnt > CAP:
+        distinct = offers_held(st, node)
+        return distinct[63] >> 32 if len(distinct) >= 64 else INV
+    if cnt >= 64 and len(offers_held(st, node)) >= S:
+        return int(st["offer_thr"][node])
+    return INV
 
 
 def _dedupe(first, second, limit):
@@ -64,8 +132,9 @@ def model_join(st, rows, seg_start, seg_len):
     norms = (rows.astype(np.float32) ** 2).sum(1, dtype=np.float32)
     for node in range(seg_start, seg_start + seg_len):
         c = st["counts"][node]
-        new = _dedupe(st["fwd_new"][node, :c[0]], st["rev_new"][node, :min(c[2], S)], seg_len)
-        old = _dedupe(st["fwd_old"][node, :c[1]], st["rev_old"][node, :min(c[3], S)], seg_len)
+        # forward samples in list order, then the 32 smallest reverse samples in ascending order
+        new = _dedupe(st["fwd_new"][node, :c[0]], reverse_samples(st, node, 0), seg_len)
+        old = _dedupe(st["fwd_old"][node, :c[1]], reverse_samples(st, node, 1), seg_len)
         if not new:
             continue
         xn, nn_ = half[seg_start + np.array(new)], norms[seg_start + np.array(new)]
@@ -94,7 +163,8 @@ def model_join(st, rows, seg_start, seg_len):
                         best, bi = d[i, j], a
                 if bi is not None:
                     offers.setdefault(b, []).append((float(best), bi))
-    return {k: sorted(v) for k, v in offers.items()}
+    # a node that overflowed has announced a threshold: offers that are not below it stay away
+    return {k: sorted(o for o in v if offer_key(*o) >> 32 < int(st["offer_thr"][seg_start + k])) for k, v in offers.items()}
 
 
 def _bloom_bits(key, sets):
@@ -116,52 +186,48 @@ def _bloom_bits(key, sets):
     return bits
 
 
-def model_merge(st, node, width, cap, sets):
-    """One node of the merge stage; returns (list_ids, list_dists, fwd_new, n_new, fwd_old, n_old, bloom words,
-    number of offers that entered the list)."""
+def model_merge(st, node, width, sets):
+    """One node of the merge stage; returns (list_ids, list_dists, fwd_new, fwd_old, bloom words, number of offers that
+    entered the list).  The list is width / 32 sub-lists keyed by id % (width / 32); entry r of sub-list s is slot
+    r * (width / 32) + s (update_graph nn_descent.cuh:1106-1126, insert_to_ordered_list :916-943)."""
+    num_sub = width // S
     ids, dists = [int(v) for v in st["list_ids"][node]], st["list_dists"][node]
-    fwd_old = [v & ~OLD for v in ids if v != INV and v & OLD]
-    n_in = min(int(st["inbox_counts"][node]), cap)
-    ent = []   # (dist bits, id, source, flag)
-    for v, d in zip(ids, dists):
-        if v != INV:
-            ent.append((int(np.float32(d).view(np.uint32)), v & ~OLD, 0, v & OLD))
-    for db, cand in st["inbox"][node, :n_in]:
-        ent.append((int(db), int(cand), 1, 0))
+    fwd_old = [v & ~OLD for v in ids if v != INV and v & OLD][:S]
+    best = offers_held(st, node)[:S]      # the round's 32-wide device list
+    held = {v & ~OLD for v in ids if v != INV}
+    words, seen_before = st["bloom"][node].copy(), st["bloom"][node].copy()
+    ent = [(int(np.float32(d).view(np.uint32)), v & ~OLD, 0, v & OLD) for v, d in zip(ids, dists) if v != INV]
+    fwd_new = []
+    for key in best:
+        db, cand = key >> 32, key & 0xFFFFFFFF
+        bits = _bloom_bits(cand, sets)
+        fresh = not all((int(seen_before[b >> 5]) >> (b & 31)) & 1 for b in bits)
+        if fresh:
+            fwd_new.append(cand)
+            for b in bits:
+                words[b >> 5] |= np.uint32(1 << (b & 31))
+        if cand not in held:          # an id the list holds is rejected whatever its distance there
+            held.add(cand)
+            ent.append((db, cand, 1, OLD if fresh else 0))
     ent.sort(key=lambda e: (e[0], e[1], e[2]))
-    words = st["bloom"][node].copy()
-    seen_before = words.copy()
-    out, fwd_new, rank = [], [], 0
-    prev = None
-    for e in ent:
-        same = prev is not None and prev[0] == e[0] and prev[1] == e[1]
-        if e[2] == 0:
-            if not same:
-                out.append((e[1] | e[3], e[0], 0))
-        elif not same or prev[2] == 0:          # first offered copy of this id
-            known = same
-            if rank < S:
-                bits = _bloom_bits(e[1], sets)
-                fresh = not all((int(seen_before[b >> 5]) >> (b & 31)) & 1 for b in bits)
-                if fresh:
-                    fwd_new.append(e[1])
-                    for b in bits:
-                        words[b >> 5] |= np.uint32(1 << (b & 31))
-                if not known:
-                    out.append((e[1] | (OLD if fresh else 0), e[0], 1))
-            rank += 1
-        prev = e
-    out = out[:width]
     l_ids = np.full(width, INV, np.uint32)
     l_d = np.full(width, np.finfo(np.float32).max, np.float32)
-    inserted = sum(o[2] for o in out)
-    for i, (v, db, _) in enumerate(out):
-        l_ids[i] = v
-        l_d[i] = np.array([db], np.uint32).view(np.float32)[0]
-    return l_ids, l_d, fwd_new, len(fwd_new), fwd_old[:S], min(len(fwd_old), S), words, inserted
+    rank, inserted, prev = [0] * num_sub, 0, None
+    for e in ent:
+        if prev is not None and prev[:2] == e[:2]:
+            continue                   # a repeated entry of a random start list
+        prev = e
+        s_ = e[1] % num_sub
+        if rank[s_] < S:
+            slot = rank[s_] * num_sub + s_
+            l_ids[slot] = e[1] | e[3]
+            l_d[slot] = np.array([e[0]], np.uint32).view(np.float32)[0]
+            inserted += e[2]
+        rank[s_] += 1
+    return l_ids, l_d, fwd_new, fwd_old, words, inserted
 
 
-@pytest.mark.parametrize("degree", [32, 64])
+@pytest.mark.parametrize("degree", [32, 64, 96, 128])
 def test_stages_match_model(hip, degree):
     num, dim = 2400, 128
     rows = lowdim_data(num, dim, seed=5)
@@ -173,13 +239,20 @@ def test_stages_match_model(hip, degree):
     hip.nnd_prepare(d_rows, num, dim, d_ss, d_sl, 2, degree, 3, ws.buf, ws.bytes)
     hip.synchronize()
     st = ws.read()
-    width, cap, sets = ws.l.width, ws.l.inbox_cap, ws.l.bloom_sets
-    # prepare: random partition-local ids, no self, all sampled (flagged) as the first "new" samples
+    width, sets = ws.l.width, ws.l.bloom_sets
+    num_sub = width // S
+    assert width == {32: 32, 64: 96, 96: 128, 128: 192}[degree] and ws.l.offer_slots == 256
+    # prepare: random partition-local ids, no self, sub-list s holds ids = s mod num_sub; the first 32 in storage
+    # order are sampled (flagged) as the first "new" samples
     local = np.arange(num) - np.repeat(seg_start, seg_len)
     lim = np.repeat(seg_len, seg_len)[:, None]
     assert ((st["list_ids"] & ~np.uint32(OLD)) < lim).all()
     assert ((st["list_ids"] & ~np.uint32(OLD)) != local[:, None]).all()
+    assert (((st["list_ids"] & ~np.uint32(OLD)) % num_sub) == (np.arange(width) % num_sub)[None, :]).all()
     assert (st["counts"][:, 0] == S).all() and (st["counts"][:, 1] == 0).all()
+    np.testing.assert_array_equal(st["fwd_new"], st["list_ids"][:, :S] & ~np.uint32(OLD))
+    assert (st["offers"] == NO_OFFER).all() and (st["rev_tables"] == INV).all() and (st["inbox_counts"] == 0).all()
+    assert (st["counts"][:, 2:] == 0).all() and (st["rev_thr"] == INV).all() and (st["offer_thr"] == INV).all()
     np.testing.assert_array_equal(st["norms"], (rows ** 2).sum(1, dtype=np.float32))
 
     for it in range(3):
@@ -187,37 +260,59 @@ def test_stages_match_model(hip, degree):
         hip.nnd_reverse_sample(*args)
         hip.synchronize()
         st = ws.read()
-        # reverse samples: v in fwd(u)  <=>  u arrives at rev(v); arrivals counted, the first 32 stored (any order)
+        # reverse samples: v in fwd(u)  <=>  u arrives at rev(v).  Every arrival is counted, the first 64 sit in the list,
+        # later ones in the overflow table; what the join uses are the 32 smallest sources (what a sweep over the lists in
+        # order keeps, add_rev_edges_kernel :490-507), whatever the order of arrival was
+        overflowed = 0
         for which, fwd, rev in ((0, "fwd_new", "rev_new"), (1, "fwd_old", "rev_old")):
             expect = {}
             for s0, l0 in zip(seg_start, seg_len):
                 for u in range(s0, s0 + l0):
                     for v in st[fwd][u, :st["counts"][u, which]]:
-                        expect.setdefault(int(s0 + v), []).append(int(u - s0))
+                        if u - s0 < st["rev_thr"][s0 + v, which]:       # sources not below a node's threshold stay away
+                            expect.setdefault(int(s0 + v), []).append(int(u - s0))
             for v in range(num):
-                e = expect.get(v, [])
+                e = sorted(expect.get(v, ()))
                 assert st["counts"][v, 2 + which] == len(e)
-                got = Counter(st[rev][v, :min(len(e), S)].tolist())
-                assert not got - Counter(e)          # a sub-multiset of the arrivals
-                if len(e) <= S:
-                    assert got == Counter(e)
-        assert (st["inbox_counts"] == 0).all()
+                assert not Counter(st[rev][v, :min(len(e), RCAP)].tolist()) - Counter(e)       # the list: a sub-multiset of the arrivals
+                in_table, bounds = table_slots(st["rev_tables"][v, which])
+                if len(e) <= RCAP:
+                    assert not in_table and all(b == INV for b in bounds)
+                else:
+                    overflowed += 1
+                    assert not Counter(in_table) - Counter(e)
+                assert reverse_samples(st, v, which) == sorted(set(e))[:S]
+        assert overflowed > 0 or it == 0 or degree > 32
+        assert (st["offers"] == NO_OFFER).all() and (st["inbox_counts"] == 0).all()
 
         hip.nnd_local_join(*args)
         hip.synchronize()
         after = ws.read()
+        assert (after["rev_tables"] == INV).all() and (after["counts"][:, 2:] == 0).all()      # consumed by the join
+        # thresholds for the next scatter: after an overflow the 56th smallest source, kept while 40 or more still arrive
+        for which in (0, 1):
+            for v in range(num):
+                cnt = int(st["counts"][v, 2 + which])
+                if cnt > RCAP:
+                    union = sorted(set([int(x) for x in st[("rev_new", "rev_old")[which]][v]] + table_slots(st["rev_tables"][v, which])[0]))
+                    want = union[55] if len(union) >= 56 else INV
+                else:
+                    want = int(st["rev_thr"][v, which]) if cnt >= 40 else INV
+                assert after["rev_thr"][v, which] == want, (which, v, cnt)
         total = 0
         for s0, l0 in zip(seg_start.tolist(), seg_len.tolist()):
             offers = model_join(st, rows, s0, l0)
             for t in range(l0):
-                exp = offers.get(t, [])
+                exp = sorted(offer_key(d, c) for d, c in offers.get(t, []))
                 cnt = int(after["inbox_counts"][s0 + t])
                 assert cnt == len(exp), (s0, t, cnt, len(exp))
-                got = sorted((float(np.array([db], np.uint32).view(np.float32)[0]), int(c)) for db, c in after["inbox"][s0 + t, :min(cnt, cap)])
-                if cnt <= cap:
+                got = sorted(int(x) for x in after["inbox"][s0 + t, :min(cnt, CAP)])
+                if cnt <= CAP:
                     assert got == exp, (s0, t)
+                    assert (after["offers"][s0 + t] == NO_OFFER).all()
                 else:
-                    assert all(g in exp for g in got)
+                    assert not Counter(got) - Counter(exp)
+                assert offers_held(after, s0 + t)[:S] == sorted(set(exp))[:S]
                 total += cnt
         assert total > 0
 
@@ -226,17 +321,26 @@ def test_stages_match_model(hip, degree):
         merged = ws.read()
         updates = [0, 0]
         for node in range(num):
-            l_ids, l_d, fn, n_new, fo, n_old, words, inserted = model_merge(after, node, width, cap, sets)
+            l_ids, l_d, fn, fo, words, inserted = model_merge(after, node, width, sets)
             if node % 100 == 0:
                 updates[0 if node < seg_len[0] else 1] += inserted
             np.testing.assert_array_equal(merged["list_ids"][node], l_ids, err_msg="list ids of node %d" % node)
             np.testing.assert_array_equal(merged["list_dists"][node], l_d)
-            assert merged["counts"][node].tolist() == [n_new, n_old, 0, 0]
-            assert merged["fwd_new"][node, :n_new].tolist() == fn
-            assert merged["fwd_old"][node, :n_old].tolist() == fo
+            assert merged["counts"][node].tolist() == [len(fn), len(fo), 0, 0]
+            assert merged["fwd_new"][node, :len(fn)].tolist() == fn
+            assert merged["fwd_old"][node, :len(fo)].tolist() == fo
             np.testing.assert_array_equal(merged["bloom"][node], words)
-        assert (merged["inbox_counts"] == 0).all()
+        assert (merged["offers"] == NO_OFFER).all() and (merged["inbox_counts"] == 0).all()
         assert merged["segment_updates"][:2].tolist() == updates
+        for node in range(num):
+            assert int(merged["offer_thr"][node]) == model_offer_threshold(after, node), node
+        # lists: no id twice, never the node itself, every sub-list nearest first
+        clean = merged["list_ids"] & ~np.uint32(OLD)
+        for node in range(0, num, 7):
+            row = clean[node][merged["list_ids"][node] != INV]
+            assert len(set(row.tolist())) == row.size and (row != local[node]).all()
+        for s_ in range(num_sub):
+            assert (np.diff(merged["list_dists"][:, s_::num_sub], axis=1) >= 0).all()
         # termination test: limit = threshold * rows * dim / 100; a partition below it gets one more round, then rests
         threshold = [0.0, 1e9, 1e9][it]
         before = merged["segment_state"][:2].tolist()
@@ -253,13 +357,105 @@ def test_stages_match_model(hip, degree):
     hip.nnd_merge(*args)
     hip.synchronize()
     rest = ws.read()
-    for key in ("list_ids", "list_dists", "fwd_new", "fwd_old", "bloom", "inbox_counts"):
+    for key in ("list_ids", "list_dists", "fwd_new", "fwd_old", "bloom", "offers", "inbox_counts", "rev_tables", "counts"):
         np.testing.assert_array_equal(rest[key], st[key], err_msg=key)
 
+    # finalize: the `degree` nearest entries of the whole list by (distance, id) (the sub-lists merged by distance)
     d_knn = hip.DeviceArray((num, degree), np.uint32)
     hip.nnd_finalize(num, dim, d_ss, d_sl, 2, degree, d_knn, None, ws.buf, ws.bytes)
     hip.synchronize()
     knn = d_knn.numpy()
-    valid = st["list_ids"][:, :degree] != INV
-    np.testing.assert_array_equal(knn[valid], (st["list_ids"][:, :degree] & ~np.uint32(OLD))[valid])
+    for node in range(num):
+        ent = sorted((int(np.float32(d).view(np.uint32)), int(v) & ~OLD) for v, d in zip(st["list_ids"][node], st["list_dists"][node]) if v != INV)
+        want = [e[1] for e in ent[:degree]]
+        assert knn[node, :len(want)].tolist() == want
     assert (knn < lim).all()
+
+
+def test_full_inbox_overflows_into_the_table(hip):
+    """A hub: far more offers for one node than its inbox holds.  Built by hand: every list samples the same two points,
+    so those receive offers from every join.  Whatever went to the inbox and whatever to the overflow table, the best 32
+    distinct offers are all there, and the merge finds them."""
+    num, dim, degree = 6000, 128, 32
+    rows = lowdim_data(num, dim, seed=9)
+    seg_start, seg_len = np.array([0], np.uint32), np.array([num], np.uint32)
+    d_rows = hip.DeviceArray.from_numpy(rows)
+    d_ss, d_sl = hip.DeviceArray.from_numpy(seg_start), hip.DeviceArray.from_numpy(seg_len)
+    ws = Workspace(hip, num, dim, degree)
+    args = (num, dim, d_ss, d_sl, 1, degree, ws.buf, ws.bytes)
+    hip.nnd_prepare(d_rows, num, dim, d_ss, d_sl, 1, degree, 1, ws.buf, ws.bytes)
+    hip.synchronize()
+    # every list's first two "new" samples become points 0 and 1 (the others stay random)
+    w = ws.buf.numpy()
+    fwd = w[ws.l.fwd_new // 4: ws.l.fwd_new // 4 + num * S].reshape(num, S)
+    fwd[2:, 0] = 0
+    fwd[2:, 1] = 1
+    for r in range(2, num):        # keep a list's samples distinct
+        for c in range(2, S):
+            if fwd[r, c] in (0, 1):
+                fwd[r, c] = 2 + (r + c) % (num - 2)
+    ws.buf.upload(w)
+    hip.nnd_local_join(*args)
+    hip.synchronize()
+    after = ws.read()
+    offers = model_join(dict(after, fwd_new=fwd), rows, 0, num)
+    assert len(offers[0]) > 4 * CAP and after["inbox_counts"][0] == len(offers[0])
+    assert len(table_slots(after["offers"][0])[0]) > 0
+    for t in (0, 1, 2, 500, 5999):
+        exp = sorted(set(offer_key(d, c) for d, c in offers.get(t, [])))
+        assert offers_held(after, t)[:S] == exp[:S], t
+    hip.nnd_merge(*args)
+    hip.synchronize()
+    merged = ws.read()
+    for node in (0, 1, 2, 500, 5999):
+        l_ids, l_d, fn, fo, words, _ = model_merge(after, node, ws.l.width, ws.l.bloom_sets)
+        np.testing.assert_array_equal(merged["list_ids"][node], l_ids)
+        np.testing.assert_array_equal(merged["list_dists"][node], l_d)
+        assert merged["fwd_new"][node, :len(fn)].tolist() == fn
+    assert (merged["offers"] == NO_OFFER).all() and (merged["inbox_counts"] == 0).all()
+    # the hub has announced a threshold; a second join of the same lists sends it only what lies below
+    thr = int(merged["offer_thr"][0])
+    assert thr == model_offer_threshold(after, 0) != INV
+    w = ws.buf.numpy()
+    w[ws.l.fwd_new // 4: ws.l.fwd_new // 4 + num * S] = fwd.reshape(-1)
+    w[ws.l.counts // 4: ws.l.counts // 4 + num * 4].reshape(num, 4)[:] = after["counts"]
+    ws.buf.upload(w)
+    hip.nnd_local_join(*args)
+    hip.synchronize()
+    again = ws.read()
+    below = sorted(offer_key(d, c) for d, c in offers[0] if offer_key(d, c) >> 32 < thr)
+    assert again["inbox_counts"][0] == len(below) < len(offers[0])
+    assert offers_held(again, 0)[:S] == sorted(set(below))[:S] == sorted(set(offer_key(d, c) for d, c in offers[0]))[:S]
+
+
+@pytest.mark.parametrize("degree", [32, 64])
+def test_small_partitions_hold_no_id_twice(hip, degree):
+    """Partitions with fewer points than list slots: the random start lists repeat ids (at distance FLT_MAX), and an offer
+    for an id the list holds is rejected whatever distance the held copy carries (insert_to_ordered_list,
+    nn_descent.cuh:916-943), so no list ever names a point twice."""
+    num, dim = 400, 128
+    rows = lowdim_data(num, dim, seed=31)
+    seg_len = np.array([40, 20, 70, 270], dtype=np.uint32)
+    seg_start = np.array([0, 40, 60, 130], dtype=np.uint32)
+    d_rows = hip.DeviceArray.from_numpy(rows)
+    d_ss, d_sl = hip.DeviceArray.from_numpy(seg_start), hip.DeviceArray.from_numpy(seg_len)
+    ws = Workspace(hip, num, dim, degree)
+    args = (num, dim, d_ss, d_sl, 4, degree, ws.buf, ws.bytes)
+    hip.nnd_prepare(d_rows, num, dim, d_ss, d_sl, 4, degree, 5, ws.buf, ws.bytes)
+    local = np.arange(num) - np.repeat(seg_start, seg_len)
+    limit = np.repeat(seg_len, seg_len)
+    for it in range(6):
+        hip.nnd_reverse_sample(*args)
+        hip.nnd_local_join(*args)
+        hip.nnd_merge(*args)
+        hip.synchronize()
+        st = ws.read()
+        for node in range(num):
+            row = st["list_ids"][node]
+            ids = (row[row != INV] & ~np.uint32(OLD)).tolist()
+            assert len(set(ids)) == len(ids), (it, node)
+            assert local[node] not in ids and all(i < limit[node] for i in ids)
+    d_knn = hip.DeviceArray((num, degree), np.uint32)
+    hip.nnd_finalize(num, dim, d_ss, d_sl, 4, degree, d_knn, None, ws.buf, ws.bytes)
+    hip.synchronize()
+    assert (d_knn.numpy() < limit[:, None]).all()

@@ -8,12 +8,12 @@ from different NN-descent runs, so the comparison is statistical:
   * search recall@10 at equal beam, mean over several NN-descent seeds on each side: GPU >= CPU - tolerance.
 On the mixture data the finished index depends strongly on which residual far edges the kNN graph still holds (an
 exact kNN graph has no edge between mixture components, so search only crosses components over edges NN-descent has
-not yet replaced).  At equal iteration counts the GPU's lists are somewhat further converged than the CPU
-restatement's (this case, 8 rounds: recall@32 0.948 against 0.923, recall@64 0.836 against 0.823; both reach 0.99 at 24
-rounds), so they hold fewer of those edges, and recall@10 varies from seed to seed with sigma 0.05 (beam 32) to 0.07
-(beam 128) on both sides: means over eight seeds 0.65 (GPU) and 0.67 (CPU) at beam 32, 0.78 and 0.83 at beam 128.
-Eight seeds and a tolerance of 0.12 on the mean keep this case from failing by chance while a broken stage (recall
-0.17 against 0.63 was one) still fails; elsewhere three seeds and 0.015, and 0.005 on the low-dimensional data.
+not yet replaced), and recall@10 varies from NN-descent seed to seed with sigma 0.04 (beam 32 and 128) on both sides,
+hence eight seeds a side for that case.  Both builds are deterministic for a seed, so the comparison is repeatable:
+this case, 8 rounds at k = 64 (three id-keyed sub-lists on both sides): graph recall@32 0.927 (GPU) / 0.923 (CPU),
+recall@64 0.826 / 0.823, mean recall@10 0.684 / 0.671 at beam 32 and 0.834 / 0.831 at beam 128.  Tolerance on the
+mean: 0.015 on the three benchmark-shaped cases, 0.005 on the low-dimensional data; graph recall two-sided within
+0.01 (a build that converges faster than the reference's algorithm is a different algorithm too).
 With the GPU's kNN graph as input, the later stages are deterministic and the finished graph must be bit-identical.
 """
 import numpy as np
@@ -52,7 +52,7 @@ def _graph_recall(D, knn, truth, k):
 
 CASES = [
     # name, generator, num, dim, partitions, graph degree, knn degree, NN-descent iterations, metric, queries
-    ("clipped-mixture-k64", "gmm_clipped", 20_000, 128, 4, 32, 64, 8, 0, 1000, 0.12),
+    ("clipped-mixture-k64", "gmm_clipped", 20_000, 128, 4, 32, 64, 8, 0, 1000, 0.015),
     ("normalised-mixture-cosine", "gmm_normalized", 20_000, 96, 4, 32, 32, 10, 1, 1000, 0.015),
     ("beta-960-degree64", "beta_scaled", 6_000, 960, 3, 64, 64, 8, 0, 300, 0.015),
     # data of low intrinsic dimension, where search recall does not hang on single edges: the 0.5-point bar applies
@@ -126,15 +126,13 @@ def test_pipeline_matches_cpu_pipeline(hip, name, gen, num, dim, parts, degree, 
     truth = _exact_knn_in_partitions(O, rdata, seg_start, seg_len, k_eval, metric)
     r_gpu, r_cpu = _graph_recall(D, knn_gpu, truth, k_eval), _graph_recall(D, knn_cpu, truth, k_eval)
     print("graph recall@%d gpu %.4f cpu %.4f" % (k_eval, r_gpu, r_cpu), flush=True)
-    assert r_gpu >= r_cpu - 0.005
+    assert r_gpu >= r_cpu - 0.005 and abs(r_gpu - r_cpu) <= 0.01
     if knn_degree > k_eval:
-        # The whole list, not only its better half.  Its tail is far from converged after 8 rounds (0.78-0.84 on both
-        # sides; the GPU build is 1-2 points ahead of the CPU restatement here, and 7 points ahead at recall@32 on the
-        # 960-d data: one list of 96 entries converges faster than three id-keyed segments of 32).
+        # The whole list, not only its better half.  Its tail is far from converged after 8 rounds (0.78-0.83 on both sides).
         truth_k = _exact_knn_in_partitions(O, rdata, seg_start, seg_len, knn_degree, metric)
         rk_gpu, rk_cpu = _graph_recall(D, knn_gpu, truth_k, knn_degree), _graph_recall(D, knn_cpu, truth_k, knn_degree)
         print("graph recall@%d gpu %.4f cpu %.4f" % (knn_degree, rk_gpu, rk_cpu), flush=True)
-        assert rk_gpu >= rk_cpu - 0.03
+        assert rk_gpu >= rk_cpu - 0.005 and abs(rk_gpu - rk_cpu) <= 0.01
 
     # ---- search recall@10 at equal beam, mean over the seeds; seed 0 of the GPU side runs on the GPU
     gt, _ = O.bruteforce_knn(data, queries, 10, metric)
