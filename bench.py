@@ -1,19 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the GLIDE hot path on one MI355X: index build seconds + graph recall@32, search QPS.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-navigable|cfg0] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg1|cfg1-navigable|cfg0|cfg2|cfg3|cfg4] [--no-cpu] [--headline-only]
 
 A "step" is one beam-search pass of the whole query batch (10 000 queries, top-10) over the finished index.
 Before the timed steps the index is built once on the GPU (partition -> NN-descent -> sub-graph build + boundary
 merge -> reverse edges -> refine) and its stage times, the kNN-graph recall@32 against exact neighbours and the
-recall@10 of the whole beam sweep are measured.  One JSON line is printed.
+recall@10 of the whole beam sweep (32 ... 512, the reference's range) are measured.  One JSON line is printed: the
+headline fields are those of the medium configuration (cfg1); the other single-GPU configurations of the benchmark
+(cfg0, cfg2, cfg3) and the same shapes on navigable data follow under "other_configs" / "navigable_variant", each with
+its build stages, graph recall, beam sweep, roofline of its timed search kernel and the CPU restatement's recall and
+throughput at the same beam.  cfg4 (50M rows staged from pinned host memory) has a run of its own: --workload cfg4.
 
 Everything on the product path goes through libglide_hip.so.  torch is imported only to compute exact ground
-truth on the GPU (a checker); the CPU oracle is used only for the cpu_baseline leg.
+truth on the GPU (a checker); the CPU oracle is used only for the cpu_baseline legs.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -22,14 +27,26 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+SWEEP_BEAMS = (32, 64, 128, 256, 512)       # the reference accepts beams up to 512 (kernel_config.cuh:41-60)
+NAMED_BEAMS = {"cfg1": (32, 64, 128, 256)}  # the medium configuration names its beams; 512 is swept there as an extra
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "search_kernels_hbm_traffic.md")
 
-# HBM bytes one launch of the timed kernel moves, measured with two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then
-# WRITE_SIZE, KiB per dispatch) and scaled by what the same counters report for copy_kernel moving exactly 1 GiB
-# (--copy-calibration: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Keyed by (workload, beam); other combinations report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("cfg1", 256): 6_383_100 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
-    ("cfg1-navigable", 32): 2_449_600 * 1024 * 2.0 + 1_250 * 1024 * 1.0,
-}
+
+def measured_traffic(workload, beam):
+    """HBM bytes one launch of the timed search kernel moves, from the committed counter summary: two `rocprofv3 --pmc` runs
+    of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for the
+    plain copy kernel of known size (--copy-calibration).  The table rows are `| workload | beam | FETCH_SIZE KiB |
+    WRITE_SIZE KiB | fetch scale | write scale |`.  A (workload, beam) the file does not hold reports null: the value is
+    an offline measurement, tied to the commit the file names, not something this run derives."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None
+    for m in re.finditer(r"^\|\s*([\w-]+)\s*\|\s*(\d+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|", text, re.M):
+        if m.group(1) == workload and int(m.group(2)) == beam:
+            return dict(bytes=float(m.group(3)) * 1024 * float(m.group(5)) + float(m.group(4)) * 1024 * float(m.group(6)),
+                        source="profiles/" + os.path.basename(TRAFFIC_PROFILE))
+    return None
 
 
 def parse():
@@ -37,11 +54,12 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg1-navigable", "cfg2", "cfg3"])
+    ap.add_argument("--workload", default="cfg1", choices=["cfg0", "cfg1", "cfg1-navigable", "cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--headline-only", action="store_true", help="cfg1 only: skip the other configurations and the navigable variant")
+    ap.add_argument("--cfg4-rows", type=int, default=50_000_000, help="rows of the cfg4 run (the named size is 50M)")
     ap.add_argument("--nnd-iterations", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--knn-only", action="store_true", help="partition + NN-descent kNN graph of the workload only (for kernel profiles)")
-    ap.add_argument("--no-navigable", action="store_true", help="skip the extra navigable-data variant")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel on 1 GiB x steps (yardstick for rocprofv3 byte counters) and exit")
     ap.add_argument("--partition-only", type=int, default=0, metavar="C",
@@ -152,7 +170,7 @@ def run_workload(args, workload, torch, want_cpu):
     d_q = capi.DeviceArray.from_numpy(queries)
     d_ids, d_dists = capi.DeviceArray((nq, top_k), np.uint32), capi.DeviceArray((nq, top_k), np.float32)
     sweep = []
-    for beam in (32, 64, 128, 256):
+    for beam in SWEEP_BEAMS:
         sp = G.make_search_parameter(beam, degree, top_k)
         cnt = capi.new_counters()
         index.search(sp, d_q, counters=cnt, out=(d_ids, d_dists))
@@ -165,8 +183,11 @@ def run_workload(args, workload, torch, want_cpu):
         alg = nq * dim * 4 + parts * dim * 4 + int(c[2]) * degree * 4 + int(c[1]) * dim * 4 + nq * top_k * 8
         sweep.append(dict(beam=beam, recall_at_10=rec, qps=r["QPS"], ms=r["search_time"] * 1e3, iterations_per_query=c[0] / nq,
                           rows_per_query=c[1] / nq, algorithmic_bytes=alg))
-    ok = [s for s in sweep if s["recall_at_10"] >= 0.95]
-    chosen = min(ok, key=lambda s: s["beam"]) if ok else sweep[-1]
+    # the metric's operating point: the smallest beam that reaches recall@10 0.95; where none does (see recall_target_met)
+    # the widest beam of the reference's range is timed instead and the line says so
+    named = [s for s in sweep if s["beam"] in NAMED_BEAMS.get(workload, SWEEP_BEAMS)]
+    ok = [s for s in named if s["recall_at_10"] >= 0.95]
+    chosen = min(ok, key=lambda s: s["beam"]) if ok else named[-1]
 
     # ---- timed steps at the chosen beam: HIP events on the launch stream, warm-up first
     sp = G.make_search_parameter(chosen["beam"], degree, top_k)
@@ -222,7 +243,8 @@ def run_workload(args, workload, torch, want_cpu):
         sweep=sweep, beam=chosen["beam"], recall_at_10=chosen["recall_at_10"], recall_target_met=bool(ok),
         qps=nq * args.steps / (wall_ms * 1e-3), ms_per_step=ms_per_step, kernel_ms=kernel_ms,
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-                      traffic=MEASURED_TRAFFIC_BYTES.get((workload, chosen["beam"])),
+                      traffic=(measured_traffic(workload, chosen["beam"]) or {}).get("bytes"),
+                      traffic_source=(measured_traffic(workload, chosen["beam"]) or {}).get("source"),
                       kernel="%s<%d,%d,%d>" % ("search_kernel_dense" if 128 < chosen["beam"] <= 256 and degree <= 128 and dim <= 512 else "search_kernel",
                                                64 if degree <= 64 else 128 if degree <= 128 else 256,
                                                64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256 if chosen["beam"] <= 256 else 512,
@@ -230,12 +252,15 @@ def run_workload(args, workload, torch, want_cpu):
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )
 
-    if want_cpu:
+    if want_cpu == "full":
         out["cpu_baseline"] = cpu_baseline(data, queries, graph, d_cent.numpy(), index.d_start_points.numpy(), sp, top_k, gt, metric)
+    elif want_cpu:
+        out["cpu_baseline"] = cpu_baseline(data, queries, graph, d_cent.numpy(), index.d_start_points.numpy(), sp, top_k, gt, metric,
+                                           search_only=True, max_queries=500)
     return out
 
 
-def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt, metric=0):
+def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt, metric=0, search_only=False, max_queries=10_000):
     """The CPU restatement of the reference algorithm, timed on this box's host cores on a bounded sample."""
     import numpy as np
     from glide_amd import datasets as D
@@ -246,11 +271,15 @@ def cpu_baseline(data, queries, graph, centroids, start_points, sp, top_k, gt, m
     except Exception:
         pass
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    nq = min(queries.shape[0], 10_000)
+    nq = min(queries.shape[0], max_queries)
     t = time.time()
     ids, _, _ = O.search(data, graph, centroids, start_points, queries[:nq], top_k, sp.beam, sp.max_iterations, sp.min_iterations,
                          sp.hash_bit, sp.hash_reset_interval, metric, threads=cores)
     search_s = time.time() - t
+    if search_only:
+        return dict(value=nq / search_s, unit="queries/s", cores=cores, kind="port",
+                    sample="beam search of the first %d queries (same index, beam %d) with the CPU restatement, %d threads" % (nq, sp.beam, cores),
+                    recall_at_10=D.recall(ids, gt[:nq], top_k))
     # NN-descent build of one partition-sized sample (1M / 16 points) with the same degree / 10 iterations
     n_s = min(62_500, data.shape[0])
     t = time.time()
@@ -329,10 +358,16 @@ def main():
         G.build_nnd(nn, d_re, h_start, h_len, res, stats=True)
         print(json.dumps({"stage": "NN-descent kNN graph", "workload": desc, "rows": int(h_len.sum()), "dim": dim, "k": knn_degree,
                           "iterations_allowed": nn.max_iterations, "knn_sec": res["knn_time"], "offers": res["nnd_stats"][0],
-                          "offers_beyond_inbox": res["nnd_stats"][1]}))
+                          "offers_turned_away_by_overflow_tables": res["nnd_stats"][1]}))
         return
 
-    main_res = run_workload(args, args.workload, torch, want_cpu=not args.no_cpu)
+    if args.workload == "cfg4":
+        from glide_amd import large_bench
+        print(json.dumps(large_bench.run(args, info), default=float))
+        return
+
+    main_res = run_workload(args, args.workload, torch, want_cpu=False if args.no_cpu else "full")
+    met = main_res["recall_target_met"]
     line = {
         "metric": "search QPS at recall@10 >= 0.95 (index build sec and graph recall@32 alongside), 1 MI355X",
         "value": main_res["qps"], "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -342,16 +377,29 @@ def main():
                    "build_beam": 64, "refine_beam": 128, "relaxant": 1.05, "boundary_factor": 1.04, "sample_factor": 0.01,
                    "nnd_iterations": main_res["nnd_iterations"], "nnd_termination_threshold": 1e-4},
         "device": info["name"],
+        # `value` is the throughput of the timed steps.  It is the metric's figure only where recall_target_met is true;
+        # otherwise no beam of the reference's range reaches recall@10 0.95 on this workload (the CPU restatement of the
+        # reference algorithm reaches the same recall: cpu_baseline.recall_at_10) and the steps ran at the widest beam.
+        "value_is_at_recall_target": met,
+        "qps_at_recall_target": main_res["qps"] if met else None,
+        "qps_at_max_beam": None if met else main_res["qps"],
     }
     for k in ("build_sec", "build_stages", "graph_recall_at_32", "graph_recall_at_32_global", "recall_at_10", "recall_target_met",
               "empty_slots_fraction", "sweep", "kernel_ms", "nnd_offers", "nnd_offers_dropped", "stage_rooflines", "roofline"):
         line[k] = main_res[k]
     if "cpu_baseline" in main_res:
         line["cpu_baseline"] = main_res["cpu_baseline"]
-    if args.workload == "cfg1" and not args.no_navigable:
-        nav = run_workload(args, "cfg1-navigable", torch, want_cpu=False)
-        line["navigable_variant"] = {k: nav[k] for k in ("workload", "build_sec", "build_stages", "graph_recall_at_32", "beam", "recall_at_10",
-                                                         "recall_target_met", "qps", "kernel_ms", "sweep", "stage_rooflines", "roofline")}
+    if args.workload == "cfg1" and not args.headline_only:
+        keys = ("workload", "build_sec", "build_stages", "graph_recall_at_32", "graph_recall_at_32_global", "empty_slots_fraction", "beam", "recall_at_10",
+                "recall_target_met", "qps", "kernel_ms", "sweep", "stage_rooflines", "roofline", "cpu_baseline")
+        nav = run_workload(args, "cfg1-navigable", torch, want_cpu=not args.no_cpu)
+        line["navigable_variant"] = {k: nav[k] for k in keys if k in nav}
+        line["other_configs"] = {}
+        for name in ("cfg0", "cfg2", "cfg3"):
+            t0 = time.time()
+            res = run_workload(args, name, torch, want_cpu=not args.no_cpu)
+            line["other_configs"][name] = {k: res[k] for k in keys if k in res}
+            line["other_configs"][name]["wall_sec"] = time.time() - t0
     print(json.dumps(line, default=float))
 
 

@@ -148,6 +148,12 @@ int go_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_t dim, 
 int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
                     const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
                     float termination_threshold, uint32_t seed, int32_t *knn_graph, int threads);
+/* The same build with the host loop as the reference ships it (length passed as end, partition-local id compared with the
+ * global row index, no merge across sub-lists before truncation; nn_descent.cuh:1276-1283, :1117, :1376-1402).  Only
+ * for quoting what the shipped executable would score; nothing is held to it. */
+int go_nnd_build_shipped(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                         const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
+                         float termination_threshold, uint32_t seed, int32_t *knn_graph, int threads);
 
 /* exact kNN by brute force (ties by smaller id); squared L2 ranking, reported per metric */
 void go_bruteforce_knn(const float *data, uint32_t num, uint32_t dim, const float *queries, uint32_t query_num,

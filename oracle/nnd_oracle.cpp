@@ -4,8 +4,9 @@
 // every partition is updated in every iteration until max_iterations or until its own update counter falls below the
 // termination limit (go_nnd_build_ex; go_nnd_build runs the fixed count).  The reference's
 // own host loop stops updating partitions >= 1 after two rounds (it passes a length where an end is
-// expected, nn_descent.cuh:1276-1279 vs :1129-1135); that behaviour is not reproduced.
-// Bit-level parity is unpinned (the reference is unseeded and racy); tests check graph recall.
+// expected, nn_descent.cuh:1276-1279 vs :1129-1135).  go_nnd_build_shipped restates that loop as it is written, so
+// that what the shipped executable would score can be quoted next to the intended algorithm; nothing is compared
+// against it.  Bit-level parity is unpinned (the reference is unseeded and racy); tests check graph recall.
 #include "glide_oracle.h"
 
 #include <algorithm>
@@ -239,15 +240,19 @@ void local_join(Partition &P, uint32_t L, std::vector<float> &xn, std::vector<fl
 
 // update_graph nn_descent.cuh:1106-1126; returns the update counter: insertions on rows whose index in the whole
 // build (row_index_base + i) is a multiple of counter_interval = 100 (:1123)
-int64_t update_lists(Partition &P, const std::vector<int> &src_ids, const std::vector<float> &src_dists, uint32_t row_index_base) {
+// `rows` limits the update to local rows [0, rows); `as_shipped` compares the (partition-local) neighbour id with the row's
+// index in the whole build, as update_graph :1117 / update_segment_graph :1139 do, instead of with its local index.
+int64_t update_lists(Partition &P, const std::vector<int> &src_ids, const std::vector<float> &src_dists, uint32_t row_index_base,
+                     uint32_t rows = 0xffffffffu, bool as_shipped = false) {
     int64_t counter = 0;
+    const int64_t end = std::min<int64_t>(P.n, rows);
 #pragma omp parallel for schedule(static) reduction(+ : counter)
-    for (int64_t i = 0; i < static_cast<int64_t>(P.n); i++) {
+    for (int64_t i = 0; i < end; i++) {
         for (uint32_t j = 0; j < kSeg; j++) {
             int nid = src_ids[static_cast<size_t>(i) * kSeg + j];
             float d = src_dists[static_cast<size_t>(i) * kSeg + j];
             if (d == FLT_MAX) break;
-            if (static_cast<uint32_t>(id_of(nid)) == static_cast<uint32_t>(i)) continue;
+            if (static_cast<uint32_t>(id_of(nid)) == (as_shipped ? row_index_base + static_cast<uint32_t>(i) : static_cast<uint32_t>(i))) continue;
             uint32_t sub = static_cast<uint32_t>(id_of(nid)) % P.num_sub;
             uint32_t pos = insert_ordered(P.lists.data() + static_cast<size_t>(i) * P.W + sub * kSeg,
                                           P.ldists.data() + static_cast<size_t>(i) * P.W + sub * kSeg, kSeg, nid, d);
@@ -257,8 +262,13 @@ int64_t update_lists(Partition &P, const std::vector<int> &src_ids, const std::v
     return counter;
 }
 
+// shipped != nullptr: the host loop as the reference ships it (GNND::build, nn_descent.cuh:1289-1402).
+struct Shipped {
+    uint32_t break_iteration;   // the iteration after whose joins every partition was marked converged (loop :1344-1351); iterations if never
+    uint32_t last_join;         // out: the iteration of this partition's last join
+};
 void build_partition(const float *data, const float *norms_in, uint32_t n, uint32_t dim, uint32_t K, uint32_t iterations, uint32_t seed,
-                     int32_t *out /* n x K local ids */, uint32_t row_index_base, float termination_limit) {
+                     int32_t *out /* n x K local ids */, uint32_t row_index_base, float termination_limit, Shipped *shipped = nullptr) {
     Partition P;
     P.n = n;
     P.dim = dim;
@@ -305,11 +315,16 @@ void build_partition(const float *data, const float *norms_in, uint32_t n, uint3
     // Termination (update_and_sample :1270-1284, loop :1305-1308): when the counter of a merge falls below the limit the
     // partition is marked; the join of that iteration is already running and still completes, later iterations skip it.
     bool converged = false;
+    // As shipped, update_segment_graph receives the partition's length where it expects the end of its row range
+    // (:1276-1279 against :1129-1135): rows [start, length) of the whole build are updated, i.e. the first
+    // length - start rows of the partition, none at all once start >= length.
+    const uint32_t shipped_rows = shipped ? (n > row_index_base ? n - row_index_base : 0u) : 0xffffffffu;
     for (uint32_t it = 0; it < iterations && !converged; it++) {
+        if (shipped) shipped->last_join = it;
         cur_old = P.fwd_old;            // upload of h_graph_old / list sizes (:1290-1302)
         n_cur_old = P.n_fwd_old;
         if (it > 0) {                   // update_and_sample (:1270-1284)
-            const int64_t counter = update_lists(P, host_ids, host_dists, row_index_base);
+            const int64_t counter = update_lists(P, host_ids, host_dists, row_index_base, shipped_rows, shipped != nullptr);
             if (static_cast<float>(counter) < termination_limit) converged = true;
         }
         sample_lists(P, false);
@@ -328,6 +343,9 @@ void build_partition(const float *data, const float *norms_in, uint32_t n, uint3
         }
         P.fwd_old = next_old;
         P.n_fwd_old = n_next_old;
+        // As shipped, the loop is left before the download once every partition is marked (:1344-1351): the results of the
+        // joins of that iteration are never seen by the host.
+        if (shipped && it >= shipped->break_iteration) break;
         host_ids = P.dev_ids;           // download (:1353-1361)
         host_dists = P.dev_dists;
         // new samples = downloaded entries not yet seen by the Bloom filter (sample_graph_new :973-1001)
@@ -346,7 +364,21 @@ void build_partition(const float *data, const float *norms_in, uint32_t n, uint3
             P.n_fwd_new[i] = c;
         }
     }
-    update_lists(P, host_ids, host_dists, row_index_base);  // nn_descent.cuh:1368
+    update_lists(P, host_ids, host_dists, row_index_base, 0xffffffffu, shipped != nullptr);  // nn_descent.cuh:1368: every row, the last download
+    if (shipped) {
+        // shrink as shipped (:1376-1402): the first K columns of the row as stored, sub-list after sub-list, no sort across
+        // sub-lists -- for K > 32 no id of the last sub-list (id % num_sub == num_sub - 1) is ever returned
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < static_cast<int64_t>(n); i++) {
+            for (uint32_t j = 0; j < K; j++) {
+                const uint32_t idx = (row_index_base + static_cast<uint32_t>(i)) * P.W + j;
+                const uint32_t id = static_cast<uint32_t>(id_of(P.lists[static_cast<size_t>(i) * P.W + j]));
+                out[static_cast<size_t>(i) * K + j] = id < n ? static_cast<int>(id) : static_cast<int>(go_xorshift32(idx) % n);
+            }
+        }
+        for (auto &l : P.locks) omp_destroy_lock(&l);
+        return;
+    }
 
     // shrink nn_descent.cuh:1376-1402.  For K > 32 the reference copies whole sub-lists in storage order and
     // therefore never returns ids with id % num_sub == num_sub-1; here sub-lists are merged by distance first.
@@ -407,4 +439,45 @@ extern "C" int go_nnd_build(const float *reorder_data, uint32_t reorder_num, uin
                             int threads) {
     return go_nnd_build_ex(reorder_data, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, iterations, 0.0f,
                            seed, knn_graph, threads);
+}
+
+// The NN-descent build as the reference ships it: partitions whose first row index is not below their length are never
+// updated between rounds, count no insertions, are marked converged after the first update step and get two rounds of
+// joins; the partition-local id is compared with the row's index in the whole build; the sub-lists are not merged before
+// truncation.  termination_threshold as in NNDescentParameter (1e-4).  Two passes: the first finds the iteration at which
+// each partition is marked, the second knows when the loop was left.
+extern "C" int go_nnd_build_shipped(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                                    const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
+                                    float termination_threshold, uint32_t seed, int32_t *knn_graph, int threads) {
+#ifdef _OPENMP
+    if (threads > 0) omp_set_num_threads(threads);
+#endif
+    if (knn_degree == 0 || knn_degree > 128) return -1;
+    std::vector<float> half(static_cast<size_t>(reorder_num) * dim), norms(reorder_num);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < static_cast<int64_t>(reorder_num); i++) {
+        float acc = 0.0f;
+        for (uint32_t t = 0; t < dim; t++) {
+            float v = reorder_data[static_cast<size_t>(i) * dim + t];
+            acc += v * v;
+            half[static_cast<size_t>(i) * dim + t] = round_half(v);
+        }
+        norms[i] = acc;
+    }
+    const float limit = termination_threshold * static_cast<float>(reorder_num) * static_cast<float>(dim) / 100.0f;
+    uint32_t break_iteration = 0;
+    for (int pass = 0; pass < 2; pass++) {
+        for (uint32_t s = 0; s < segment_num; s++) {
+            uint32_t start = segment_starts[s], len = segment_lengths[s];
+            if (len == 0) continue;
+            if (start + len > reorder_num) return -2;
+            Shipped sh{pass == 0 ? iterations : break_iteration, 0};
+            build_partition(half.data() + static_cast<size_t>(start) * dim, norms.data() + start, len, dim, knn_degree, iterations, seed,
+                            knn_graph + static_cast<size_t>(start) * knn_degree, start, limit, &sh);
+            if (pass == 0) break_iteration = std::max(break_iteration, sh.last_join);
+        }
+        // the loop runs all its iterations unless every partition was marked before the last one
+        if (pass == 0 && break_iteration + 1 >= iterations) break_iteration = iterations;
+    }
+    return 0;
 }

@@ -307,11 +307,13 @@ def refine_segment(seg_data, graph, start_point, sp, relaxant, metric=EUCLIDEAN,
     return g, st.as_dict()
 
 
-def nnd_build(reorder_data, seg_start, seg_len, knn_degree, iterations, seed=0, threads=0, termination_threshold=0.0):
-    """termination_threshold = 0 runs exactly `iterations` rounds; the reference's default is 1e-4 (params.cuh:21)."""
+def nnd_build(reorder_data, seg_start, seg_len, knn_degree, iterations, seed=0, threads=0, termination_threshold=0.0, shipped_loop=False):
+    """termination_threshold = 0 runs exactly `iterations` rounds; the reference's default is 1e-4 (params.cuh:21).
+    shipped_loop: the host loop as the reference ships it (partitions whose first row is not below their length get two
+    rounds, no merge across sub-lists) instead of the intended algorithm."""
     reorder_data, seg_start, seg_len = _f32(reorder_data), _u32(seg_start), _u32(seg_len)
     out = np.empty((reorder_data.shape[0], knn_degree), dtype=np.int32)
-    rc = lib().go_nnd_build_ex(_p(reorder_data), u32(reorder_data.shape[0]), u32(reorder_data.shape[1]), _p(seg_start),
+    rc = (lib().go_nnd_build_shipped if shipped_loop else lib().go_nnd_build_ex)(_p(reorder_data), u32(reorder_data.shape[0]), u32(reorder_data.shape[1]), _p(seg_start),
                                _p(seg_len), u32(seg_start.size), u32(knn_degree), u32(iterations),
                                C.c_float(termination_threshold), u32(seed), _p(out), C.c_int(threads))
     if rc != 0:

@@ -83,12 +83,32 @@ def test_cli_usage_error():
     assert r.returncode != 0 and "data_file" in r.stdout      # exit(-1) on a bad argument count, like the reference
 
 
-def test_large_pipeline_cli(tmp_path):
+LARGE_CASES = [
+    # name, rows, partitions, boundary factor of the merged build, least recall@10 the searches must reach
+    ("low-dimensional", 9003, 5, 1.04, 0.9),          # rows: not a multiple of the 10 preprocessing batches
+    # the large configuration of the benchmark at a size the oracle covers: the clipped 64-component mixture, 64 partitions
+    # (more than 32 centroids: the wider centroid buckets of partitioning, partition selection and query grouping), boundary
+    # copies at the factor the 50M run uses.  Recall on this data is low for the reference algorithm itself; what is
+    # held here is that every stage equals the oracle's.
+    ("mixture-64-partitions", 60_000, 64, 1.002, 0.0),
+]
+
+
+def _large_data(name, n, nq):
+    from glide_amd import datasets as D
+    if name == "low-dimensional":
+        return lowdim_data(n, 128, seed=51), lowdim_data(nq, 128, seed=52)
+    return D.gmm_clipped(n, 128, seed=1234), D.gmm_clipped(nq, 128, seed=4321)
+
+
+@pytest.mark.parametrize("name,n,c,bf,least_recall", LARGE_CASES, ids=[x[0] for x in LARGE_CASES])
+def test_large_pipeline_cli(tmp_path, name, n, c, bf, least_recall):
     """large_* executables: host-resident data staged partition by partition; every stage checked against the oracle."""
     from glide_amd import datasets as D
     from oracle import oracle as O
-    n, dim, nq, c = 9003, 128, 200, 5          # not a multiple of the 10 preprocessing batches
-    data, queries = lowdim_data(n, dim, seed=51), lowdim_data(nq, dim, seed=52)
+    dim, nq = 128, 200
+    data, queries = _large_data(name, n, nq)
+    print("case", name, n, c, flush=True)
     truth, _ = O.bruteforce_knn(data, queries, 100)
     f = lambda name: str(tmp_path / name)
     D.write_fbin(f("base.fbin"), data)
@@ -114,7 +134,8 @@ def test_large_pipeline_cli(tmp_path):
     assert knn.shape == (n, 32)
     for s, l in zip(starts.tolist(), lengths.tolist()):
         assert (knn[s:s + l] < l).all()
-    s, l = int(starts[1]), int(lengths[1])
+    big = int(np.argmax(lengths))
+    s, l = int(starts[big]), int(lengths[big])
     gt, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + 200], 32, exclude_self=True)
     assert D.recall(knn[s:s + 200], gt, 32) >= 0.95
 
@@ -135,7 +156,7 @@ def test_large_pipeline_cli(tmp_path):
     spp = O.search_params(50, 32)
     for i, (s, l) in enumerate(zip(starts.tolist(), lengths.tolist())):
         O.search_sub(rdata[s:s + l], graph[s:s + l], mp[s:s + l], queries, seg_ids, i, int(sp[i]), 10, spp, e_ids, e_d)
-    assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= 0.9
+    assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= least_recall
     assert "index upload time" in out        # the index fits the GPU: uploaded once, partitions searched in place
     row = open(result).read().strip().splitlines()[1].split(",")
     assert len(row) == 8
@@ -146,15 +167,17 @@ def test_large_pipeline_cli(tmp_path):
     assert float(out2.split("total_recall:")[1].split()[0]) == recall
 
 
-def test_large_merged_pipeline_cli(tmp_path):
+@pytest.mark.parametrize("name,n,c,bf,least_recall", LARGE_CASES, ids=[x[0] for x in LARGE_CASES])
+def test_large_merged_pipeline_cli(tmp_path, name, n, c, bf, least_recall):
     """large_* executables on a partitioning with a boundary segment: partitions built one by one, placed into one
     graph, joined through the boundary copies, reverse edges and refinement over the whole graph
     (GLIDE_large::build_with_merge);
     the merged index is searched resident in device memory.  Every stage against the oracle."""
     from glide_amd import datasets as D
     from oracle import oracle as O
-    n, dim, nq, c = 9003, 128, 200, 5
-    data, queries = lowdim_data(n, dim, seed=61), lowdim_data(nq, dim, seed=62)
+    dim, nq = 128, 200
+    data, queries = _large_data(name, n, nq)
+    print("case", name, n, c, bf, flush=True)
     truth, _ = O.bruteforce_knn(data, queries, 100)
     f = lambda name: str(tmp_path / name)
     D.write_fbin(f("base.fbin"), data)
@@ -162,7 +185,7 @@ def test_large_merged_pipeline_cli(tmp_path):
     D.write_fbin(f("truth"), truth.astype(np.uint32))
     pre, knn_file, graph_base, result = f("pre"), f("knn"), f("graph"), f("result.csv")
 
-    run(os.path.join(BIN, "large_preprocess"), f("base.fbin"), pre, result, c, 0.05, "Euclidean", 1.04)
+    run(os.path.join(BIN, "large_preprocess"), f("base.fbin"), pre, result, c, 0.05, "Euclidean", bf)
     centroids = D.read_fbin(pre + ".centroid")
     starts, lengths = D.read_segment(pre + ".segment")
     mp = D.read_vector(pre + ".map")
@@ -171,9 +194,9 @@ def test_large_merged_pipeline_cli(tmp_path):
     assert starts.size == c + 1 and lengths[:c].sum() == n and starts[c] == n and copies > 0
     assert rdata.shape == (n + copies, dim) and mp.size == n + copies
     assert np.array_equal(rdata, data[mp]) and np.array_equal(np.sort(mp[:n]), np.arange(n))
-    e_idx, e_len, near = O.partition_assign(data, centroids, 1.04)
+    e_idx, e_len, near = O.partition_assign(data, centroids, bf)
     ratio = near[:, 1] / near[:, 0]
-    if (np.abs(ratio - 1) > 1e-4).all() and (np.abs(ratio - 1.04) > 1e-4).all():   # no point on a border or on the threshold
+    if (np.abs(ratio - 1) > 1e-4).all() and (np.abs(ratio - bf) > 1e-4).all():   # no point on a border or on the threshold
         assert np.array_equal(e_len, lengths)
         e_rdata, e_map = O.reorder(data, e_idx, O.segment_starts(e_len), n + copies)
         assert np.array_equal(e_map, mp) and np.array_equal(e_rdata, rdata)       # input order inside every segment
@@ -220,7 +243,7 @@ def test_large_merged_pipeline_cli(tmp_path):
     recall = float(out.split("total_recall:")[1].split()[0])
     e_ids, _, _ = O.search(rdata[:n], graph, centroids, entries, queries, 10, **O.search_params(64, 32))
     e_ids = np.where(e_ids < n, mp[np.minimum(e_ids, n - 1)], e_ids)
-    assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= 0.95
+    assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6 and recall >= (0.95 if least_recall else 0.0)
     row = open(result).read().strip().splitlines()[1].split(",")
     assert len(row) == 8
 
