@@ -30,6 +30,7 @@ HBM_PEAK_GBS = 8000.0
 SWEEP_BEAMS = (32, 64, 128, 256, 512)       # the reference accepts beams up to 512 (kernel_config.cuh:41-60)
 NAMED_BEAMS = {"cfg1": (32, 64, 128, 256)}  # the medium configuration names its beams; 512 is swept there as an extra
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "search_kernels_hbm_traffic.md")
+VALU_PROFILE = os.path.join(ROOT, "profiles", "build_refine_kernels_cfg1_counters.md")
 
 
 def measured_traffic(workload, beam):
@@ -49,6 +50,21 @@ def measured_traffic(workload, beam):
     return None
 
 
+def measured_valu(kernel, workload):
+    """(vector-ALU wave instructions one point costs in `kernel`, the chip's issue rate for that kind of instruction in
+    G wave instructions / s), from the committed counter summary of the build kernels (SQ_INSTS_VALU per launch over the
+    points of the launch; the rate is what --valu-calibration measures for compare + select).  Rows read
+    `| kernel | workload | instructions per point | yardstick |`; None for a pair the file does not hold."""
+    try:
+        text = open(VALU_PROFILE).read()
+    except OSError:
+        return None
+    for m in re.finditer(r"^\|\s*(\w+)\s*\|\s*([\w-]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*$", text, re.M):
+        if m.group(1) == kernel and m.group(2) == workload:
+            return float(m.group(3)), float(m.group(4))
+    return None
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -62,6 +78,8 @@ def parse():
     ap.add_argument("--knn-only", action="store_true", help="partition + NN-descent kNN graph of the workload only (for kernel profiles)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel on 1 GiB x steps (yardstick for rocprofv3 byte counters) and exit")
+    ap.add_argument("--valu-calibration", action="store_true",
+                    help="only run the register-only multiply-add kernel (yardstick for the vector-ALU issue rate) and exit")
     ap.add_argument("--partition-only", type=int, default=0, metavar="C",
                     help="only time partition assignment of 1M x 128 rows against C centroids (fp32 matrix-core tile) and exit")
     return ap.parse_args()
@@ -216,8 +234,22 @@ def run_workload(args, workload, torch, want_cpu):
     def hbm_stage(seconds, nbytes):
         gbs = nbytes / seconds / 1e9 if seconds > 0 else 0.0
         out = dict(bound="hbm", seconds=seconds, algorithmic_bytes=int(nbytes), achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS)
-        if gbs > HBM_PEAK_GBS:   # rows are scored again and again inside one partition (32 MB at cfg1): most gathers hit L2 / the memory-side cache
-            out["note"] = "algorithmic bytes exceed what HBM can deliver: the stage is served from cache, see the FETCH_SIZE counters"
+        return out
+
+    def valu_stage(seconds, nbytes, kernel, points):
+        """The per-point graph kernels score rows that sit in L2 (hit rate 0.96 in the counters) and spend their time
+        issuing vector instructions (sorting networks, cross-lane sums, distances): their ceiling is the vector-ALU
+        issue rate, and the bytes their algorithm names, which one partition's cache serves many times over, are
+        reported beside it without a fraction."""
+        out = dict(bound="valu", seconds=seconds, kernel=kernel, points=int(points), unit="G wave instructions/s",
+                   algorithmic_bytes=int(nbytes), algorithmic_GBps=nbytes / seconds / 1e9 if seconds > 0 else 0.0)
+        m = measured_valu(kernel, workload)
+        if m and seconds > 0:
+            out.update(instructions_per_point=m[0], achieved=m[0] * points / seconds / 1e9, peak=m[1], frac=m[0] * points / seconds / 1e9 / m[1],
+                       source="profiles/" + os.path.basename(VALU_PROFILE))
+        else:
+            out.update(instructions_per_point=None, achieved=None, peak=None, frac=None,
+                       note="no SQ_INSTS_VALU count committed for this kernel on this workload")
         return out
 
     stage_rooflines = {}
@@ -227,11 +259,13 @@ def run_workload(args, workload, torch, want_cpu):
     stage_rooflines["reorder"] = hbm_stage(det["reorder"], (num + reorder_rows) * dim * 4)
     if "build_counters" in res:
         _, rows, grows = res["build_counters"]
-        stage_rooflines["subgraph+boundary"] = hbm_stage(det["subgraph"] + det["boundary"],
-                                                         reorder_rows * dim * 4 + grows * knn_degree * 4 + rows * dim * 4 + reorder_rows * degree * 4)
+        stage_rooflines["subgraph+boundary"] = valu_stage(det["subgraph"] + det["boundary"],
+                                                          reorder_rows * dim * 4 + grows * knn_degree * 4 + rows * dim * 4 + reorder_rows * degree * 4,
+                                                          "build_kernel", num)   # the boundary launch adds 0.3% to the count
     if "refine_counters" in res:
         _, rows, grows = res["refine_counters"]
-        stage_rooflines["refine"] = hbm_stage(det["refine"], num * dim * 4 + 2 * num * degree * 4 + grows * degree * 4 + rows * dim * 4)
+        stage_rooflines["refine"] = valu_stage(det["refine"], num * dim * 4 + 2 * num * degree * 4 + grows * degree * 4 + rows * dim * 4,
+                                               "refine_kernel", num)
 
     out = dict(
         workload=desc, gen_sec=gen_s, build_sec=build_sec, stage_rooflines=stage_rooflines,
@@ -320,6 +354,23 @@ def main():
         ms = e0.elapsed_ms(e1) / args.steps
         print(json.dumps({"kernel": "copy_kernel", "bytes_read": nbytes, "bytes_written": nbytes, "ms": ms,
                           "GBps_read_plus_write": 2 * nbytes / ms / 1e6}))
+        return
+
+    if args.valu_calibration:
+        import numpy as np
+        out = capi.DeviceArray(4, np.float32)
+        rounds, res = 20000, {}
+        for mode, (name, per_step) in enumerate((("fused multiply-add", 1), ("integer add", 1), ("compare + select", 2), ("DPP move + add", 2))):
+            capi.valu_probe(mode, rounds, out)
+            e0, e1 = capi.Event(), capi.Event()
+            e0.record()
+            for _ in range(args.steps):
+                capi.valu_probe(mode, rounds, out)
+            e1.record()
+            ms = e0.elapsed_ms(e1) / args.steps
+            insts = 2048 * 4 * rounds * 16 * per_step
+            res[name] = {"wave_instructions": insts, "ms": ms, "G_wave_instructions_per_s": insts / ms / 1e6}
+        print(json.dumps({"kernel": "valu_probe_kernel", "compute_units": info["compute_units"], "modes": res}))
         return
 
     if args.partition_only:

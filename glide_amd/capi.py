@@ -389,6 +389,10 @@ def widen_u8(src, count, dst, stream=None):
     check(lib().glide_hip_widen_u8(_ptr(src), C.c_size_t(count), _ptr(dst), vp(stream)), "glide_hip_widen_u8")
 
 
+def valu_probe(mode, rounds, out, stream=None):
+    check(lib().glide_hip_valu_probe(C.c_int(mode), u32(rounds), _ptr(out), vp(stream)), "glide_hip_valu_probe")
+
+
 def copy_bytes(dst, src, nbytes, stream=None):
     check(lib().glide_hip_copy_bytes(_ptr(dst), _ptr(src), C.c_size_t(nbytes), vp(stream)), "glide_hip_copy_bytes")
 

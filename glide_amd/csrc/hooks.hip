@@ -17,6 +17,35 @@ __global__ __launch_bounds__(256) void widen_u8_kernel(const unsigned char* src,
     if (blockIdx.x == 0 && threadIdx.x < count % 4) dst[quads * 4 + threadIdx.x] = static_cast<float>(src[quads * 4 + threadIdx.x]);
 }
 
+// Yardstick for the vector-ALU issue rate (no counterpart in the reference): every lane runs `rounds` x 16 independent
+// register-only instructions, nothing else.  2048 workgroups of 256 threads keep eight wavefronts on every SIMD.
+// MODE 0: fused multiply-add; 1: 32-bit integer add; 2: compare + select (two instructions per step, the pair a
+// sorting network is made of); 3: cross-lane move (DPP quad permute) + add.
+template <int MODE>
+__global__ __launch_bounds__(256) void valu_probe_kernel(uint32_t rounds, float seed, float* out) {
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) v[i] = seed + static_cast<float>(threadIdx.x + i);
+    for (uint32_t r = 0; r < rounds; r++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if constexpr (MODE == 0) {
+                v[i] = fmaf(v[i], 1.0000001f, 0.5f);
+            } else if constexpr (MODE == 1) {
+                v[i] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v[i]) + 0x9E3779B1u);
+            } else if constexpr (MODE == 2) {
+                v[i] = v[i] < v[(i + 1) & 15] ? v[(i + 3) & 15] : v[i];
+            } else {
+                v[i] = __builtin_bit_cast(float, __builtin_bit_cast(int, lane_xor<1>(v[i])) + 1);
+            }
+        }
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) sum += v[i];
+    if (sum == 12345.678f) out[0] = sum;   // keeps the loop alive; practically never taken
+}
+
 __global__ __launch_bounds__(64) void distance_batch_kernel(const float* a, const float* b, uint32_t n, uint32_t dim,
                                                             int metric, float* out) {
     const int lane = lane_id();
@@ -145,6 +174,17 @@ int glide_hip_hashmap_insert_seq(uint32_t* table, uint32_t bitlen, const uint32_
     if (bitlen < 1 || bitlen > 13) return GLIDE_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(hashmap_seq_kernel, dim3(1), dim3(64), (size_t{1} << bitlen) * sizeof(uint32_t), as_stream(stream), table,
                        bitlen, keys, n, flags);
+    return launch_status();
+}
+
+int glide_hip_valu_probe(int mode, uint32_t rounds, float* out, void* stream) {
+    if (!out || mode < 0 || mode > 3) return GLIDE_ERR_BAD_ARGUMENT;
+    switch (mode) {
+        case 0: hipLaunchKernelGGL(valu_probe_kernel<0>, dim3(2048), dim3(256), 0, as_stream(stream), rounds, 1.0f, out); break;
+        case 1: hipLaunchKernelGGL(valu_probe_kernel<1>, dim3(2048), dim3(256), 0, as_stream(stream), rounds, 1.0f, out); break;
+        case 2: hipLaunchKernelGGL(valu_probe_kernel<2>, dim3(2048), dim3(256), 0, as_stream(stream), rounds, 1.0f, out); break;
+        default: hipLaunchKernelGGL(valu_probe_kernel<3>, dim3(2048), dim3(256), 0, as_stream(stream), rounds, 1.0f, out); break;
+    }
     return launch_status();
 }
 
