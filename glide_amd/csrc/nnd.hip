@@ -7,11 +7,11 @@
 // What is kept: fp16 rows with fp32 squared norms, <= 32 new + <= 32 old forward samples per node, reverse
 // samples capped at 32, a 64 x 64 distance tile per phase (new x new, new x old) computed on the matrix cores
 // with the norm-trick epilogue, and one offer per row / column (its nearest partner) per phase.
-// What is different: the kNN lists, flags, Bloom filters and samples never leave HBM.  Offers and reverse samples go to
-// plain per-node inboxes (one atomic add reserves a slot, no locks); whatever arrives after an inbox is full goes to an
-// overflow table that keeps the smallest keys by atomic minimum with displacement, so the smallest 32 keys of a node --
-// all that the reference's 32-wide device list and its 32 reverse samples ever use -- are the same whatever the order
-// of arrival, and a build is reproducible.  A merge kernel then applies the reference's rules: of a node's offers the
+// What is different: the kNN lists, flags, Bloom filters and samples never leave HBM.  An offer is one 64-bit atomic
+// minimum on a slot of its target's table (no locks, nothing returned); reverse samples go to plain per-node lists with
+// an overflow table that keeps the smallest sources.  What a node holds at the end of a round -- all that the
+// reference's 32-wide device list and its 32 reverse samples would be drawn from -- is the same whatever the order of
+// arrival, so a build is reproducible.  A merge kernel then applies the reference's rules: of a node's offers the
 // best 32 count, those not yet listed enter the sub-list id % num_sub (each sub-list keeps its 32 nearest), those the
 // Bloom filter has not seen are the next "new" samples.  All ids are partition-local.
 #include "common.hpp"
@@ -171,10 +171,10 @@ __global__ __launch_bounds__(256) void nnd_sample_kernel(uint32_t* list_ids, uin
     }
 }
 
-// ---- where offers and reverse samples arrive ---------------------------------------------------------------------
-// Both go first to a plain inbox of the receiving node: one atomic add reserves a slot, a store fills it.  As long as
-// an inbox does not fill up it holds every arrival, so the set it ends up with does not depend on the order of arrival;
-// the consumer sorts it.  What arrives after an inbox is full goes to the node's overflow table, which keeps the
+// ---- where reverse samples arrive -----------------------------------------------------------------------------------
+// They go first to a plain list of the receiving node: one atomic add reserves a slot, a store fills it.  As long as
+// a list does not fill up it holds every arrival, so the set it ends up with does not depend on the order of arrival;
+// the consumer sorts it.  What arrives after a list is full goes to the node's overflow table, which keeps the
 // smallest keys whatever the order of arrival:
 //   a table is made of buckets of 16 words, 15 slots and, last, the bucket's bound = the smallest key it has turned
 //   away (all ones: none yet); a key's bucket and first slot are hashes of its id.  A slot keeps the smaller of the key
@@ -182,31 +182,46 @@ __global__ __launch_bounds__(256) void nnd_sample_kernel(uint32_t* list_ids, uin
 //   Slot contents only ever decrease, so a key that has passed all 15 slots is larger than everything the bucket holds
 //   in the end and is dropped: a bucket ends with the 15 smallest distinct keys sent to it.  A key that is not smaller
 //   than the bound need not look further, which keeps a node that receives thousands of keys cheap.
-// The consumers only use the smallest 32 keys of inbox + table (the reference's 32-wide device list; its 32 reverse
-// samples).  One of those could only be missing if 15 smaller keys shared its bucket, i.e. if 16 of a node's 32
-// smallest keys fell into one of 16 buckets: with the smallest 32 of every node intact, the result is the same on
-// every run.
+// The join only uses the smallest 32 sources of list + table (the reference's 32 reverse samples).  One of those could
+// only be missing if 15 smaller keys shared its bucket, i.e. if 16 of a node's 32 smallest keys fell into one of 16
+// buckets: with the smallest 32 of every node intact, the result is the same on every run.
 // A node that receives thousands of keys round after round would make every sender wait for atomics on the same few
 // cache lines.  Such a node therefore announces a threshold for the next round, read by the senders before anything
-// else (a plain read of a read-only array): when its inbox overflowed, the 64th best distinct offer (the 56th smallest
-// source) of this round -- like the smallest 32, the smallest 64 of inbox + table do not depend on the order of arrival.  Keys that are not below the threshold stay away.  As long as at least 32 keys below it
-// arrive, the smallest 32 are what they would have been without it; the threshold is kept while arrivals stay
-// plentiful and withdrawn when they do not.  Everything it depends on is itself independent of arrival order.
+// else (a plain read of a read-only array): when its list overflowed, the 56th smallest source of this round -- like
+// the smallest 32, the smallest 56 of list + table do not depend on the order of arrival.  Sources that are not below
+// the threshold stay away.  As long as at least 32 sources below it arrive, the smallest 32 are what they would have
+// been without it; the threshold is kept while arrivals stay plentiful and withdrawn when they do not.  Nodes that are
+// offered thousands of candidates announce a distance threshold in the same way (kOfferCrowded below).
 constexpr uint32_t kBucketWords = 16, kBucketData = 15;
-constexpr uint32_t kInboxCap = 256;      // offers per node and round before the overflow table takes over
 constexpr uint32_t kRevCap = 64;         // reverse samples per node, kind and round before the overflow table takes over
-// Row strides of the inboxes and reverse lists, in entries.  Arrivals fill a row from its start, so with a power-of-two
-// stride (2 KB, 256 B) the busy front parts of all rows would sit on the same few memory channels.
-constexpr uint32_t kInboxStride = kInboxCap + 8, kRevStride = kRevCap + 8;
-constexpr uint32_t kOfferSlots = 256;    // overflow table per node: 16 buckets of (distance bits : candidate id) keys
+// Row stride of the reverse lists, in entries.  Arrivals fill a row from its start, so with a power-of-two stride
+// (256 B) the busy front parts of all rows would sit on the same few memory channels.
+constexpr uint32_t kRevStride = kRevCap + 8;
+// Offers of a round: per node a table of 256 (distance bits : candidate id) keys.  An offer goes to the slot its
+// candidate's id hashes to and stays if it is the smallest key that slot has seen this round (one 64-bit atomic
+// minimum without a return value).  Copies of one offer, found by several joins, are the same key and fall together;
+// two different candidates in one slot leave the nearer one.  What the table holds at the end of the round does not
+// depend on the order of arrival.
+constexpr uint32_t kOfferSlotsNarrow = 256, kOfferSlotsWide = 512;   // lists of one sub-list; of several (SLOTS below)
+// With several sub-lists an offer is sent to two slots (two hashes of its candidate) and is lost only if both hold a
+// nearer candidate: those lists are filled 32 offers a round, and each one that a fixed number of rounds loses shows in
+// the graph.  A single sub-list converges to the same graph either way (measured), and one atomic per offer is faster.
+__host__ __device__ constexpr uint32_t offer_slots_for(uint32_t width) { return width > 32 ? kOfferSlotsWide : kOfferSlotsNarrow; }
 constexpr uint32_t kRevSlots = 256;      // overflow table per node and kind: 16 buckets of source ids
 constexpr unsigned long long kNoOffer = ~0ull;
-constexpr uint32_t kOfferThrRank = 64;    // the threshold of a node whose inbox overflowed: its 64th best distinct offer
-constexpr uint32_t kRevThrRank = 56;      // ... and of a node whose reverse list overflowed: its 56th smallest source
-constexpr uint32_t kOfferKeepArrivals = 64, kRevKeepArrivals = 40;   // fewer arrivals than this withdraw a threshold
+constexpr uint32_t kOfferCrowdedEighths = 5;   // a node whose table is this full (in eighths) announces a threshold: ...
+constexpr uint32_t kOfferThrRank = 64;    // ... the distance of its 64th best offer
+constexpr uint32_t kOfferKeepHeld = 40;   // a threshold in force is withdrawn when fewer offers than this are held
+constexpr uint32_t kRevThrRank = 56;      // the threshold of a node whose reverse list overflowed: its 56th smallest source
+constexpr uint32_t kRevKeepArrivals = 40; // fewer arrivals than this withdraw it
 
 __device__ __forceinline__ uint32_t id_hash(uint32_t id) { return id * 0x9E3779B1u; }
 __device__ __forceinline__ uint32_t first_slot(uint32_t hash) { return __umulhi(hash * 0x85EBCA6Bu, kBucketData); }   // 0..14
+// Slot of a candidate in an offer table.  The salt changes with the round, so two candidates that share a slot in one
+// round do not share it in the next.
+__device__ __forceinline__ uint32_t offer_slot(uint32_t cand, uint32_t salt, uint32_t shift) { return id_hash(cand ^ salt) >> shift; }
+__device__ __forceinline__ uint32_t offer_slot2(uint32_t cand, uint32_t salt, uint32_t shift) { return ((cand ^ salt) * 0xC2B2AE35u) >> shift; }
+__device__ __forceinline__ uint32_t round_salt(uint32_t round) { return round * 0x85EBCA6Bu; }
 
 // One source id into a reverse overflow table (256 words).  The bound is read first: a table only comes into play for
 // nodes with many arrivals, and once its buckets are full nearly every further arrival ends here after one read.
@@ -263,10 +278,10 @@ struct JoinArgs {
     uint32_t* rev_tables;          // num x 2 x kRevSlots: where later arrivals went; emptied by the join that reads them
     uint32_t* rev_thr;             // num x 2: sources not below it stay away in the next scatter (all ones: none)
     uint32_t* counts;              // num x 4: forward new / old, reverse new / old arrivals (restarted by the join)
-    uint32_t* inbox_counts;        // num: offers that have arrived
-    unsigned long long* inbox;     // num x kInboxCap
-    unsigned long long* offers;    // num x kOfferSlots overflow tables
-    unsigned long long* stats;     // striped: [1] offers turned away by a full bucket of an overflow table (nullable)
+    unsigned long long* offers;    // num x offer_slots: the offer tables
+    uint32_t offer_slots, slot_shift, two_slots;   // slot_shift = 32 - log2(offer_slots)
+    const uint32_t* round;         // rounds completed so far (salt of the slot hash)
+    unsigned long long* stats;     // striped: [1] offers that stayed away because of their target's threshold (nullable)
     uint32_t num, dim_pad;
     Segments segs;
 };
@@ -506,24 +521,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         L.dist[i][j] = d;
     }
     __syncthreads();
-    // Every offer reserves a slot of its target's inbox; the atomic of phase 1 is in flight while phase 2 computes.
-    unsigned long long key[3] = {kNoOffer, kNoOffer, kNoOffer};
-    size_t row[3] = {0, 0, 0};
-    uint32_t slot[3] = {0, 0, 0};
-    bool live[3] = {false, false, false};
-    auto send = [&](int o, uint32_t target, uint32_t cand, float dist, uint32_t thr) {
+    // An offer is one atomic minimum on its slot of the target's table; nothing comes back, so the wave does not wait.
+    const uint32_t salt = round_salt(*a.round);
+    uint32_t declined = 0;
+    auto send = [&](uint32_t target, uint32_t cand, float dist, uint32_t thr) {
         if (cand == kInvalid || cand == target || cand >= seg_len || !(dist < FLT_MAX)) return;
-        if (__float_as_uint(dist) >= thr) return;   // the target has asked offers from this distance on to stay away
-        key[o] = (static_cast<unsigned long long>(__float_as_uint(dist)) << 32) | cand;
-        row[o] = static_cast<size_t>(seg_start) + target;
-        live[o] = true;
-        slot[o] = atomicAdd(&a.inbox_counts[row[o]], 1u);
+        if (__float_as_uint(dist) >= thr) {   // the target has asked offers from this distance on to stay away
+            declined++;
+            return;
+        }
+        const unsigned long long key = (static_cast<unsigned long long>(__float_as_uint(dist)) << 32) | cand;
+        unsigned long long* row = a.offers + (static_cast<size_t>(seg_start) + target) * a.offer_slots;
+        const uint32_t s1 = offer_slot(cand, salt, a.slot_shift), s2 = offer_slot2(cand, salt, a.slot_shift);
+        __hip_atomic_fetch_min(&row[s1], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (a.two_slots && s2 != s1) __hip_atomic_fetch_min(&row[s2], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
     {
         float best;
         uint32_t bj;
         line_argmin<true>(L.dist, line, part, best, bj);
-        if (part == 0 && line < n_new && bj != kInvalid) send(0, L.new_ids[line], L.new_ids[bj], best, L.new_thr[line]);
+        if (part == 0 && line < n_new && bj != kInvalid) send(L.new_ids[line], L.new_ids[bj], best, L.new_thr[line]);
     }
     if (n_old != 0) {
         // ---- phase 2: new x old (rows: new, columns: old)
@@ -542,80 +559,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
             uint32_t bj;
             const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
             line_argmin<true>(L.dist, line, part, best, bj);
-            if (part == 0 && line < n_new && bj != kInvalid) send(1, me, L.old_ids[bj], best, L.new_thr[line]);
+            if (part == 0 && line < n_new && bj != kInvalid) send(me, L.old_ids[bj], best, L.new_thr[line]);
         }
         {
             float best;
             uint32_t bi;
             const uint32_t me = line < n_old ? L.old_ids[line] : kInvalid;
             line_argmin<false>(L.dist, line, part, best, bi);
-            if (part == 0 && line < n_old && bi != kInvalid) send(2, me, L.new_ids[bi], best, L.old_thr[line]);
+            if (part == 0 && line < n_old && bi != kInvalid) send(me, L.new_ids[bi], best, L.old_thr[line]);
         }
     }
-    bool any = false;
-#pragma unroll
-    for (int o = 0; o < 3; o++) {
-        if (live[o] && slot[o] < kInboxCap) {
-            a.inbox[row[o] * kInboxStride + slot[o]] = key[o];
-            live[o] = false;
-        }
-        any |= live[o];
-    }
-    if (any) {
-        // The inbox of the target is full: the overflow table takes the offer (the up to three chains of a thread side by side).
-        unsigned long long* bucket[3];
-        unsigned long long seen[3], bound[3];
-        uint32_t at[3], dropped = 0;
-#pragma unroll
-        for (int o = 0; o < 3; o++) {
-            const uint32_t h = id_hash(static_cast<uint32_t>(key[o]));
-            bucket[o] = a.offers + row[o] * kOfferSlots + (h >> 28) * kBucketWords;
-            at[o] = first_slot(h);
-            // the bound first: once the buckets of a node that receives thousands of offers are full, nearly every
-            // further offer ends here after one read
-            bound[o] = live[o] ? __hip_atomic_load(&bucket[o][kBucketData], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : kNoOffer;
-        }
-#pragma unroll
-        for (int o = 0; o < 3; o++) {
-            if (live[o] && key[o] >= bound[o]) {   // the bucket has already turned a smaller key away
-                live[o] = false;
-                dropped++;
-            }
-            seen[o] = live[o] ? atomicMin(&bucket[o][at[o]], key[o]) : kNoOffer;
-        }
-#pragma unroll
-        for (int o = 0; o < 3; o++) {
-            if (live[o]) {
-                if (seen[o] == kNoOffer || seen[o] == key[o]) live[o] = false;     // settled, or a copy was there
-                else if (seen[o] > key[o]) key[o] = seen[o];                       // the displaced key carries on
-            }
-        }
-        for (uint32_t probe = 1; probe < kBucketData; probe++) {
-            if (!(live[0] || live[1] || live[2])) break;
-#pragma unroll
-            for (int o = 0; o < 3; o++) {
-                if (live[o]) {
-                    at[o] = at[o] + 1 == kBucketData ? 0 : at[o] + 1;
-                    seen[o] = atomicMin(&bucket[o][at[o]], key[o]);
-                }
-            }
-#pragma unroll
-            for (int o = 0; o < 3; o++) {
-                if (live[o]) {
-                    if (seen[o] == kNoOffer || seen[o] == key[o]) live[o] = false;
-                    else if (seen[o] > key[o]) key[o] = seen[o];
-                }
-            }
-        }
-#pragma unroll
-        for (int o = 0; o < 3; o++) {
-            if (live[o]) {   // it has met 15 smaller keys: the bucket is full of better offers
-                atomicMin(&bucket[o][kBucketData], key[o]);
-                dropped++;
-            }
-        }
-        if (dropped && a.stats) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(dropped));
-    }
+    if (declined && a.stats) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(declined));
 }
 
 // ---- merge ------------------------------------------------------------------------------------------------------
@@ -708,9 +662,7 @@ __device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, uint32_t
 struct MergeArgs {
     uint32_t* list_ids;
     float* list_dists;
-    uint32_t* inbox_counts;
-    const unsigned long long* inbox;
-    unsigned long long* offers;  // overflow tables
+    unsigned long long* offers;  // num x SLOTS offer tables: read and emptied
     uint32_t* bloom;
     uint32_t* fwd_new;
     uint32_t* fwd_old;
@@ -726,9 +678,10 @@ struct MergeArgs {
 };
 
 constexpr uint32_t kKnownBits = 9;   // 512-slot id set per wavefront: lists of up to 192 entries + 32 offers
+template <uint32_t SLOTS>
 struct MergeLds {
-    unsigned long long keys[4][kInboxCap];   // the node's offers as they arrived
-    unsigned long long best[4][2 * kOfferThrRank];   // the best 32 distinct ones (64 + 64 while inbox and overflow table are combined)
+    unsigned long long keys[4][SLOTS];   // the node's offers, gaps closed
+    unsigned long long best[4][kOfferThrRank];  // the best 32 of them (64 where a threshold is due)
     unsigned long long enter[4][kSamples];      // those that enter the list, as keys of the second sort
     uint32_t known[4][1u << kKnownBits];
     uint32_t filter[4][128];
@@ -774,7 +727,10 @@ __device__ __forceinline__ uint32_t best_offers(const unsigned long long* keys, 
     return total < N_OUT ? total : N_OUT;
 }
 
+template <uint32_t SLOTS>
 __device__ __forceinline__ uint32_t best_offers_sized(const unsigned long long* keys, uint32_t held, unsigned long long* best, int lane) {
+    if constexpr (SLOTS > 256)
+        if (held > 256) return best_offers<SLOTS>(keys, held, best, lane);
     if (held > 128) return best_offers<256>(keys, held, best, lane);
     if (held > 64) return best_offers<128>(keys, held, best, lane);
     if (held > 0) return best_offers<64>(keys, held, best, lane);
@@ -791,9 +747,9 @@ __device__ __forceinline__ uint32_t best_offers_sized(const unsigned long long* 
 //   sorted together with the list, and every sub-list keeps its 32 nearest;
 //   new samples = those of the best 32 that the Bloom filter has not seen; the ones entering the list are flagged old.
 // M2 = size of the second network >= width + 32.
-template <int M2>
+template <int M2, uint32_t SLOTS>
 __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
-    __shared__ MergeLds L;
+    __shared__ MergeLds<SLOTS> L;
     constexpr int NR = M2 / 64;
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
@@ -810,57 +766,53 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
     uint32_t* filter = L.filter[wave];
     uint32_t* flags = L.flags[wave];
     const uint32_t bloom_words = a.bloom_sets * 16;
-    const uint32_t arrived = a.inbox_counts[node];
     for (uint32_t w = lane; w < bloom_words; w += 64) filter[w] = a.bloom[static_cast<size_t>(node) * bloom_words + w];
     for (uint32_t i = lane; i < (1u << kKnownBits); i += 64) known[i] = kInvalid;
 
-    // ---- this round's offers: the inbox, four slots per lane
-    const uint32_t held = arrived < kInboxCap ? arrived : kInboxCap;
-    if (4u * lane < held) {
-        const unsigned long long* src = a.inbox + static_cast<size_t>(node) * kInboxStride + 4 * lane;
-        const uint4 lo = *reinterpret_cast<const uint4*>(src), hi = *reinterpret_cast<const uint4*>(src + 2);
-        *reinterpret_cast<uint4*>(keys + 4 * lane) = lo;
-        *reinterpret_cast<uint4*>(keys + 4 * lane + 2) = hi;
+    // ---- this round's offers: the node's table, four slots per lane and pass, emptied where something was found
+    uint32_t held;
+    {
+        unsigned long long* row = a.offers + static_cast<size_t>(node) * SLOTS;
+        constexpr int PASSES = SLOTS / 256;
+        unsigned long long o[PASSES][4];
+        uint32_t mine = 0;
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            unsigned long long* at = row + 256 * p + 4 * lane;
+            const uint4 lo = *reinterpret_cast<const uint4*>(at), hi = *reinterpret_cast<const uint4*>(at + 2);
+            o[p][0] = (static_cast<unsigned long long>(lo.y) << 32) | lo.x;
+            o[p][1] = (static_cast<unsigned long long>(lo.w) << 32) | lo.z;
+            o[p][2] = (static_cast<unsigned long long>(hi.y) << 32) | hi.x;
+            o[p][3] = (static_cast<unsigned long long>(hi.w) << 32) | hi.z;
+            if ((o[p][0] & o[p][1] & o[p][2] & o[p][3]) != kNoOffer) {
+                const uint4 empty = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
+                *reinterpret_cast<uint4*>(at) = empty;
+                *reinterpret_cast<uint4*>(at + 2) = empty;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) mine += o[p][j] != kNoOffer;
+        }
+        uint32_t at = wave_exclusive_scan(mine, held);
+#pragma unroll
+        for (int p = 0; p < PASSES; p++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (o[p][j] != kNoOffer) keys[at++] = o[p][j];
     }
     __builtin_amdgcn_wave_barrier();
     uint32_t n_best;
     uint32_t next_thr;
     const uint32_t in_force = __float_as_uint(a.norms[node].y);
-    if (arrived <= kInboxCap) {
-        n_best = best_offers_sized(keys, held, best, lane);
+    if (held < SLOTS / 8 * kOfferCrowdedEighths) {
+        n_best = best_offers_sized<SLOTS>(keys, held, best, lane);
         // a threshold that is in force stays while the node still receives plenty of offers and its best 32 are complete
-        next_thr = arrived >= kOfferKeepArrivals && n_best == kSamples ? in_force : kInvalid;
+        next_thr = held >= kOfferKeepHeld && n_best == kSamples ? in_force : kInvalid;
     } else {
-        // The inbox filled up and later offers went to the overflow table: the round's best distinct offers are those
-        // of the inbox's best 64 and the table's best 64.  The table is emptied (bounds included) where something was found.
-        const uint32_t n_inbox = best_offers<256, kOfferThrRank>(keys, held, best, lane);
-        unsigned long long* row = a.offers + static_cast<size_t>(node) * kOfferSlots;
-        const uint4 lo = *reinterpret_cast<const uint4*>(row + 4 * lane), hi = *reinterpret_cast<const uint4*>(row + 4 * lane + 2);
-        unsigned long long o[4] = {(static_cast<unsigned long long>(lo.y) << 32) | lo.x, (static_cast<unsigned long long>(lo.w) << 32) | lo.z,
-                                   (static_cast<unsigned long long>(hi.y) << 32) | hi.x, (static_cast<unsigned long long>(hi.w) << 32) | hi.z};
-        if ((o[0] & o[1] & o[2] & o[3]) != kNoOffer) {
-            const uint4 empty = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
-            *reinterpret_cast<uint4*>(row + 4 * lane) = empty;
-            *reinterpret_cast<uint4*>(row + 4 * lane + 2) = empty;
-        }
-        if ((lane & 3) == 3) o[3] = kNoOffer;   // word 15 of a bucket is its bound, not an offer
-        uint32_t mine = 0, in_table;
-#pragma unroll
-        for (int j = 0; j < 4; j++) mine += o[j] != kNoOffer;
-        uint32_t at = wave_exclusive_scan(mine, in_table);
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            if (o[j] != kNoOffer) keys[at++] = o[j];
-        __builtin_amdgcn_wave_barrier();
-        const uint32_t n_table = best_offers<256, kOfferThrRank>(keys, in_table, best + kOfferThrRank, lane);
-        // best[0 .. n_inbox) and best[64 .. 64 + n_table): close the gap, then once more through a 128-key network.
-        // The distance of the 64th best distinct offer of the round becomes the node's threshold for the next join (none if it has fewer).
-        if (static_cast<uint32_t>(lane) < n_table) keys[n_inbox + lane] = best[kOfferThrRank + lane];
-        if (static_cast<uint32_t>(lane) < n_inbox) keys[lane] = best[lane];
-        __builtin_amdgcn_wave_barrier();
-        const uint32_t n_union = best_offers<128, kOfferThrRank>(keys, n_inbox + n_table, best, lane);
-        n_best = n_union < kSamples ? n_union : kSamples;
-        next_thr = n_union == kOfferThrRank ? static_cast<uint32_t>(best[kOfferThrRank - 1] >> 32) : kInvalid;
+        // A crowded table: thousands of offers may have met here, and most of the round's cost for this node was their
+        // atomics on these few lines.  The distance of the 64th best offer becomes the node's threshold for the next join.
+        const uint32_t n64 = held > 256 ? best_offers<SLOTS, kOfferThrRank>(keys, held, best, lane) : best_offers<256, kOfferThrRank>(keys, held, best, lane);
+        n_best = n64 < kSamples ? n64 : kSamples;
+        next_thr = n64 == kOfferThrRank ? static_cast<uint32_t>(best[kOfferThrRank - 1] >> 32) : kInvalid;
     }
     if (lane == 0 && next_thr != in_force) a.norms[node].y = __uint_as_float(next_thr);
 
@@ -995,7 +947,6 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
     __builtin_amdgcn_wave_barrier();
     for (uint32_t w = lane; w < bloom_words; w += 64) a.bloom[static_cast<size_t>(node) * bloom_words + w] = filter[w];
     if (lane == 0) {
-        a.inbox_counts[node] = 0;
         a.counts[static_cast<size_t>(node) * 4 + 0] = total_new;
         a.counts[static_cast<size_t>(node) * 4 + 1] = total_old < kSamples ? total_old : kSamples;
         if (!a.rev_new) {   // with the scatter fused in, other wavefronts are adding to these two right now; the join clears them
@@ -1003,15 +954,16 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
             a.counts[static_cast<size_t>(node) * 4 + 3] = 0;
         }
         // striped over 1024 slots: one shared address would serialise every wavefront of the launch
-        if (a.stats && arrived) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u)], static_cast<unsigned long long>(arrived));
+        if (a.stats && held) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u)], static_cast<unsigned long long>(held));
     }
 }
 
 // Termination test of GNND::build's update_and_sample (nn_descent.cuh:1270-1284): a partition whose sampled update
 // count falls below termination_threshold * rows * dim / 100 (rows = all rows of the build, as in the reference) runs
 // one more round -- the reference has already started that round's join when the host notices -- and then rests.
-__global__ void nnd_converge_kernel(Segments segs, float limit) {
+__global__ void nnd_converge_kernel(Segments segs, float limit, uint32_t* round) {
     const uint32_t s = blockIdx.x * blockDim.x + threadIdx.x;
+    if (s == 0) round[0] += 1;
     if (s >= segs.count) return;
     const uint32_t state = segs.state[s];
     if (state == kLastRound) {
@@ -1094,8 +1046,8 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 constexpr uint32_t kMaxWidth = 192;   // six sub-lists: degrees up to 128 (width + 32 offers fit one 256-key network)
 
 struct NndLayout {
-    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts, inbox_counts, inbox, offers, bloom, stats,
-        seg_state, seg_updates, total;
+    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts, offers, bloom, stats, seg_state,
+        seg_updates, round, total;
     uint32_t width, dim_pad, bloom_sets;
 };
 NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
@@ -1118,13 +1070,12 @@ NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
     l.rev_tables = take(n * 2 * kRevSlots * 4);
     l.rev_thr = take(n * 8);
     l.counts = take(n * 16);
-    l.inbox_counts = take(n * 4);
-    l.inbox = take(n * kInboxStride * 8);
-    l.offers = take(n * kOfferSlots * 8);
+    l.offers = take(n * offer_slots_for(l.width) * 8);
     l.bloom = take(n * l.bloom_sets * 64);
     l.stats = take(1024 * 16);
     l.seg_state = take(kMaxSegments * 4);
     l.seg_updates = take(kMaxSegments * 4);
+    l.round = take(4);
     l.total = off;
     return l;
 }
@@ -1143,8 +1094,8 @@ struct NndCtx {
     float2* norms;
     uint32_t* list_ids;
     float* list_dists;
-    uint32_t *fwd_new, *fwd_old, *rev_new, *rev_old, *rev_tables, *rev_thr, *counts, *inbox_counts;
-    unsigned long long *inbox, *offers;
+    uint32_t *fwd_new, *fwd_old, *rev_new, *rev_old, *rev_tables, *rev_thr, *counts, *round;
+    unsigned long long* offers;
     uint32_t* bloom;
     unsigned long long* stats;
     Segments segs;
@@ -1178,11 +1129,10 @@ int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* s
     c.rev_tables = reinterpret_cast<uint32_t*>(w + c.l.rev_tables);
     c.rev_thr = reinterpret_cast<uint32_t*>(w + c.l.rev_thr);
     c.counts = reinterpret_cast<uint32_t*>(w + c.l.counts);
-    c.inbox_counts = reinterpret_cast<uint32_t*>(w + c.l.inbox_counts);
-    c.inbox = reinterpret_cast<unsigned long long*>(w + c.l.inbox);
     c.offers = reinterpret_cast<unsigned long long*>(w + c.l.offers);
     c.bloom = reinterpret_cast<uint32_t*>(w + c.l.bloom);
     c.stats = reinterpret_cast<unsigned long long*>(w + c.l.stats);
+    c.round = reinterpret_cast<uint32_t*>(w + c.l.round);
     c.segs = Segments{segment_starts, segment_lengths, segment_num, reinterpret_cast<uint32_t*>(w + c.l.seg_state),
                       reinterpret_cast<uint32_t*>(w + c.l.seg_updates)};
     c.n = reorder_num;
@@ -1195,14 +1145,12 @@ int nnd_prepare(const NndCtx& c, const float* data, uint32_t dim, uint32_t seed)
     if (rc != GLIDE_OK) return rc;
     rc = glide_hip_fill_u32(c.bloom, 0u, static_cast<size_t>(c.n) * c.l.bloom_sets * 16, c.s);
     if (rc != GLIDE_OK) return rc;
-    rc = glide_hip_fill_u32(c.segs.state, 0u, 2 * kMaxSegments, c.s);   // state and updates are adjacent
+    rc = glide_hip_fill_u32(c.segs.state, 0u, 2 * kMaxSegments + 1, c.s);   // state, updates and the round count are adjacent
     if (rc != GLIDE_OK) return rc;
-    // empty overflow tables (their bounds included: nothing turned away yet), empty inboxes
+    // empty overflow tables (their bounds included: nothing turned away yet), empty offer tables
     rc = glide_hip_fill_u32(c.rev_tables, kInvalid, (c.l.counts - c.l.rev_tables) / 4, c.s);
     if (rc != GLIDE_OK) return rc;
-    rc = glide_hip_fill_u32(c.inbox_counts, 0u, c.n, c.s);
-    if (rc != GLIDE_OK) return rc;
-    rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(c.offers), kInvalid, static_cast<size_t>(c.n) * kOfferSlots * 2, c.s);
+    rc = glide_hip_fill_u32(reinterpret_cast<uint32_t*>(c.offers), kInvalid, static_cast<size_t>(c.n) * offer_slots_for(c.l.width) * 2, c.s);
     if (rc != GLIDE_OK) return rc;
     hipLaunchKernelGGL(nnd_prepare_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, data, c.n, dim, c.l.dim_pad, c.half_rows, c.norms);
     hipLaunchKernelGGL(nnd_init_kernel, dim3(ceil_div(c.n * c.l.width, 256)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, c.segs, seed);
@@ -1220,8 +1168,8 @@ int nnd_reverse(const NndCtx& c) {
 int nnd_join(const NndCtx& c, bool with_stats) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
-    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.inbox_counts, c.inbox,
-                c.offers, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
+    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.offers, offer_slots_for(c.l.width),
+                offer_slots_for(c.l.width) == 512 ? 23u : 24u, c.l.width > 32 ? 1u : 0u, c.round, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
     hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja);
     return launch_status();
 }
@@ -1229,23 +1177,23 @@ int nnd_join(const NndCtx& c, bool with_stats) {
 // scatter_reverse: the new and old samples a node draws enter the reverse tables of their targets right away
 // (what the next round's nnd_reverse would do), while the sort of other nodes keeps the vector ALU busy
 int nnd_merge(const NndCtx& c, bool with_stats, bool scatter_reverse = false) {
-    MergeArgs ma{c.list_ids, c.list_dists, c.inbox_counts, c.inbox, c.offers, c.bloom, c.fwd_new, c.fwd_old, c.counts, with_stats ? c.stats : nullptr, c.segs,
+    MergeArgs ma{c.list_ids, c.list_dists, c.offers, c.bloom, c.fwd_new, c.fwd_old, c.counts, with_stats ? c.stats : nullptr, c.segs,
                  scatter_reverse ? c.rev_new : nullptr, scatter_reverse ? c.rev_old : nullptr, scatter_reverse ? c.rev_tables : nullptr, c.rev_thr, c.norms,
                  c.n, c.l.width, c.l.width / kSamples, c.l.bloom_sets};
     const uint32_t m = c.l.width + kSamples;
     if (m <= 64)
-        hipLaunchKernelGGL(nnd_merge_kernel<64>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
+        hipLaunchKernelGGL((nnd_merge_kernel<64, kOfferSlotsNarrow>), dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
     else if (m <= 128)
-        hipLaunchKernelGGL(nnd_merge_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
+        hipLaunchKernelGGL((nnd_merge_kernel<128, kOfferSlotsWide>), dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
     else
-        hipLaunchKernelGGL(nnd_merge_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
+        hipLaunchKernelGGL((nnd_merge_kernel<256, kOfferSlotsWide>), dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
     return launch_status();
 }
 
 int nnd_converge(const NndCtx& c, uint32_t dim, float termination_threshold) {
     // update_counter < termination_threshold * nrow * dim / counter_interval (nn_descent.cuh:1280), evaluated in float
     const float limit = termination_threshold * static_cast<float>(c.n) * static_cast<float>(dim) / static_cast<float>(kCounterInterval);
-    hipLaunchKernelGGL(nnd_converge_kernel, dim3(ceil_div(c.segs.count, 256)), dim3(256), 0, c.s, c.segs, limit);
+    hipLaunchKernelGGL(nnd_converge_kernel, dim3(ceil_div(c.segs.count, 256)), dim3(256), 0, c.s, c.segs, limit, c.round);
     return launch_status();
 }
 
@@ -1297,9 +1245,9 @@ int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree
     const NndLayout l = nnd_layout(reorder_num, dim, knn_degree);
     out->half_rows = l.half_rows; out->norms = l.norms; out->list_ids = l.list_ids; out->list_dists = l.list_dists;
     out->fwd_new = l.fwd_new; out->fwd_old = l.fwd_old; out->rev_new = l.rev_new; out->rev_old = l.rev_old; out->rev_tables = l.rev_tables; out->rev_thr = l.rev_thr;
-    out->counts = l.counts; out->inbox_counts = l.inbox_counts; out->inbox = l.inbox; out->offers = l.offers; out->bloom = l.bloom;
-    out->segment_state = l.seg_state; out->segment_updates = l.seg_updates; out->total = l.total;
-    out->width = l.width; out->reverse_cap = kRevCap; out->reverse_stride = kRevStride; out->inbox_cap = kInboxCap; out->inbox_stride = kInboxStride; out->offer_slots = kOfferSlots; out->reverse_slots = kRevSlots; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
+    out->counts = l.counts; out->offers = l.offers; out->bloom = l.bloom;
+    out->segment_state = l.seg_state; out->segment_updates = l.seg_updates; out->round = l.round; out->total = l.total;
+    out->width = l.width; out->reverse_cap = kRevCap; out->reverse_stride = kRevStride; out->offer_slots = offer_slots_for(l.width); out->reverse_slots = kRevSlots; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
     return GLIDE_OK;
 }
 

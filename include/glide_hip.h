@@ -149,9 +149,8 @@ int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim,
  * (nn_descent.cuh:1123,1280) runs one more round and is then left alone; from the third round on the partition
  * states are read back after each round (the call then waits on `stream`) and the loop ends once every partition
  * rests.  At most 2048 partitions.
- * stats_out (nullable, 2 device u64): offers the merge steps received; offers turned away by a full bucket of an overflow
- * table, i.e. offers to a node whose inbox was full that were worse than 15 others in their bucket (see `offers` below;
- * a diagnostic that depends on the order of arrival, which the graph does not).
+ * stats_out (nullable, 2 device u64): distinct offers the merge steps found in the offer tables; offers that stayed
+ * away because their target had announced a distance threshold (see `offers` and `norms` below).
  * Limits: knn_degree <= 128 (list width round_up32(1.3 * knn_degree) <= 192 = six sub-lists, Bloom filter <= 4096 bits),
  * dim % 4 == 0, reorder_num < 2^26 and reorder_num * list width < 2^32 per call (the large path calls it partition by
  * partition).  Two builds with the same inputs and seed give the same graph: nothing depends on the order in which
@@ -167,7 +166,7 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *   prepare         preprocess_data_kernel :445 (fp16 rows + fp32 squared norms), init_random_graph :1003,
  *                   Bloom filter cleared, first samples (sample_graph(true) :1040-1071)
  *   reverse_sample  add_rev_edges_kernel :490-507
- *   local_join      local_join_kernel :668-914; offers go to the per-node inbox (overflow table) instead of a spin-locked
+ *   local_join      local_join_kernel :668-914; offers go to the per-node offer table instead of a spin-locked
  *                   list; it restarts the reverse lists it has read
  *   merge           update_graph :1106-1126 + sample_graph_new :973-1001 + sample_segment_graph :1073-1104
  *   converge        the termination test of update_and_sample :1270-1284 (marks partitions that rest from now on)
@@ -182,24 +181,30 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *   fwd_new / fwd_old  num x 32 u32 sample lists, rev_new / rev_old  num rows of reverse_stride (72) u32 holding up to
  *                   reverse_cap (64) reverse samples in order of arrival; counts num x 4 u32 = their lengths (the reverse lengths count every arrival and may exceed
  *                   reverse_cap; the join uses the 32 smallest)
- *   inbox      num rows of inbox_stride (264) u64 holding up to inbox_cap (256) offers (distance bits << 32 | candidate id)
- *                   in order of arrival (the strides are not powers of two on purpose: rows fill from their start);
- *                   inbox_counts num u32 (arrivals, may exceed inbox_cap)
- *   rev_tables num x 2 (new, old) x reverse_slots (128) u32 and offers num x offer_slots (256) u64: overflow tables for
- *                   what arrives after a reverse list / an inbox is full.  They are made of buckets of 16 words: 15
- *                   slots (all ones = empty, slot order is a hash order) and, last, the bucket's bound = the smallest
- *                   key it has turned away (all ones: none).  A key's bucket is the top 3 (reverse) or 4 (offers) bits
- *                   of id * 0x9E3779B1; a bucket keeps the 15 smallest distinct keys sent to it.  The consumers use the
- *                   32 smallest keys of list + table (inbox + table), which do not depend on the order of arrival.
+ *   offers     num x offer_slots u64 keys (distance bits << 32 | candidate id, all ones = empty): the offers of the
+ *                   round.  offer_slots is 256 when the list is one sub-list (knn_degree <= 32) and 512 otherwise.  An
+ *                   offer goes to slot (x * 0x9E3779B1) >> (32 - log2 offer_slots), x = candidate ^ round * 0x85EBCA6B,
+ *                   of its target's row -- with 512 slots also to slot (x * 0xC2B2AE35) >> 23 -- and stays where it is
+ *                   the smallest key the slot has seen (an atomic minimum): copies of one offer fall together, of two
+ *                   candidates that share a slot the nearer one stays.  The merge reads the row, uses its 32 smallest
+ *                   distinct keys and empties it.  `round` (one u32, raised by converge) changes the slots from round
+ *                   to round.
+ *   rev_tables num x 2 (new, old) x reverse_slots (256) u32: overflow tables for what arrives after a reverse list is
+ *                   full.  They are made of buckets of 16 words: 15 slots (all ones = empty, slot order is a hash
+ *                   order) and, last, the bucket's bound = the smallest key it has turned away (all ones: none).  A
+ *                   key's bucket is the top 4 bits of id * 0x9E3779B1; a bucket keeps the 15 smallest distinct keys sent
+ *                   to it.  The join uses the 32 smallest sources of list + table.
  *   norms      num x (f32 squared norm of the fp32 row, u32 offer threshold); rev_thr num x 2 u32.  Thresholds are
- *                   what a node that overflowed announces for the next round: offers whose distance bits (sources whose
- *                   ids) are not below it stay away; all ones = none
+ *                   what a crowded node announces for the next round (an offer table with five eighths of its slots taken:
+ *                   the distance bits of its 64th smallest key; a reverse list that overflowed: its 56th smallest source):
+ *                   offers whose distance bits (sources whose ids) are not below it stay away; all ones = none.  None
+ *                   of this depends on the order in which atomic operations arrive.
  *   bloom      num x bloom_sets x 512 bits
  *   segment_state   u32 per partition: 0 active, 1 last round, 2 resting;  segment_updates  u32 per partition */
 typedef struct {
     uint64_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts,
-        inbox_counts, inbox, offers, bloom, segment_state, segment_updates, total;
-    uint32_t width, reverse_cap, reverse_stride, inbox_cap, inbox_stride, offer_slots, reverse_slots, row_halfs, bloom_sets, reserved;
+        offers, bloom, segment_state, segment_updates, round, total;
+    uint32_t width, reverse_cap, reverse_stride, offer_slots, reverse_slots, row_halfs, bloom_sets, reserved;
 } glide_nnd_layout;
 int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree, glide_nnd_layout *out);
 int glide_hip_nnd_prepare(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,

@@ -16,7 +16,7 @@ INV = 0xFFFFFFFF
 OLD = 0x80000000
 S = 32   # samples per list (NUM_SAMPLES, nn_descent.cuh:391)
 R = 256  # words of a reverse overflow table: 16 buckets of 15 slots + the bucket's bound
-CAP = 256  # offers an inbox holds before the overflow table takes over
+SLOTS = 256  # slots of a node's offer table when the list is one sub-list; 512 with several, where every offer goes to two slots
 RCAP = 64  # reverse samples a list holds before the overflow table takes over
 
 
@@ -45,8 +45,7 @@ class Workspace:
             rev_new=f(l.rev_new, n * l.reverse_stride).reshape(n, l.reverse_stride)[:, :RCAP], rev_old=f(l.rev_old, n * l.reverse_stride).reshape(n, l.reverse_stride)[:, :RCAP],
             rev_tables=f(l.rev_tables, n * 2 * R).reshape(n, 2, R), counts=f(l.counts, n * 4).reshape(n, 4),
             rev_thr=f(l.rev_thr, n * 2).reshape(n, 2),
-            inbox_counts=f(l.inbox_counts, n), inbox=f(l.inbox, n * l.inbox_stride * 2).view(np.uint64).reshape(n, l.inbox_stride)[:, :CAP],
-            segment_state=f(l.segment_state, 16), segment_updates=f(l.segment_updates, 16),
+            segment_state=f(l.segment_state, 16), segment_updates=f(l.segment_updates, 16), round=int(f(l.round, 1)[0]),
             offers=f(l.offers, n * l.offer_slots * 2).view(np.uint64).reshape(n, l.offer_slots),
             bloom=f(l.bloom, n * l.bloom_sets * 16).reshape(n, l.bloom_sets * 16),
             norms=f(l.norms, 2 * n, np.float32)[0::2].copy(), offer_thr=f(l.norms, 2 * n)[1::2].copy())
@@ -58,22 +57,6 @@ SLOT = np.arange(256) % 16 != 15          # word 15 of every bucket of 16 is the
 
 def offer_key(dist, cand):
     return (int(np.float32(dist).view(np.uint32)) << 32) | int(cand)
-
-
-def bucket_table(keys, bucket_bits, empty):
-    """What a table of 2^bucket_bits buckets holds of `keys` (their low 32 bits are the id that is hashed): per bucket the
-    15 smallest distinct keys; returns (kept keys sorted, {bucket: bound}) where a bucket's bound is the smallest key it
-    turned away."""
-    buckets = {}
-    for key in set(keys):
-        buckets.setdefault((((key & 0xFFFFFFFF) * 0x9E3779B1) & 0xFFFFFFFF) >> (32 - bucket_bits), []).append(key)
-    kept = sorted(k for b in buckets.values() for k in sorted(b)[:15])
-    bounds = {i: (sorted(b)[15] if len(b) > 15 else empty) for i, b in buckets.items()}
-    return kept, bounds
-
-
-def kept_by_table(keys):
-    return bucket_table(keys, 4, int(NO_OFFER))[0]
 
 
 def table_slots(row):
@@ -93,23 +76,36 @@ def reverse_samples(st, node, which):
     return sorted(set(got))[:S]
 
 
-def offers_held(st, node):
-    """Distinct offers a node holds after a join, ascending: inbox and, beyond CAP arrivals, its overflow table."""
-    cnt = int(st["inbox_counts"][node])
-    got = [int(x) for x in st["inbox"][node, :min(cnt, CAP)]]
-    if cnt > CAP:
-        got += table_slots(st["offers"][node])[0]
-    return sorted(set(got))
+def offers_held(st, node, distinct=True):
+    """The offers a node's table holds after a join, ascending."""
+    row = st["offers"][node]
+    held = [int(x) for x in row[row != NO_OFFER]]
+    return sorted(set(held) if distinct else held)
+
+
+def model_offer_table(keys, round_, slots=SLOTS):
+    """What a node's offer table holds once `keys` (distance bits << 32 | candidate) have all been sent to it: a slot
+    keeps the smallest key it was sent.  A key goes to slot (x * 0x9E3779B1) >> (32 - log2 slots), x = candidate ^
+    round * 0x85EBCA6B, and in a table of 512 also to slot (x * 0xC2B2AE35) >> 23."""
+    row = np.full(slots, NO_OFFER, np.uint64)
+    salt = (round_ * 0x85EBCA6B) & 0xFFFFFFFF
+    for key in keys:
+        x, shift = (key & 0xFFFFFFFF) ^ salt, 32 - slots.bit_length() + 1
+        for mult in (0x9E3779B1, 0xC2B2AE35)[:2 if slots == 512 else 1]:
+            slot = ((x * mult) & 0xFFFFFFFF) >> shift
+            if key < int(row[slot]):
+                row[slot] = np.uint64(key)
+    return row
 
 
 def model_offer_threshold(st, node):
-    """The threshold a node announces for the next join: after an overflow of its inbox the distance (bits) of the 64th best
-    distinct offer of the round; one in force is kept while 64 or more offers arrive and the best 32 are complete."""
-    cnt = int(st["inbox_counts"][node])
-    if cnt > CAP:
-        distinct = offers_held(st, node)
-        return distinct[63] >> 32 if len(distinct) >= 64 else INV
-    if cnt >= 64 and len(offers_held(st, node)) >= S:
+    """The threshold a node announces for the next join: when five eighths of its table's slots or more were taken, the
+    distance (bits) of the 64th best offer; one in force is kept while 40 or more slots are taken and 32 or more
+    offers held."""
+    taken, held = len(offers_held(st, node, distinct=False)), offers_held(st, node)
+    if taken >= st["offers"].shape[1] * 5 // 8:
+        return held[63] >> 32 if len(held) >= 64 else INV
+    if taken >= 40 and len(held) >= S:
         return int(st["offer_thr"][node])
     return INV
 
@@ -241,7 +237,7 @@ def test_stages_match_model(hip, degree):
     st = ws.read()
     width, sets = ws.l.width, ws.l.bloom_sets
     num_sub = width // S
-    assert width == {32: 32, 64: 96, 96: 128, 128: 192}[degree] and ws.l.offer_slots == 256
+    assert width == {32: 32, 64: 96, 96: 128, 128: 192}[degree] and ws.l.offer_slots == (256 if degree == 32 else 512)
     # prepare: random partition-local ids, no self, sub-list s holds ids = s mod num_sub; the first 32 in storage
     # order are sampled (flagged) as the first "new" samples
     local = np.arange(num) - np.repeat(seg_start, seg_len)
@@ -251,7 +247,7 @@ def test_stages_match_model(hip, degree):
     assert (((st["list_ids"] & ~np.uint32(OLD)) % num_sub) == (np.arange(width) % num_sub)[None, :]).all()
     assert (st["counts"][:, 0] == S).all() and (st["counts"][:, 1] == 0).all()
     np.testing.assert_array_equal(st["fwd_new"], st["list_ids"][:, :S] & ~np.uint32(OLD))
-    assert (st["offers"] == NO_OFFER).all() and (st["rev_tables"] == INV).all() and (st["inbox_counts"] == 0).all()
+    assert (st["offers"] == NO_OFFER).all() and (st["rev_tables"] == INV).all() and st["round"] == 0
     assert (st["counts"][:, 2:] == 0).all() and (st["rev_thr"] == INV).all() and (st["offer_thr"] == INV).all()
     np.testing.assert_array_equal(st["norms"], (rows ** 2).sum(1, dtype=np.float32))
 
@@ -283,7 +279,7 @@ def test_stages_match_model(hip, degree):
                     assert not Counter(in_table) - Counter(e)
                 assert reverse_samples(st, v, which) == sorted(set(e))[:S]
         assert overflowed > 0 or it == 0 or degree > 32
-        assert (st["offers"] == NO_OFFER).all() and (st["inbox_counts"] == 0).all()
+        assert (st["offers"] == NO_OFFER).all() and st["round"] == it
 
         hip.nnd_local_join(*args)
         hip.synchronize()
@@ -299,22 +295,16 @@ def test_stages_match_model(hip, degree):
                 else:
                     want = int(st["rev_thr"][v, which]) if cnt >= 40 else INV
                 assert after["rev_thr"][v, which] == want, (which, v, cnt)
-        total = 0
+        total = sent = 0
         for s0, l0 in zip(seg_start.tolist(), seg_len.tolist()):
             offers = model_join(st, rows, s0, l0)
             for t in range(l0):
-                exp = sorted(offer_key(d, c) for d, c in offers.get(t, []))
-                cnt = int(after["inbox_counts"][s0 + t])
-                assert cnt == len(exp), (s0, t, cnt, len(exp))
-                got = sorted(int(x) for x in after["inbox"][s0 + t, :min(cnt, CAP)])
-                if cnt <= CAP:
-                    assert got == exp, (s0, t)
-                    assert (after["offers"][s0 + t] == NO_OFFER).all()
-                else:
-                    assert not Counter(got) - Counter(exp)
-                assert offers_held(after, s0 + t)[:S] == sorted(set(exp))[:S]
-                total += cnt
-        assert total > 0
+                # the table: per slot the smallest key sent there, whatever the order of arrival
+                exp = model_offer_table([offer_key(d, c) for d, c in offers.get(t, [])], it, ws.l.offer_slots)
+                np.testing.assert_array_equal(after["offers"][s0 + t], exp, err_msg="offer table of node %d" % (s0 + t))
+                total += len(set(exp[exp != NO_OFFER].tolist()))
+                sent += len(set(offers.get(t, [])))
+        assert total > 0.8 * sent > 0          # few offers share a slot with a nearer one
 
         hip.nnd_merge(*args)
         hip.synchronize()
@@ -330,7 +320,7 @@ def test_stages_match_model(hip, degree):
             assert merged["fwd_new"][node, :len(fn)].tolist() == fn
             assert merged["fwd_old"][node, :len(fo)].tolist() == fo
             np.testing.assert_array_equal(merged["bloom"][node], words)
-        assert (merged["offers"] == NO_OFFER).all() and (merged["inbox_counts"] == 0).all()
+        assert (merged["offers"] == NO_OFFER).all()
         assert merged["segment_updates"][:2].tolist() == updates
         for node in range(num):
             assert int(merged["offer_thr"][node]) == model_offer_threshold(after, node), node
@@ -349,7 +339,7 @@ def test_stages_match_model(hip, degree):
         st = ws.read()
         expect = [2 if b == 1 else (1 if b == 0 and u < threshold * num * dim / 100 else b) for b, u in zip(before, updates)]
         assert st["segment_state"][:2].tolist() == expect and st["segment_updates"][:2].tolist() == [0, 0]
-        assert expect == [[0, 0], [1, 1], [2, 2]][it]
+        assert expect == [[0, 0], [1, 1], [2, 2]][it] and st["round"] == it + 1
 
     # a resting partition is skipped by every stage
     hip.nnd_reverse_sample(*args)
@@ -357,7 +347,7 @@ def test_stages_match_model(hip, degree):
     hip.nnd_merge(*args)
     hip.synchronize()
     rest = ws.read()
-    for key in ("list_ids", "list_dists", "fwd_new", "fwd_old", "bloom", "offers", "inbox_counts", "rev_tables", "counts"):
+    for key in ("list_ids", "list_dists", "fwd_new", "fwd_old", "bloom", "offers", "rev_tables", "counts"):
         np.testing.assert_array_equal(rest[key], st[key], err_msg=key)
 
     # finalize: the `degree` nearest entries of the whole list by (distance, id) (the sub-lists merged by distance)
@@ -372,11 +362,11 @@ def test_stages_match_model(hip, degree):
     assert (knn < lim).all()
 
 
-def test_full_inbox_overflows_into_the_table(hip):
-    """A hub: far more offers for one node than its inbox holds.  Built by hand: every list samples the same two points,
-    so those receive offers from every join.  Whatever went to the inbox and whatever to the overflow table, the best 32
-    distinct offers are all there, and the merge finds them."""
-    num, dim, degree = 6000, 128, 32
+def test_crowded_offer_table_announces_a_threshold(hip):
+    """A hub: thousands of offers for one node.  Built by hand: every list samples the same two points, so those receive
+    offers from every join.  Whatever the order of arrival, every slot of the hub's table ends with the smallest key sent
+    to it, the merge uses the 32 best of them, and the hub announces a distance threshold for the next join."""
+    num, dim, degree = 10000, 128, 32
     rows = lowdim_data(num, dim, seed=9)
     seg_start, seg_len = np.array([0], np.uint32), np.array([num], np.uint32)
     d_rows = hip.DeviceArray.from_numpy(rows)
@@ -399,23 +389,24 @@ def test_full_inbox_overflows_into_the_table(hip):
     hip.synchronize()
     after = ws.read()
     offers = model_join(dict(after, fwd_new=fwd), rows, 0, num)
-    assert len(offers[0]) > 4 * CAP and after["inbox_counts"][0] == len(offers[0])
-    assert len(table_slots(after["offers"][0])[0]) > 0
-    for t in (0, 1, 2, 500, 5999):
-        exp = sorted(set(offer_key(d, c) for d, c in offers.get(t, [])))
-        assert offers_held(after, t)[:S] == exp[:S], t
+    assert len(offers[0]) > 4 * SLOTS and len(set(offers[0])) > 200          # thousands of arrivals, a few hundred distinct
+    for t in (0, 1, 2, 500, 9999):
+        np.testing.assert_array_equal(after["offers"][t], model_offer_table([offer_key(d, c) for d, c in offers.get(t, [])], 0))
+    print("the hub holds", len(offers_held(after, 0)), "offers", flush=True)
+    assert len(offers_held(after, 0)) >= 160 > len(offers_held(after, 2))
     hip.nnd_merge(*args)
     hip.synchronize()
     merged = ws.read()
-    for node in (0, 1, 2, 500, 5999):
+    for node in (0, 1, 2, 500, 9999):
         l_ids, l_d, fn, fo, words, _ = model_merge(after, node, ws.l.width, ws.l.bloom_sets)
         np.testing.assert_array_equal(merged["list_ids"][node], l_ids)
         np.testing.assert_array_equal(merged["list_dists"][node], l_d)
         assert merged["fwd_new"][node, :len(fn)].tolist() == fn
-    assert (merged["offers"] == NO_OFFER).all() and (merged["inbox_counts"] == 0).all()
+    assert (merged["offers"] == NO_OFFER).all()
     # the hub has announced a threshold; a second join of the same lists sends it only what lies below
     thr = int(merged["offer_thr"][0])
-    assert thr == model_offer_threshold(after, 0) != INV
+    assert thr == model_offer_threshold(after, 0) == offers_held(after, 0)[63] >> 32
+    assert int(merged["offer_thr"][2]) == INV
     w = ws.buf.numpy()
     w[ws.l.fwd_new // 4: ws.l.fwd_new // 4 + num * S] = fwd.reshape(-1)
     w[ws.l.counts // 4: ws.l.counts // 4 + num * 4].reshape(num, 4)[:] = after["counts"]
@@ -423,9 +414,10 @@ def test_full_inbox_overflows_into_the_table(hip):
     hip.nnd_local_join(*args)
     hip.synchronize()
     again = ws.read()
-    below = sorted(offer_key(d, c) for d, c in offers[0] if offer_key(d, c) >> 32 < thr)
-    assert again["inbox_counts"][0] == len(below) < len(offers[0])
-    assert offers_held(again, 0)[:S] == sorted(set(below))[:S] == sorted(set(offer_key(d, c) for d, c in offers[0]))[:S]
+    below = [offer_key(d, c) for d, c in offers[0] if offer_key(d, c) >> 32 < thr]
+    assert 0 < len(below) < len(offers[0])
+    np.testing.assert_array_equal(again["offers"][0], model_offer_table(below, 0))
+    assert offers_held(again, 0)[:S] == offers_held(after, 0)[:S]
 
 
 @pytest.mark.parametrize("degree", [32, 64])
