@@ -51,20 +51,25 @@ __device__ __forceinline__ void locate(const Segments& s, uint32_t node, uint32_
 
 // Same result for a node every lane of the wavefront shares: the lanes test one segment each, so the lookup costs
 // one memory round trip instead of one per segment.  Every lane of the wavefront must call it.  Returns the index.
-__device__ __forceinline__ uint32_t locate_uniform(const Segments& s, uint32_t node, uint32_t& start, uint32_t& len) {
-    uint32_t found = s.count - 1;
-    for (uint32_t base = 0; base + 1 < s.count; base += 64) {
+__device__ __forceinline__ uint32_t locate_uniform(const Segments& s, uint32_t node, uint32_t& start, uint32_t& len, uint32_t* state = nullptr) {
+    for (uint32_t base = 0; base < s.count; base += 64) {
         const uint32_t i = base + lane_id();
-        const bool hit = i + 1 < s.count && node < s.starts[i] + s.lengths[i];
-        const uint64_t m = ballot(hit);
+        const bool in_range = i < s.count;
+        const uint32_t st = in_range ? s.starts[i] : 0u, ln = in_range ? s.lengths[i] : 0u;
+        const uint32_t state_i = state && in_range ? s.state[i] : 0u;
+        // the last segment takes whatever lies beyond it, as the scalar search does
+        const uint64_t m = ballot(in_range && (node < st + ln || i + 1 == s.count));
         if (m) {
-            found = base + static_cast<uint32_t>(__ffsll(static_cast<long long>(m))) - 1;
-            break;
+            const int at = __ffsll(static_cast<long long>(m)) - 1;   // the values come from the lane that tested the segment
+            start = read_lane(st, at);
+            len = read_lane(ln, at);
+            if (state) *state = read_lane(state_i, at);
+            return base + at;
         }
     }
-    start = s.starts[found];
-    len = s.lengths[found];
-    return found;
+    start = len = 0;   // no segments at all: not reached, the entry points refuse segment_num == 0
+    if (state) *state = kDone;
+    return 0;
 }
 
 // ---- prepare: fp32 rows -> fp16 rows (stride dim_pad, zero padded) + squared norms of the fp32 input
@@ -259,8 +264,9 @@ __global__ __launch_bounds__(256) void nnd_reverse_kernel(const uint32_t* fwd_ne
     const uint32_t node = idx / 64, j = idx % 64;
     if (node >= num) return;
     uint32_t start, len;
-    const uint32_t seg = locate_uniform(segs, node, start, len);
-    if (segs.state[seg] == kDone) return;
+    uint32_t state;
+    locate_uniform(segs, node, start, len, &state);
+    if (state == kDone) return;
     const uint32_t which = j / kSamples, k = j % kSamples;   // 0: new, 1: old
     if (k >= counts[static_cast<size_t>(node) * 4 + which]) return;
     const uint32_t v = (which ? fwd_old : fwd_new)[static_cast<size_t>(node) * kSamples + k];
@@ -295,8 +301,8 @@ struct JoinLds {
         JoinRows rows;
         float dist[kBi][kDStride];
     };
-    uint32_t new_ids[kBi], old_ids[kBi];
-    float new_norms[kBi], old_norms[kBi];
+    __attribute__((aligned(16))) uint32_t new_ids[kBi], old_ids[kBi];   // read four at a time
+    __attribute__((aligned(16))) float new_norms[kBi], old_norms[kBi];
     uint32_t hash_new[128], hash_old[128];
     __attribute__((aligned(16))) uint32_t rev_raw[2][kRevCap + kRevSlots];   // reverse samples as read: the list, then the overflow table
     uint32_t rev_sel[2][kSamples];                                 // their 32 smallest entries, ascending
@@ -381,11 +387,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     if (sampler) {
         L.hash_new[tid] = kInvalid;
         L.hash_old[tid] = kInvalid;
+        (is_old ? L.old_norms : L.new_norms)[k] = __builtin_inff();   // replaced below for the rows the lists hold
     }
     const uint4 c4 = *reinterpret_cast<const uint4*>(a.counts + static_cast<size_t>(node) * 4);
     uint32_t seg_start, seg_len;
-    const uint32_t seg = locate_uniform(a.segs, node, seg_start, seg_len);
-    if (a.segs.state[seg] == kDone) return;
+    uint32_t state;
+    locate_uniform(a.segs, node, seg_start, seg_len, &state);
+    if (state == kDone) return;
     // The counts must have arrived in every thread before thread 0 restarts them below; the barrier itself waits
     // for LDS traffic only, so the registers are consumed here.
     asm volatile("" ::"v"(c4.x), "v"(c4.y), "v"(c4.z), "v"(c4.w), "v"(my_id), "v"(thr_in_force));
@@ -513,12 +521,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     const uint32_t line = tid >> 2, part = tid & 3;
     // ---- phase 1: new x new
     __syncthreads();   // every wave is done with the rows: the tile may overwrite them
+    // Rows and columns beyond the lists carry an infinite norm (and zero rows), so their entries come out infinite
+    // without a test; the diagonal lies in the two wavefronts whose row and column blocks coincide.
+    {
+        const uint32_t j = cb * 32 + t;
+        const float nj = L.new_norms[j];
+        const bool diagonal_block = rb == cb;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
-        float d = FLT_MAX;
-        if (i < n_new && j < n_new && i != j) d = fmaxf((L.new_norms[i] + L.new_norms[j]) - 2.f * acc_nn[r], 0.f);
-        L.dist[i][j] = d;
+        for (int q = 0; q < 4; q++) {
+            const uint32_t i0 = rb * 32 + 8 * q + 4 * kh;
+            const float4 ni = *reinterpret_cast<const float4*>(&L.new_norms[i0]);
+            const float n4[4] = {ni.x, ni.y, ni.z, ni.w};
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                float d = fmaxf((n4[m] + nj) - 2.f * acc_nn[4 * q + m], 0.f);
+                if (diagonal_block && i0 + m == j) d = FLT_MAX;
+                L.dist[i0 + m][j] = d;
+            }
+        }
     }
     __syncthreads();
     // An offer is one atomic minimum on its slot of the target's table; nothing comes back, so the wave does not wait.
@@ -545,13 +565,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     if (n_old != 0) {
         // ---- phase 2: new x old (rows: new, columns: old)
         __syncthreads();
-        const uint32_t col_id = cb * 32 + t < n_old ? L.old_ids[cb * 32 + t] : kInvalid;
+        const uint32_t j = cb * 32 + t;
+        const uint32_t col_id = j < n_old ? L.old_ids[j] : kInvalid;
+        const float nj = L.old_norms[j];
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const uint32_t i = rb * 32 + 8 * (r / 4) + 4 * kh + (r % 4), j = cb * 32 + t;
-            float d = FLT_MAX;   // also where the same point sits in both lists: it is no partner of itself
-            if (i < n_new && j < n_old && L.new_ids[i] != col_id) d = fmaxf((L.new_norms[i] + L.old_norms[j]) - 2.f * acc_no[r], 0.f);
-            L.dist[i][j] = d;
+        for (int q = 0; q < 4; q++) {
+            const uint32_t i0 = rb * 32 + 8 * q + 4 * kh;
+            const float4 ni = *reinterpret_cast<const float4*>(&L.new_norms[i0]);
+            const uint4 idi = *reinterpret_cast<const uint4*>(&L.new_ids[i0]);
+            const float n4[4] = {ni.x, ni.y, ni.z, ni.w};
+            const uint32_t id4[4] = {idi.x, idi.y, idi.z, idi.w};
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                float d = fmaxf((n4[m] + nj) - 2.f * acc_no[4 * q + m], 0.f);
+                if (id4[m] == col_id) d = FLT_MAX;   // the same point sits in both lists: it is no partner of itself
+                L.dist[i0 + m][j] = d;
+            }
         }
         __syncthreads();
         {
@@ -751,43 +780,110 @@ template <int M2, uint32_t SLOTS>
 __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
     __shared__ MergeLds<SLOTS> L;
     constexpr int NR = M2 / 64;
+    constexpr int PASSES = SLOTS / 256;
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     const uint32_t node = blockIdx.x * 4 + wave;
     if (node >= a.num) return;
-    uint32_t seg_start, seg_len;
-    const uint32_t seg = locate_uniform(a.segs, node, seg_start, seg_len);
-    if (a.segs.state[seg] == kDone) return;
     const uint32_t width = a.width, num_sub = a.num_sub;
+    const uint32_t bloom_words = a.bloom_sets * 16;   // at most 128
+
+    // ---- everything the node needs from memory is asked for at once: the kernel is bound by the latency of its
+    // dependent memory round trips (this one, the thresholds of the sampled nodes, the slots of their reverse lists),
+    // not by bandwidth or arithmetic
+    unsigned long long* const table = a.offers + static_cast<size_t>(node) * SLOTS;
+    uint4 t_lo[PASSES], t_hi[PASSES];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        t_lo[p] = *reinterpret_cast<const uint4*>(table + 256 * p + 4 * lane);
+        t_hi[p] = *reinterpret_cast<const uint4*>(table + 256 * p + 4 * lane + 2);
+    }
+    uint32_t l_id[NR];
+    float l_dist[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        const uint32_t e = NR * lane + r;
+        l_id[r] = e < width ? a.list_ids[static_cast<size_t>(node) * width + e] : kInvalid;
+        l_dist[r] = e < width ? a.list_dists[static_cast<size_t>(node) * width + e] : FLT_MAX;
+    }
+    uint32_t bloom_in[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) bloom_in[j] = lane + 64u * j < bloom_words ? a.bloom[static_cast<size_t>(node) * bloom_words + lane + 64 * j] : 0u;
+    const uint32_t in_force = __float_as_uint(a.norms[node].y);
+    uint32_t seg_start, seg_len, state;
+    const uint32_t seg = locate_uniform(a.segs, node, seg_start, seg_len, &state);
+    if (state == kDone) return;
+
     unsigned long long* keys = L.keys[wave];
     unsigned long long* best = L.best[wave];
     unsigned long long* enter = L.enter[wave];
     uint32_t* known = L.known[wave];
     uint32_t* filter = L.filter[wave];
     uint32_t* flags = L.flags[wave];
-    const uint32_t bloom_words = a.bloom_sets * 16;
-    for (uint32_t w = lane; w < bloom_words; w += 64) filter[w] = a.bloom[static_cast<size_t>(node) * bloom_words + w];
     for (uint32_t i = lane; i < (1u << kKnownBits); i += 64) known[i] = kInvalid;
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+        if (lane + 64u * j < bloom_words) filter[lane + 64 * j] = bloom_in[j];
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- the incoming list, in storage order; its ids go into the wavefront's id set
+    unsigned long long k[NR];
+    uint32_t v[NR];
+    uint32_t old_count = 0;
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        k[r] = ~0ull;
+        v[r] = 0;
+        const uint32_t id = l_id[r];
+        if (id != kInvalid) {
+            k[r] = (static_cast<unsigned long long>(__float_as_uint(l_dist[r])) << 32) | (static_cast<unsigned long long>(id & ~kOld) << 1);
+            v[r] = id & kOld;
+            old_count += (id & kOld) != 0;
+            hash_insert(known, kKnownBits, id & ~kOld);
+        }
+    }
+    // old samples from the incoming list (element order = storage order = the reference's scan order).  With the
+    // scatter fused in, a sample also enters the reverse list of the node it names: first the threshold that node has
+    // announced is asked for, further down a slot, and the entry is stored at the very end.
+    const uint32_t me = node - seg_start;
+    uint32_t total_old;
+    size_t old_target[NR];
+    uint32_t old_thr[NR], old_pos[NR];
+    {
+        uint32_t rank = wave_exclusive_scan(old_count, total_old);
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+            old_target[r] = ~static_cast<size_t>(0);
+            old_thr[r] = 0;
+            if (k[r] != ~0ull && (v[r] & kOld)) {
+                if (rank < kSamples) {
+                    const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
+                    a.fwd_old[static_cast<size_t>(node) * kSamples + rank] = id;
+                    if (a.rev_old) {
+                        old_target[r] = static_cast<size_t>(seg_start) + id;
+                        old_thr[r] = a.rev_thr[old_target[r] * 2 + 1];
+                    }
+                }
+                rank++;
+            }
+        }
+    }
 
     // ---- this round's offers: the node's table, four slots per lane and pass, emptied where something was found
     uint32_t held;
     {
-        unsigned long long* row = a.offers + static_cast<size_t>(node) * SLOTS;
-        constexpr int PASSES = SLOTS / 256;
         unsigned long long o[PASSES][4];
         uint32_t mine = 0;
 #pragma unroll
         for (int p = 0; p < PASSES; p++) {
-            unsigned long long* at = row + 256 * p + 4 * lane;
-            const uint4 lo = *reinterpret_cast<const uint4*>(at), hi = *reinterpret_cast<const uint4*>(at + 2);
-            o[p][0] = (static_cast<unsigned long long>(lo.y) << 32) | lo.x;
-            o[p][1] = (static_cast<unsigned long long>(lo.w) << 32) | lo.z;
-            o[p][2] = (static_cast<unsigned long long>(hi.y) << 32) | hi.x;
-            o[p][3] = (static_cast<unsigned long long>(hi.w) << 32) | hi.z;
+            o[p][0] = (static_cast<unsigned long long>(t_lo[p].y) << 32) | t_lo[p].x;
+            o[p][1] = (static_cast<unsigned long long>(t_lo[p].w) << 32) | t_lo[p].z;
+            o[p][2] = (static_cast<unsigned long long>(t_hi[p].y) << 32) | t_hi[p].x;
+            o[p][3] = (static_cast<unsigned long long>(t_hi[p].w) << 32) | t_hi[p].z;
             if ((o[p][0] & o[p][1] & o[p][2] & o[p][3]) != kNoOffer) {
                 const uint4 empty = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
-                *reinterpret_cast<uint4*>(at) = empty;
-                *reinterpret_cast<uint4*>(at + 2) = empty;
+                *reinterpret_cast<uint4*>(table + 256 * p + 4 * lane) = empty;
+                *reinterpret_cast<uint4*>(table + 256 * p + 4 * lane + 2) = empty;
             }
 #pragma unroll
             for (int j = 0; j < 4; j++) mine += o[p][j] != kNoOffer;
@@ -802,7 +898,6 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
     __builtin_amdgcn_wave_barrier();
     uint32_t n_best;
     uint32_t next_thr;
-    const uint32_t in_force = __float_as_uint(a.norms[node].y);
     if (held < SLOTS / 8 * kOfferCrowdedEighths) {
         n_best = best_offers_sized<SLOTS>(keys, held, best, lane);
         // a threshold that is in force stays while the node still receives plenty of offers and its best 32 are complete
@@ -816,46 +911,10 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
     }
     if (lane == 0 && next_thr != in_force) a.norms[node].y = __uint_as_float(next_thr);
 
-    // ---- the incoming list, in storage order; its ids go into the wavefront's id set
-    unsigned long long k[NR];
-    uint32_t v[NR];
-    uint32_t old_count = 0;
-#pragma unroll
-    for (int r = 0; r < NR; r++) {
-        const uint32_t e = NR * lane + r;
-        k[r] = ~0ull;
-        v[r] = 0;
-        if (e < width) {
-            const uint32_t id = a.list_ids[static_cast<size_t>(node) * width + e];
-            const float d = a.list_dists[static_cast<size_t>(node) * width + e];
-            if (id != kInvalid) {
-                k[r] = (static_cast<unsigned long long>(__float_as_uint(d)) << 32) | (static_cast<unsigned long long>(id & ~kOld) << 1);
-                v[r] = id & kOld;
-                old_count += (id & kOld) != 0;
-                hash_insert(known, kKnownBits, id & ~kOld);
-            }
-        }
-    }
-    // old samples from the incoming list (element order = storage order = the reference's scan order)
-    uint32_t total_old;
-    {
-        uint32_t rank = wave_exclusive_scan(old_count, total_old);
-#pragma unroll
-        for (int r = 0; r < NR; r++) {
-            if (k[r] != ~0ull && (v[r] & kOld)) {
-                if (rank < kSamples) {
-                    const uint32_t id = static_cast<uint32_t>((k[r] >> 1) & 0x7fffffffull);
-                    a.fwd_old[static_cast<size_t>(node) * kSamples + rank] = id;
-                    if (a.rev_old) reverse_append(a.counts, a.rev_old, a.rev_tables, a.rev_thr, static_cast<size_t>(seg_start) + id, 1, node - seg_start);
-                }
-                rank++;
-            }
-        }
-    }
-    __builtin_amdgcn_wave_barrier();
-
     // ---- the best 32 offers, one per lane: new samples, and which of them enter the list
     uint32_t total_new = 0;
+    size_t new_target = ~static_cast<size_t>(0);
+    uint32_t new_thr = 0, new_pos = 0;
     {
         const bool mine = static_cast<uint32_t>(lane) < n_best;
         const unsigned long long key = mine ? best[lane] : kNoOffer;
@@ -874,7 +933,10 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
         __builtin_amdgcn_wave_barrier();   // every lane has tested the filter before bits are added
         if (fresh) {   // at most 32 of them: all become samples
             a.fwd_new[static_cast<size_t>(node) * kSamples + prefix_count(fm)] = id;
-            if (a.rev_new) reverse_append(a.counts, a.rev_new, a.rev_tables, a.rev_thr, static_cast<size_t>(seg_start) + id, 0, node - seg_start);
+            if (a.rev_new) {
+                new_target = static_cast<size_t>(seg_start) + id;
+                new_thr = a.rev_thr[new_target * 2];
+            }
             atomicOr(&filter[b[0] >> 5], 1u << (b[0] & 31));
             atomicOr(&filter[b[1] >> 5], 1u << (b[1] & 31));
             atomicOr(&filter[b[2] >> 5], 1u << (b[2] & 31));
@@ -884,6 +946,16 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
             flags[lane] = fresh ? kOld : 0u;
         }
     }
+    // the slots of the reverse entries (add_rev_edges_kernel :490-507 for one sample each): a sample whose source is
+    // not below the threshold of the node it names stays away
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        if (old_target[r] != ~static_cast<size_t>(0) && me >= old_thr[r]) old_target[r] = ~static_cast<size_t>(0);
+        old_pos[r] = old_target[r] != ~static_cast<size_t>(0) ? atomicAdd(&a.counts[old_target[r] * 4 + 3], 1u) : 0u;
+    }
+    if (new_target != ~static_cast<size_t>(0) && me >= new_thr) new_target = ~static_cast<size_t>(0);
+    if (new_target != ~static_cast<size_t>(0)) new_pos = atomicAdd(&a.counts[new_target * 4 + 2], 1u);
+
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int r = 0; r < NR; r++) {
@@ -955,6 +1027,22 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
         }
         // striped over 1024 slots: one shared address would serialise every wavefront of the launch
         if (a.stats && held) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u)], static_cast<unsigned long long>(held));
+    }
+    // ---- the reverse entries, now that their slots have come back: into the list, or past its end into the overflow table
+#pragma unroll
+    for (int r = 0; r < NR; r++) {
+        if (old_target[r] != ~static_cast<size_t>(0)) {
+            if (old_pos[r] < kRevCap)
+                a.rev_old[old_target[r] * kRevStride + old_pos[r]] = me;
+            else
+                reverse_insert(a.rev_tables + (old_target[r] * 2 + 1) * kRevSlots, me);
+        }
+    }
+    if (new_target != ~static_cast<size_t>(0)) {
+        if (new_pos < kRevCap)
+            a.rev_new[new_target * kRevStride + new_pos] = me;
+        else
+            reverse_insert(a.rev_tables + new_target * 2 * kRevSlots, me);
     }
 }
 
