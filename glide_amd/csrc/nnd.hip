@@ -941,8 +941,21 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
             atomicOr(&filter[b[1] >> 5], 1u << (b[1] & 31));
             atomicOr(&filter[b[2] >> 5], 1u << (b[2] & 31));
         }
-        if (lane < static_cast<int>(kSamples)) {
-            enter[lane] = enters ? ((key >> 32) << 32) | (static_cast<unsigned long long>(id) << 1) | 1ull : ~0ull;
+        const unsigned long long entering = ((key >> 32) << 32) | (static_cast<unsigned long long>(id) << 1) | 1ull;
+        if constexpr (NR == 1) {
+            // One sub-list: the list is in ascending order from the second round on, and so are the offers.  The
+            // entering ones are packed in descending order behind it, which makes the whole a bitonic sequence that
+            // six exchange steps sort.
+            const uint64_t em = ballot(enters);
+            if (lane < static_cast<int>(kSamples)) enter[lane] = ~0ull;
+            __builtin_amdgcn_wave_barrier();
+            if (enters) {
+                const uint32_t at = kSamples - 1 - prefix_count(em);
+                enter[at] = entering;
+                flags[at] = fresh ? kOld : 0u;
+            }
+        } else if (lane < static_cast<int>(kSamples)) {
+            enter[lane] = enters ? entering : ~0ull;
             flags[lane] = fresh ? kOld : 0u;
         }
     }
@@ -965,7 +978,18 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
             v[r] = flags[e - width];
         }
     }
-    Net64<M2, true>::sort(k, v, lane);
+    if constexpr (NR == 1) {
+        const unsigned long long before =
+            (static_cast<unsigned long long>(static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[0] >> 32), 0x138, 0xf, 0xf, false))) << 32) |
+            static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(k[0]), 0x138, 0xf, 0xf, false));   // wave_shr:1
+        const bool out_of_order = lane > 0 && lane < static_cast<int>(kSamples) && before > k[0];
+        if (ballot(out_of_order) == 0)
+            Net64<M2, true>::template merge_from<M2, M2 / 2>(k, v, lane);
+        else   // the random start lists, or a list a caller has replaced
+            Net64<M2, true>::sort(k, v, lane);
+    } else {
+        Net64<M2, true>::sort(k, v, lane);
+    }
 
     // ---- every sub-list keeps its 32 nearest: rank of an entry among those of its sub-list, in sorted order
     const unsigned long long last_of_prev =
