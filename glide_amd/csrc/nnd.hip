@@ -674,20 +674,6 @@ __device__ __forceinline__ void bloom_bits(uint32_t id, uint32_t bloom_sets, uin
     b[2] = base + h % 512;
 }
 
-// Prefix sum over the 64 lanes without LDS traffic: four shifted adds inside each row of 16 lanes, then lane 15 of a row
-// is added to the next row (rows 1 and 3) and lane 31 to the upper half (rows 2 and 3).  Lanes a step does not feed add 0.
-__device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t value, uint32_t& total) {
-    int x = static_cast<int>(value);
-    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, true);   // row_shr:1
-    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, true);   // row_shr:2
-    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, true);   // row_shr:4
-    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, true);   // row_shr:8
-    x += __builtin_amdgcn_update_dpp(0, x, 0x142, 0xa, 0xf, true);   // row_bcast:15
-    x += __builtin_amdgcn_update_dpp(0, x, 0x143, 0xc, 0xf, true);   // row_bcast:31
-    total = static_cast<uint32_t>(__builtin_amdgcn_readlane(x, 63));
-    return static_cast<uint32_t>(x) - value;
-}
-
 struct MergeArgs {
     uint32_t* list_ids;
     float* list_dists;

@@ -1,5 +1,5 @@
-// Locality partitioning: point -> centroid assignment (fp32 MFMA tile + norm-trick ranking, exact rescoring of
-// the best few), stable slot numbering, row reordering, row sampling and a small Lloyd k-means.
+// Locality partitioning: point -> centroid assignment (fp32 MFMA tile + norm-trick ranking, exact distances to the
+// centroids within the ranking's error band of the second best), stable slot numbering, row reordering, row sampling and a small Lloyd k-means.
 // Reference: define_partition_kernel (partition_kernel.cuh:22-66), reorder_kernel (:68-100), sample_kernel
 // (:7-20), host sequencing partition.cuh:8-193.
 #include "common.hpp"
@@ -13,7 +13,6 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 constexpr int kTilePoints = 128;   // points per workgroup (4 wavefronts x 32)
 constexpr int kChunk = 32;         // dims staged per step
 constexpr int kLdsStride = 36;     // floats per staged row (32 + 4 pad keeps 16-byte alignment, spreads banks)
-constexpr int kTop = 4;            // candidates kept from the ranking pass and rescored exactly
 
 struct AssignArgs {
     const float* data;
@@ -42,14 +41,48 @@ __device__ __forceinline__ float exact_distance_half(const float* x, const float
     return half_wave_sum(acc);
 }
 
-// CB = number of 32-centroid column blocks held in accumulators (centroid_num <= 32*CB)
+// Ranking pass of assign_kernel: which centroids have to be measured exactly.
+// The matrix cores give s(c) = ||c||^2 - 2 x.c, which ranks the centroids of one point like the squared distance but
+// carries rounding error.  With E bounding |s(c) + ||x||^2 - D(c)| for the distance D(c) that the exact pass computes
+// (squared, before the root), a centroid among the two nearest by D has s(c) <= s2 + 2 E, s2 being the second smallest
+// score: were it larger, two other centroids would have scores below s(c) - 2 E and therefore smaller D.  So the
+// centroids within `band` = 2 E of the second smallest score are the only ones the exact pass has to see -- two of
+// them for nearly every point -- and the nearest two come out as if every centroid had been measured.
+// E: the dot product of dim terms is off by at most (dim + 2) u (||x||^2 + ||c||^2) / 2 whatever the order of its sums
+// (u = 2^-24; doubled here in case the matrix pipeline rounds products and sums separately), ||c||^2 as stored by
+// (dim + 6) u ||c||^2, the final multiply-add by u |s|, D by (dim + 2) u D <= 2 (dim + 2) u (||x||^2 + ||c||^2), and
+// roots of D within 3 u of each other may tie: together below 6 (2 dim + 16) u (||x||^2 + max ||c||^2).
+__device__ __forceinline__ float assign_band(uint32_t dim, float x_norm, float max_centroid_norm) {
+    return 12.f * static_cast<float>(2 * dim + 16) * 5.9604645e-8f * 1.01f * (x_norm + max_centroid_norm);
+}
+
+constexpr int kKeep = 4;   // candidates one lane can pass to the exact pass; a point with more is measured against every centroid
+
+// smallest two of a point's candidates by (distance, centroid id)
+__device__ __forceinline__ void nearest_two(float dk, uint32_t ck, float& d0, uint32_t& c0, float& d1, uint32_t& c1) {
+    const bool lt0 = dk < d0 || (dk == d0 && ck < c0);
+    const bool lt1 = dk < d1 || (dk == d1 && ck < c1);
+    if (lt0) {
+        d1 = d0; c1 = c0;
+        d0 = dk; c0 = ck;
+    } else if (lt1) {
+        d1 = dk; c1 = ck;
+    }
+}
+
+// CB = number of 32-centroid row blocks held in accumulators (centroid_num <= 32*CB).
+// One wavefront owns 32 points.  The matrix instruction takes the centroids as its A operand and the points as B, so
+// lane (t, half) ends with the scores of point t against 16 centroids of every block in its own registers and ranks
+// them there: no score tile, no barrier after the matrix passes.
+// At least two wavefronts per SIMD: with eight blocks the 128 accumulators leave 128 registers for everything else, and
+// a second wavefront is what keeps the matrix cores fed while the first one ranks and measures.
 template <int CB>
-__global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void assign_kernel(AssignArgs a) {
     extern __shared__ __align__(16) float smem[];
     float* cent_tile = smem;                                   // [32*CB][kLdsStride]
     float* x_tile = cent_tile + 32 * CB * kLdsStride;          // [4 waves][32][kLdsStride]
-    float* score_tile = x_tile + 4 * 32 * kLdsStride;          // [4 waves][32][33]
-    uint32_t* hist = reinterpret_cast<uint32_t*>(score_tile + 4 * 32 * 33);  // [C + 1]
+    float* cnorm = x_tile + 4 * 32 * kLdsStride;               // [32*CB]: ||c||^2, +inf beyond centroid_num
+    uint32_t* hist = reinterpret_cast<uint32_t*>(cnorm + 32 * CB);   // [C + 1]
 
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
@@ -57,9 +90,9 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
     const uint32_t tile_base = blockIdx.x * kTilePoints;
     const uint32_t wave_base = tile_base + wave * 32;
     float* xw = x_tile + wave * 32 * kLdsStride;
-    float* sw = score_tile + wave * 32 * 33;
 
     for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256) hist[i] = 0;
+    for (uint32_t i = threadIdx.x; i < 32 * CB; i += 256) cnorm[i] = i < a.centroid_num ? a.centroid_norms[i] : __builtin_inff();
 
     float16v acc[CB];
 #pragma unroll
@@ -68,8 +101,10 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
         for (int r = 0; r < 16; r++) acc[cb][r] = 0.f;
 
     // Chunks of kChunk dims go global -> registers -> LDS; the loads of chunk k+1 are issued before the matrix
-    // instructions of chunk k, so their latency is covered by the MFMA work.
+    // instructions of chunk k, so their latency is covered by the MFMA work.  The squared norms of the points (for the
+    // error band of the ranking) are summed on the way.
     float4 cpre[CB], xpre[4];
+    float xsq[4] = {0.f, 0.f, 0.f, 0.f};
     auto prefetch = [&](uint32_t k0) {
 #pragma unroll
         for (int it = 0; it < CB; it++) {   // centroid chunk: 8 lanes x float4 per row, 32*CB rows over 256 threads
@@ -95,132 +130,177 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
             *reinterpret_cast<float4*>(cent_tile + (idx >> 3) * kLdsStride + (idx & 7) * 4) = cpre[it];
         }
 #pragma unroll
-        for (int it = 0; it < 4; it++) *reinterpret_cast<float4*>(xw + (it * 8 + (lane >> 3)) * kLdsStride + (lane & 7) * 4) = xpre[it];
+        for (int it = 0; it < 4; it++) {
+            *reinterpret_cast<float4*>(xw + (it * 8 + (lane >> 3)) * kLdsStride + (lane & 7) * 4) = xpre[it];
+            xsq[it] = fmaf(xpre[it].x, xpre[it].x, fmaf(xpre[it].y, xpre[it].y, fmaf(xpre[it].z, xpre[it].z, fmaf(xpre[it].w, xpre[it].w, xsq[it]))));
+        }
         __syncthreads();
         if (k0 + kChunk < a.dim) prefetch(k0 + kChunk);
         // v_mfma_f32_32x32x2_f32: lane supplies A[i = lane%32][k-slot = lane/32] and B[k-slot][j = lane%32].
         // A k-slot pair is fed from one float4 per half (dims kk+4*half .. +3), component by component.
 #pragma unroll
         for (int kk = 0; kk < kChunk; kk += 8) {
-            const float4 av = *reinterpret_cast<const float4*>(xw + t * kLdsStride + kk + 4 * half);
+            const float4 xv = *reinterpret_cast<const float4*>(xw + t * kLdsStride + kk + 4 * half);
 #pragma unroll
             for (int cb = 0; cb < CB; cb++) {
-                const float4 bv = *reinterpret_cast<const float4*>(cent_tile + (cb * 32 + t) * kLdsStride + kk + 4 * half);
-                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc[cb], 0, 0, 0);
-                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc[cb], 0, 0, 0);
-                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc[cb], 0, 0, 0);
-                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc[cb], 0, 0, 0);
+                const float4 cv = *reinterpret_cast<const float4*>(cent_tile + (cb * 32 + t) * kLdsStride + kk + 4 * half);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(cv.x, xv.x, acc[cb], 0, 0, 0);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(cv.y, xv.y, acc[cb], 0, 0, 0);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(cv.z, xv.z, acc[cb], 0, 0, 0);
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x2f32(cv.w, xv.w, acc[cb], 0, 0, 0);
             }
         }
     }
 
-    // ranking epilogue: score = ||c||^2 - 2 x.c (the ||x||^2 term is constant per point).  Lane (i = lane % 32,
-    // half) keeps the kTop smallest scores of point i over its half of every 32-column block; the halves are merged
-    // afterwards, so both lanes of a point end with the same kTop candidates.
-    float best_s[kTop];
-    uint32_t best_c[kTop];
+    // From here on the wavefront is on its own.  Its x tile is free (LDS operations of one wavefront complete in order,
+    // and the last matrix pass has read it) and becomes its scratch:
+    uint32_t* cand_by_lane = reinterpret_cast<uint32_t*>(xw);      // [64][kKeep] centroids within the band, per lane
+    uint32_t* lane_first = cand_by_lane + 64 * kKeep;              // [64] where a lane's pairs start
+    uint32_t* lane_pairs = lane_first + 64;                        // [64] how many it has
+    uint32_t* pairs = lane_pairs + 64;                             // [64 * kKeep] (point << 16 | centroid), one per exact distance
+    float* exact = reinterpret_cast<float*>(pairs + 64 * kKeep);   // [64 * kKeep]
+    float* x_norm = exact + 64 * kKeep;                            // [32]
+    static_assert(64 * kKeep * 3 + 128 + 32 <= 32 * kLdsStride, "scratch fits the x tile");
 #pragma unroll
-    for (int k = 0; k < kTop; k++) {
-        best_s[k] = FLT_MAX;
-        best_c[k] = kInvalid;
+    for (int it = 0; it < 4; it++) {
+        const float total = row_sum<1>(xsq[it]);   // the 8 lanes that staged a row
+        if ((lane & 7) == 0) x_norm[it * 8 + (lane >> 3)] = total;
     }
-    auto offer = [&](float s, uint32_t c) {
+    float max_cn = 0.f;
+    for (uint32_t i = lane; i < a.centroid_num; i += 64) max_cn = fmaxf(max_cn, cnorm[i]);
 #pragma unroll
-        for (int k = 0; k < kTop; k++) {
-            if (s < best_s[k]) {
-                const float ts = best_s[k];
-                const uint32_t tc = best_c[k];
-                best_s[k] = s;
-                best_c[k] = c;
-                s = ts;
-                c = tc;
-            }
-        }
-    };
+    for (int m = 32; m >= 1; m >>= 1) max_cn = fmaxf(max_cn, __shfl_xor(max_cn, m));
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- ranking, first sweep: score = ||c||^2 - 2 x.c and the two smallest scores of the point.  The scores are not
+    // kept (a second copy of every accumulator would halve the wavefronts a SIMD holds): the second sweep forms them again.
+    // Accumulator r of block cb belongs to centroid cb*32 + 8*(r/4) + 4*half + r%4 and point t.
+    float m1 = __builtin_inff(), m2 = __builtin_inff();   // m1 <= m2
 #pragma unroll
     for (int cb = 0; cb < CB; cb++) {
-        const uint32_t j = cb * 32 + t;
-        const float cn = j < a.centroid_num ? a.centroid_norms[j] : 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int i = 8 * (r / 4) + 4 * half + (r % 4);   // accumulator layout of the 32x32 tile
-            sw[i * 33 + t] = j < a.centroid_num ? cn - 2.f * acc[cb][r] : FLT_MAX;
-        }
-        __syncthreads();
-#pragma unroll 4
-        for (int jj = 0; jj < 16; jj++) offer(sw[t * 33 + half * 16 + jj], cb * 32 + half * 16 + jj);
-        __syncthreads();
-    }
-    {
-        float os[kTop];
-        uint32_t oc[kTop];
+        for (int q = 0; q < 4; q++) {
+            const float4 c4 = *reinterpret_cast<const float4*>(cnorm + cb * 32 + 8 * q + 4 * half);
+            const float cn[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
-        for (int k = 0; k < kTop; k++) {
-            os[k] = lane_xor<32>(best_s[k]);
-            oc[k] = lane_xor<32>(best_c[k]);
-        }
-#pragma unroll
-        for (int k = 0; k < kTop; k++) offer(os[k], oc[k]);
-    }
-
-    // exact rescoring of the kept candidates: 32 points x kTop pairs per wavefront, one pair per group of 8 lanes,
-    // four steps (32 pairs) in flight.  Candidates and distances are exchanged through this wave's score tile.
-    uint32_t* cand = reinterpret_cast<uint32_t*>(sw);          // [32][kTop]
-    float* exact = sw + 32 * kTop;                             // [32][kTop]
-    if (half == 0) {
-#pragma unroll
-        for (int k = 0; k < kTop; k++) cand[t * kTop + k] = best_c[k];
-    }
-    __syncthreads();
-    {
-        const int g = lane >> 3, t8 = lane & 7;
-        const uint32_t last = a.num - 1;
-        for (int s0 = 0; s0 < 32 * kTop / 8; s0 += 4) {
-            const float* xr[4];
-            const float* cr[4];
-            uint32_t cid[4];
-            float part[4];
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int pair = (s0 + u) * 8 + g;
-                const uint32_t pt = wave_base + (pair / kTop);
-                cid[u] = cand[pair];
-                xr[u] = a.data + static_cast<size_t>(pt < a.num ? pt : last) * a.dim;
-                cr[u] = a.centroids + static_cast<size_t>(cid[u] != kInvalid ? cid[u] : 0u) * a.dim;
-                part[u] = 0.f;
+            for (int m = 0; m < 4; m++) {
+                const float sc = fmaf(-2.f, acc[cb][4 * q + m], cn[m]);   // +inf beyond centroid_num
+                m2 = __builtin_amdgcn_fmed3f(m1, m2, sc);   // the second smallest of the three
+                m1 = fminf(m1, sc);
             }
-            for (uint32_t d0 = t8 * 4; d0 < a.dim; d0 += 32) {
-                float4 xv[4], cv[4];
+        }
+    }
+    {
+        const float o1 = lane_xor<32>(m1), o2 = lane_xor<32>(m2);   // the other half of the point's centroids
+        m2 = fminf(fmaxf(m1, o1), fminf(m2, o2));
+        m1 = fminf(m1, o1);
+    }
+    // ---- second sweep: the centroids within the band of the second smallest score
+    const float limit = fminf(m2 + assign_band(a.dim, x_norm[t], max_cn), FLT_MAX);   // one centroid only: every valid score passes
+    uint32_t found = 0;
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    xv[u] = *reinterpret_cast<const float4*>(xr[u] + d0);
-                    cv[u] = *reinterpret_cast<const float4*>(cr[u] + d0);
+    for (int cb = 0; cb < CB; cb++) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const float4 c4 = *reinterpret_cast<const float4*>(cnorm + cb * 32 + 8 * q + 4 * half);
+            const bool h0 = fmaf(-2.f, acc[cb][4 * q], c4.x) <= limit, h1 = fmaf(-2.f, acc[cb][4 * q + 1], c4.y) <= limit,
+                       h2 = fmaf(-2.f, acc[cb][4 * q + 2], c4.z) <= limit, h3 = fmaf(-2.f, acc[cb][4 * q + 3], c4.w) <= limit;
+            if (h0 | h1 | h2 | h3) {
+                const uint32_t c_first = cb * 32 + 8 * q + 4 * half;
+                const bool h[4] = {h0, h1, h2, h3};
+#pragma unroll
+                for (int m = 0; m < 4; m++) {
+                    if (h[m]) {
+                        if (found < kKeep) cand_by_lane[lane * kKeep + found] = c_first + m;
+                        found++;
+                    }
                 }
-#pragma unroll
-                for (int u = 0; u < 4; u++) part[u] = sqdist4(xv[u], cv[u], part[u]);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const float sq = row_sum<1>(part[u]);   // 8-lane groups
-                if (t8 == 0) exact[(s0 + u) * 8 + g] = cid[u] != kInvalid ? finish_distance(sq, a.metric) : FLT_MAX;
             }
         }
     }
-    __syncthreads();
-    // smallest two by (distance, centroid id); lane i < 32 owns point i
+    const bool crowded = found > kKeep;
+    const uint32_t mine = crowded ? kKeep : found;
+    uint32_t pair_count;
+    const uint32_t first = wave_exclusive_scan(mine, pair_count);
+    lane_first[lane] = first;
+    lane_pairs[lane] = mine;
+    for (uint32_t k = 0; k < mine; k++) pairs[first + k] = (static_cast<uint32_t>(t) << 16) | cand_by_lane[lane * kKeep + k];
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- exact distances of the pairs: one pair per group of 8 lanes, four steps (32 pairs) in flight
+    const int g = lane >> 3, t8 = lane & 7;
+    const uint32_t last = a.num - 1;
+    for (uint32_t s0 = 0; s0 < pair_count; s0 += 32) {
+        const float* xr[4];
+        const float* cr[4];
+        float part[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t pair = s0 + u * 8 + g;
+            const uint32_t pc = pairs[pair < pair_count ? pair : 0u];
+            const uint32_t pt = wave_base + (pc >> 16);
+            xr[u] = a.data + static_cast<size_t>(pt < a.num ? pt : last) * a.dim;
+            cr[u] = a.centroids + static_cast<size_t>(pc & 0xffffu) * a.dim;
+            part[u] = 0.f;
+        }
+        for (uint32_t d0 = t8 * 4; d0 < a.dim; d0 += 32) {
+            float4 xv[4], cv[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                xv[u] = *reinterpret_cast<const float4*>(xr[u] + d0);
+                cv[u] = *reinterpret_cast<const float4*>(cr[u] + d0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) part[u] = sqdist4(xv[u], cv[u], part[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t pair = s0 + u * 8 + g;
+            const float sq = row_sum<1>(part[u]);   // 8-lane groups
+            if (t8 == 0 && pair < pair_count) exact[pair] = finish_distance(sq, a.metric);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    // smallest two by (distance, centroid id); lane i < 32 owns point i and reads the pairs of both its halves
     float d0 = FLT_MAX, d1 = FLT_MAX;
     uint32_t c0 = kInvalid, c1 = kInvalid;
 #pragma unroll
-    for (int k = 0; k < kTop; k++) {
-        const float dk = exact[t * kTop + k];
-        const uint32_t ck = cand[t * kTop + k];
-        const bool lt0 = dk < d0 || (dk == d0 && ck < c0);
-        const bool lt1 = dk < d1 || (dk == d1 && ck < c1);
-        if (lt0) {
-            d1 = d0; c1 = c0;
-            d0 = dk; c0 = ck;
-        } else if (lt1) {
-            d1 = dk; c1 = ck;
+    for (int hh = 0; hh < 2; hh++) {
+        const uint32_t from = lane_first[t + 32 * hh], n = lane_pairs[t + 32 * hh];
+#pragma unroll
+        for (uint32_t k = 0; k < kKeep; k++)
+            if (k < n) nearest_two(exact[from + k], pairs[from + k] & 0xffffu, d0, c0, d1, c1);
+    }
+    // A point with more than kKeep centroids within the band in one half (near-coincident centroids): every centroid
+    // is measured, eight at a time by the same groups of 8 lanes, and the groups' nearest two are combined.
+    uint64_t crowded_points = ballot(crowded);
+    crowded_points = (crowded_points | (crowded_points >> 32)) & 0xffffffffull;
+    while (crowded_points) {
+        const int fp = __ffsll(static_cast<long long>(crowded_points)) - 1;
+        crowded_points &= crowded_points - 1;
+        const uint32_t pt = wave_base + fp;
+        const float* xrow = a.data + static_cast<size_t>(pt < a.num ? pt : last) * a.dim;
+        float bd0 = FLT_MAX, bd1 = FLT_MAX;
+        uint32_t bc0 = kInvalid, bc1 = kInvalid;
+        for (uint32_t cbase = 0; cbase < a.centroid_num; cbase += 8) {
+            const uint32_t cid = cbase + g;
+            const float* crow = a.centroids + static_cast<size_t>(cid < a.centroid_num ? cid : 0u) * a.dim;
+            float part = 0.f;
+            for (uint32_t dd = t8 * 4; dd < a.dim; dd += 32)
+                part = sqdist4(*reinterpret_cast<const float4*>(xrow + dd), *reinterpret_cast<const float4*>(crow + dd), part);
+            const float sq = row_sum<1>(part);
+            if (cid < a.centroid_num) nearest_two(finish_distance(sq, a.metric), cid, bd0, bc0, bd1, bc1);
+        }
+#pragma unroll
+        for (int m = 8; m <= 32; m <<= 1) {   // the eight groups hold disjoint sets of centroids
+            const float od0 = __shfl_xor(bd0, m), od1 = __shfl_xor(bd1, m);
+            const uint32_t oc0 = __shfl_xor(bc0, m), oc1 = __shfl_xor(bc1, m);
+            nearest_two(od0, oc0, bd0, bc0, bd1, bc1);
+            nearest_two(od1, oc1, bd0, bc0, bd1, bc1);
+        }
+        if (lane == fp) {
+            d0 = bd0; c0 = bc0;
+            d1 = bd1; c1 = bc1;
         }
     }
     (void) c1;
@@ -248,7 +328,7 @@ __global__ __launch_bounds__(256) void assign_kernel(AssignArgs a) {
 // after the one barrier that publishes it the four wavefronts run without meeting again.  Each wavefront issues
 // the loads of all its 32 points at once (coalesced, 16 KB in flight at 128 dims), passes them chunk by chunk
 // through a private LDS tile into the matrix-instruction operand layout and KEEPS those operand registers, so the
-// exact rescoring of the kTop best centroids reads no point a second time: lane (i, half) rescans its half of
+// exact pass over the centroids the ranking leaves reads no point a second time: lane (i, half) rescans its half of
 // row i against centroid rows in LDS and the two halves are added.
 template <int NQ>
 __global__ __launch_bounds__(256) void assign_resident_kernel(AssignArgs a) {
@@ -257,7 +337,8 @@ __global__ __launch_bounds__(256) void assign_resident_kernel(AssignArgs a) {
     constexpr int CS = DP + 4;            // centroid row stride
     float* cent = smem;                                            // [32][CS], zero outside centroid_num x dim
     float* x_tile = cent + 32 * CS;                                // [4 waves][32][kLdsStride]
-    uint32_t* hist = reinterpret_cast<uint32_t*>(x_tile + 4 * 32 * kLdsStride);   // [C + 1]
+    float* cnorm = x_tile + 4 * 32 * kLdsStride;                   // [32]: ||c||^2, +inf beyond centroid_num
+    uint32_t* hist = reinterpret_cast<uint32_t*>(cnorm + 32);      // [C + 1]
 
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
@@ -281,6 +362,7 @@ __global__ __launch_bounds__(256) void assign_resident_kernel(AssignArgs a) {
                                                  : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256) hist[i] = 0;
+    if (threadIdx.x < 32) cnorm[threadIdx.x] = threadIdx.x < a.centroid_num ? a.centroid_norms[threadIdx.x] : __builtin_inff();
     __syncthreads();
 
     float16v acc;
@@ -297,88 +379,69 @@ __global__ __launch_bounds__(256) void assign_resident_kernel(AssignArgs a) {
         for (int q = 0; q < 4; q++) {
             xr[c][q] = *reinterpret_cast<const float4*>(xw + t * kLdsStride + q * 8 + 4 * half);
             const float4 bv = *reinterpret_cast<const float4*>(cent + t * CS + c * 32 + q * 8 + 4 * half);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].x, bv.x, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].y, bv.y, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].z, bv.z, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xr[c][q].w, bv.w, acc, 0, 0, 0);
+            // centroids as the A operand, points as B: lane (t, half) ends with the scores of point t
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bv.x, xr[c][q].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bv.y, xr[c][q].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bv.z, xr[c][q].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(bv.w, xr[c][q].w, acc, 0, 0, 0);
         }
         __builtin_amdgcn_wave_barrier();
     }
 
-    // ranking: score = ||c||^2 - 2 x.c through this wave's tile (now free), kTop best per point
-    float* sw = xw;   // [32][33]
-    float best_s[kTop];
-    uint32_t best_c[kTop];
+    // ---- ranking in registers (see assign_band): accumulator r belongs to centroid 8*(r/4) + 4*half + r%4 and point t.
+    // The two smallest scores of the point, then the centroids within the band of the second smallest as a bit mask
+    // (bit = centroid id) that both lanes of the point share.
+    float xsq = 0.f;
 #pragma unroll
-    for (int k = 0; k < kTop; k++) {
-        best_s[k] = FLT_MAX;
-        best_c[k] = kInvalid;
-    }
-    auto offer = [&](float sc, uint32_t c) {
+    for (int c = 0; c < NQ; c++)
 #pragma unroll
-        for (int k = 0; k < kTop; k++) {
-            if (sc < best_s[k]) {
-                const float ts = best_s[k];
-                const uint32_t tc = best_c[k];
-                best_s[k] = sc;
-                best_c[k] = c;
-                sc = ts;
-                c = tc;
-            }
+        for (int q = 0; q < 4; q++)
+            xsq = fmaf(xr[c][q].x, xr[c][q].x, fmaf(xr[c][q].y, xr[c][q].y, fmaf(xr[c][q].z, xr[c][q].z, fmaf(xr[c][q].w, xr[c][q].w, xsq))));
+    xsq += lane_xor<32>(xsq);
+    float max_cn = t < static_cast<int>(a.centroid_num) ? cnorm[t] : 0.f;
+#pragma unroll
+    for (int m = 16; m >= 1; m >>= 1) max_cn = fmaxf(max_cn, __shfl_xor(max_cn, m));
+    float sc[16];
+    float m1 = __builtin_inff(), m2 = __builtin_inff();   // m1 <= m2
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const float4 c4 = *reinterpret_cast<const float4*>(cnorm + 8 * q + 4 * half);
+        const float cn[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            sc[4 * q + m] = fmaf(-2.f, acc[4 * q + m], cn[m]);   // +inf beyond centroid_num
+            m2 = __builtin_amdgcn_fmed3f(m1, m2, sc[4 * q + m]);
+            m1 = fminf(m1, sc[4 * q + m]);
         }
-    };
-    {
-        const uint32_t j = t;
-        const float cn = j < a.centroid_num ? a.centroid_norms[j] : 0.f;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int i = 8 * (r / 4) + 4 * half + (r % 4);   // accumulator layout of the 32x32 tile
-            sw[i * 33 + t] = j < a.centroid_num ? cn - 2.f * acc[r] : FLT_MAX;
-        }
-        __builtin_amdgcn_wave_barrier();
-        // the valid columns are shared out evenly between the two lanes of a point
-        const uint32_t per = (a.centroid_num + 1) / 2, col0 = half * per;
-#pragma unroll 4
-        for (uint32_t jj = 0; jj < per; jj++) offer(sw[t * 33 + col0 + jj], col0 + jj);
     }
     {
-        float os[kTop];
-        uint32_t oc[kTop];
-#pragma unroll
-        for (int k = 0; k < kTop; k++) {
-            os[k] = lane_xor<32>(best_s[k]);
-            oc[k] = lane_xor<32>(best_c[k]);
-        }
-#pragma unroll
-        for (int k = 0; k < kTop; k++) offer(os[k], oc[k]);
+        const float o1 = lane_xor<32>(m1), o2 = lane_xor<32>(m2);
+        m2 = fminf(fmaxf(m1, o1), fminf(m2, o2));
+        m1 = fminf(m1, o1);
     }
-    // Both lanes of a point must rescore the same candidates in the same order: equal scores could have been
-    // ranked differently by the two halves, so the upper half takes the lower half's list.
+    const float limit = fminf(m2 + assign_band(a.dim, xsq, max_cn), FLT_MAX);   // one centroid only: every valid score passes
+    uint32_t within = 0;
 #pragma unroll
-    for (int k = 0; k < kTop; k++) best_c[k] = static_cast<uint32_t>(__shfl(static_cast<int>(best_c[k]), t));
+    for (int r = 0; r < 16; r++)
+        if (sc[r] <= limit) within |= 1u << (8 * (r / 4) + (r % 4));
+    within <<= 4 * half;
+    within |= lane_xor<32>(within);
 
-    // exact rescoring from the kept registers; smallest two by (distance, centroid id)
+    // exact distances of those centroids from the kept registers, lowest id first; smallest two by (distance, centroid id)
     float d0 = FLT_MAX, d1 = FLT_MAX;
     uint32_t c0 = kInvalid, c1 = kInvalid;
-#pragma unroll
-    for (int k = 0; k < kTop; k++) {
-        const uint32_t ck = best_c[k];
-        const float* crow = cent + (ck != kInvalid ? ck : 0u) * CS + 4 * half;
+    while (ballot(within != 0)) {
+        const bool have = within != 0;
+        const uint32_t ck = have ? static_cast<uint32_t>(__ffs(static_cast<int>(within))) - 1u : 0u;
+        within &= within - 1;
+        const float* crow = cent + ck * CS + 4 * half;
         float part = 0.f;
 #pragma unroll
         for (int c = 0; c < NQ; c++)
 #pragma unroll
             for (int q = 0; q < 4; q++) part = sqdist4(xr[c][q], *reinterpret_cast<const float4*>(crow + c * 32 + q * 8), part);
         const float sq = part + lane_xor<32>(part);
-        const float dk = ck != kInvalid ? finish_distance(sq, a.metric) : FLT_MAX;
-        const bool lt0 = dk < d0 || (dk == d0 && ck < c0);
-        const bool lt1 = dk < d1 || (dk == d1 && ck < c1);
-        if (lt0) {
-            d1 = d0; c1 = c0;
-            d0 = dk; c0 = ck;
-        } else if (lt1) {
-            d1 = dk; c1 = ck;
-        }
+        if (have) nearest_two(finish_distance(sq, a.metric), ck, d0, c0, d1, c1);
     }
     (void) c1;
 
@@ -401,7 +464,7 @@ __global__ __launch_bounds__(256) void assign_resident_kernel(AssignArgs a) {
 }
 
 size_t assign_resident_lds_bytes(int nq, uint32_t centroid_num) {
-    return (static_cast<size_t>(32) * (32 * nq + 4) + 4 * 32 * kLdsStride) * sizeof(float) + (centroid_num + 1) * sizeof(uint32_t);
+    return (static_cast<size_t>(32) * (32 * nq + 4) + 4 * 32 * kLdsStride + 32) * sizeof(float) + (centroid_num + 1) * sizeof(uint32_t);
 }
 
 // exclusive scan over tiles, one workgroup per bin; also emits the bin totals (segment lengths)
@@ -778,7 +841,7 @@ __global__ void kmeans_update_kernel(float* centroids, const long long* sums, co
 }
 
 size_t assign_lds_bytes(int cb, uint32_t centroid_num) {
-    return (static_cast<size_t>(32) * cb * kLdsStride + 4 * 32 * kLdsStride + 4 * 32 * 33) * sizeof(float) + (centroid_num + 1) * sizeof(uint32_t);
+    return (static_cast<size_t>(32) * cb * kLdsStride + 4 * 32 * kLdsStride + 32 * cb) * sizeof(float) + (centroid_num + 1) * sizeof(uint32_t);
 }
 
 }  // namespace glide

@@ -64,6 +64,36 @@ def test_assign_matches_oracle(hip, n, dim, c, metric):
         assert np.array_equal(g_idx, e_idx) and np.array_equal(g_len, e_len)
 
 
+@pytest.mark.parametrize("n,dim,c,copies", [(1500, 128, 48, 12), (600, 64, 200, 200), (500, 256, 40, 9), (700, 128, 256, 6)])
+def test_assign_coincident_centroids(hip, n, dim, c, copies):
+    """Centroids that coincide: more candidates tie for the two nearest than the ranking pass hands on per lane, so the
+    points near them are measured against every centroid.  Integer rows make every distance exact: the two nearest
+    distances and the boundary flags must be the oracle's to the bit.  Between centroids at exactly the same distance
+    the reference's choice falls out of its bitonic network; here the smaller centroid id wins."""
+    from oracle import oracle as O
+    data = lowdim_data(n, dim, seed=n + c)
+    centroids = O.kmeans(data, c, iterations=3)
+    centroids = np.round(centroids).astype(np.float32)
+    rng = np.random.default_rng(c)
+    where = rng.permutation(c)[:copies]
+    centroids[where] = centroids[where[0]]
+    e_idx, e_len, e_near = O.partition_assign(data, centroids, 1.04, 0)
+    _, seg_idx, g_len, g_near = gpu_assign(hip, data, centroids, 1.04, 0)
+    g_idx = seg_idx.numpy()
+    assert np.array_equal(g_near, e_near)
+    assert np.array_equal(g_idx[:, 2], e_idx[:, 2]) and g_len[c] == e_len[c]
+    tied = e_near[:, 0] == e_near[:, 1]
+    assert np.array_equal(g_idx[~tied, 0], e_idx[~tied, 0])
+    assert tied.sum() > 0
+    for p in np.nonzero(tied)[0]:
+        d = np.sqrt(((data[p] - centroids) ** 2).sum(1, dtype=np.float32))
+        assert g_idx[p, 0] == np.nonzero(d == d.min())[0][0], p
+    assert (g_idx[tied, 0] == where.min()).any()
+    for s_ in range(c):
+        members = np.nonzero(g_idx[:, 0] == s_)[0]
+        assert np.array_equal(g_idx[members, 1], np.arange(members.size)) and g_len[s_] == members.size
+
+
 def test_assign_brute_force_float64(hip):
     # independent of the oracle: float64 argmin and ratio with a margin
     rng = np.random.default_rng(0)
