@@ -227,15 +227,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (uint32_t k = 0; k < mine; k++) pairs[first + k] = (static_cast<uint32_t>(t) << 16) | cand_by_lane[lane * kKeep + k];
     __builtin_amdgcn_wave_barrier();
 
-    // ---- exact distances of the pairs: one pair per group of 8 lanes, four steps (32 pairs) in flight
+    // ---- exact distances of the pairs: one pair per group of 8 lanes, kExactSteps steps in flight.  With eight blocks
+    // that is 96 pairs, more than a wavefront usually has, so the pass costs dim / 32 memory round trips and not three
+    // times that: the 128 accumulators are dead by now and their registers hold the rows on their way in.  With fewer
+    // blocks the registers are worth more as a further wavefront per SIMD.
+    constexpr int kExactSteps = CB >= 8 ? 12 : 4;
     const int g = lane >> 3, t8 = lane & 7;
     const uint32_t last = a.num - 1;
-    for (uint32_t s0 = 0; s0 < pair_count; s0 += 32) {
-        const float* xr[4];
-        const float* cr[4];
-        float part[4];
+    for (uint32_t s0 = 0; s0 < pair_count; s0 += 8 * kExactSteps) {
+        const float* xr[kExactSteps];
+        const float* cr[kExactSteps];
+        float part[kExactSteps];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kExactSteps; u++) {
             const uint32_t pair = s0 + u * 8 + g;
             const uint32_t pc = pairs[pair < pair_count ? pair : 0u];
             const uint32_t pt = wave_base + (pc >> 16);
@@ -244,17 +248,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
             part[u] = 0.f;
         }
         for (uint32_t d0 = t8 * 4; d0 < a.dim; d0 += 32) {
-            float4 xv[4], cv[4];
+            float4 xv[kExactSteps], cv[kExactSteps];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < kExactSteps; u++) {
                 xv[u] = *reinterpret_cast<const float4*>(xr[u] + d0);
                 cv[u] = *reinterpret_cast<const float4*>(cr[u] + d0);
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) part[u] = sqdist4(xv[u], cv[u], part[u]);
+            for (int u = 0; u < kExactSteps; u++) part[u] = sqdist4(xv[u], cv[u], part[u]);
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kExactSteps; u++) {
             const uint32_t pair = s0 + u * 8 + g;
             const float sq = row_sum<1>(part[u]);   // 8-lane groups
             if (t8 == 0 && pair < pair_count) exact[pair] = finish_distance(sq, a.metric);
