@@ -325,6 +325,12 @@ __device__ __forceinline__ bool lds_set_insert(uint32_t* table, uint32_t key) { 
 // No filtering of offers against the target's current list: the reference also explores offers that do not enter
 // the list (they are the "new" samples of the next round, nn_descent.cuh:973-1001).
 
+// Row (of a pass of 32) that thread `tid` of the workgroup stages: groups of 8 lanes 0, 1, 2, 3 ... take rows 0, 8, 1, 9 ...
+__device__ __forceinline__ uint32_t staged_row(int tid) {
+    const uint32_t g = static_cast<uint32_t>(tid) >> 3;
+    return ((g & 1u) << 3) | ((g >> 1) & 7u) | (g & 16u);
+}
+
 // A (rows) x B (rows) dot products of one chunk of dims for this wave's 32 x 32 quadrant.
 // v_mfma_f32_32x32x16_f16 (gfx950): lane supplies A[i = lane%32][k = 8*(lane/32) .. +7] and B[k = same][j = lane%32].
 __device__ __forceinline__ void mfma_chunk(float16v& acc, const _Float16 (*A)[kRowHalfs], const _Float16 (*B)[kRowHalfs], int rb, int cb, int lane) {
@@ -481,13 +487,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     const bool need_no = (rb * 32 < static_cast<int>(n_new)) && (cb * 32 < static_cast<int>(n_old));
 
     // Chunks of kJoinChunk dims go global -> registers -> LDS: 8 lanes x 16 B per row and chunk, 32 rows per pass (new
-    // rows, then old rows).  The loads of chunk k+1 are issued before the matrix instructions of chunk k.  Short chunks
+    // rows, then old rows).  The two rows that 16 adjacent lanes store together are eight apart: with the row stride of
+    // 36 words they then fall on opposite halves of the 64 banks (adjacent rows would overlap by four banks).  The loads of chunk k+1 are issued before the matrix instructions of chunk k.  Short chunks
     // keep the workgroup at 20 KB of LDS, so six of them share a CU instead of four.
     float4 pre[4];
     auto prefetch = [&](uint32_t k0) {
 #pragma unroll
         for (int pass = 0; pass < 4; pass++) {
-            const uint32_t r = pass * 32 + (tid >> 3), q = tid & 7;
+            const uint32_t r = pass * 32 + staged_row(tid), q = tid & 7;
             const bool old_row = r >= 64;
             const uint32_t rr = r & 63;
             const uint32_t d0 = k0 + q * 8;
@@ -508,7 +515,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         if (k0) __syncthreads();   // every wave is done with the previous chunk
 #pragma unroll
         for (int pass = 0; pass < 4; pass++) {
-            const uint32_t r = pass * 32 + (tid >> 3), q = tid & 7;
+            const uint32_t r = pass * 32 + staged_row(tid), q = tid & 7;
             *reinterpret_cast<float4*>(&(r >= 64 ? L.rows.xo : L.rows.xn)[r & 63][q * 8]) = pre[pass];
         }
         __syncthreads();
