@@ -491,6 +491,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     // 36 words they then fall on opposite halves of the 64 banks (adjacent rows would overlap by four banks).  The loads of chunk k+1 are issued before the matrix instructions of chunk k.  Short chunks
     // keep the workgroup at 20 KB of LDS, so six of them share a CU instead of four.
     float4 pre[4];
+    // Norm and offer threshold of a row are asked for with its first chunk and stored with it (a store right behind the
+    // load would make the wavefront wait for every pass in turn).  Lane q of a row's group takes pass q, so a lane
+    // holds one pair.
+    float2 pre_norm = make_float2(0.f, 0.f);
     auto prefetch = [&](uint32_t k0) {
 #pragma unroll
         for (int pass = 0; pass < 4; pass++) {
@@ -502,11 +506,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
             if (rr < (old_row ? n_old : n_new)) {
                 const uint32_t id = (old_row ? L.old_ids : L.new_ids)[rr];
                 if (d0 < a.dim_pad) pre[pass] = *reinterpret_cast<const float4*>(a.half_rows + static_cast<size_t>(seg_start + id) * a.dim_pad + d0);
-                if (k0 == 0 && q == 0) {   // same round trip as the row
-                    const float2 nt = a.norms[seg_start + id];
-                    (old_row ? L.old_norms : L.new_norms)[rr] = nt.x;
-                    (old_row ? L.old_thr : L.new_thr)[rr] = __float_as_uint(nt.y);
-                }
+                if (k0 == 0 && q == static_cast<uint32_t>(pass)) pre_norm = a.norms[seg_start + id];   // same round trip as the row
             }
         }
     };
@@ -517,6 +517,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         for (int pass = 0; pass < 4; pass++) {
             const uint32_t r = pass * 32 + staged_row(tid), q = tid & 7;
             *reinterpret_cast<float4*>(&(r >= 64 ? L.rows.xo : L.rows.xn)[r & 63][q * 8]) = pre[pass];
+            if (k0 == 0 && q == static_cast<uint32_t>(pass) && (r & 63) < (r >= 64 ? n_old : n_new)) {
+                (r >= 64 ? L.old_norms : L.new_norms)[r & 63] = pre_norm.x;
+                (r >= 64 ? L.old_thr : L.new_thr)[r & 63] = __float_as_uint(pre_norm.y);
+            }
         }
         __syncthreads();
         if (k0 + kJoinChunk < a.dim_pad) prefetch(k0 + kJoinChunk);
