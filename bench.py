@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 SWEEP_BEAMS = (32, 64, 128, 256, 512)       # the reference accepts beams up to 512 (kernel_config.cuh:41-60)
 NAMED_BEAMS = {"cfg1": (32, 64, 128, 256)}  # the medium configuration names its beams; 512 is swept there as an extra
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "search_kernels_hbm_traffic.md")
-VALU_PROFILE = os.path.join(ROOT, "profiles", "build_refine_kernels_cfg1_counters.md")
+VALU_PROFILE = os.path.join(ROOT, "profiles", "build_refine_kernels_counters.md")
 
 
 def measured_traffic(workload, beam):
@@ -50,18 +50,19 @@ def measured_traffic(workload, beam):
     return None
 
 
-def measured_valu(kernel, workload):
-    """(vector-ALU wave instructions one point costs in `kernel`, the chip's issue rate for that kind of instruction in
-    G wave instructions / s), from the committed counter summary of the build kernels (SQ_INSTS_VALU per launch over the
-    points of the launch; the rate is what --valu-calibration measures for compare + select).  Rows read
-    `| kernel | workload | instructions per point | yardstick |`; None for a pair the file does not hold."""
+def measured_stage(stage, workload):
+    """(vector-ALU wave instructions, FETCH_SIZE KiB, vector-ALU yardstick in G wave instructions / s, fetch scale) of one
+    build stage (all launches of `build_kernel`, or the launch of `refine_kernel`) on one workload, from the committed
+    counter summary: SQ_INSTS_VALU and FETCH_SIZE per launch from `rocprofv3 --pmc` runs of this script, the yardstick
+    from --valu-calibration (compare + select), the scale from --copy-calibration.  The builds are reproducible, so the
+    counts belong to the workload, not to a run.  None for a pair the file does not hold."""
     try:
         text = open(VALU_PROFILE).read()
     except OSError:
         return None
-    for m in re.finditer(r"^\|\s*(\w+)\s*\|\s*([\w-]+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*$", text, re.M):
-        if m.group(1) == kernel and m.group(2) == workload:
-            return float(m.group(3)), float(m.group(4))
+    for m in re.finditer(r"^\|\s*([\w+]+)\s*\|\s*([\w-]+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*$", text, re.M):
+        if m.group(1) == stage and m.group(2) == workload:
+            return float(m.group(3)), float(m.group(4)), float(m.group(5)), float(m.group(6))
     return None
 
 
@@ -236,20 +237,23 @@ def run_workload(args, workload, torch, want_cpu):
         out = dict(bound="hbm", seconds=seconds, algorithmic_bytes=int(nbytes), achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s", frac=gbs / HBM_PEAK_GBS)
         return out
 
-    def valu_stage(seconds, nbytes, kernel, points):
-        """The per-point graph kernels score rows that sit in L2 (hit rate 0.96 in the counters) and spend their time
-        issuing vector instructions (sorting networks, cross-lane sums, distances): their ceiling is the vector-ALU
-        issue rate, and the bytes their algorithm names, which one partition's cache serves many times over, are
-        reported beside it without a fraction."""
-        out = dict(bound="valu", seconds=seconds, kernel=kernel, points=int(points), unit="G wave instructions/s",
-                   algorithmic_bytes=int(nbytes), algorithmic_GBps=nbytes / seconds / 1e9 if seconds > 0 else 0.0)
-        m = measured_valu(kernel, workload)
+    def graph_stage(seconds, nbytes, stage):
+        """The per-point graph kernels are bound by vector-ALU issue where their searches stay in cache (the sorting
+        networks, cross-lane sums and distances of the beam loop) and by HBM where they do not; the committed counters
+        say which.  The bytes their algorithm names, which a partition's cache may serve many times over, are reported
+        beside it without a fraction."""
+        out = dict(seconds=seconds, algorithmic_bytes=int(nbytes), algorithmic_GBps=nbytes / seconds / 1e9 if seconds > 0 else 0.0)
+        m = measured_stage(stage, workload)
         if m and seconds > 0:
-            out.update(instructions_per_point=m[0], achieved=m[0] * points / seconds / 1e9, peak=m[1], frac=m[0] * points / seconds / 1e9 / m[1],
+            instructions, fetch_kib, yardstick, scale = m
+            valu, hbm = instructions / seconds / 1e9, fetch_kib * 1024 * scale / seconds / 1e9
+            by_valu = valu / yardstick >= hbm / HBM_PEAK_GBS
+            out.update(bound="valu" if by_valu else "hbm", achieved=valu if by_valu else hbm, peak=yardstick if by_valu else HBM_PEAK_GBS,
+                       unit="G wave instructions/s" if by_valu else "GB/s", frac=max(valu / yardstick, hbm / HBM_PEAK_GBS),
+                       valu_G_wave_instructions_per_s=valu, valu_frac=valu / yardstick, hbm_GBps=hbm, hbm_frac=hbm / HBM_PEAK_GBS,
                        source="profiles/" + os.path.basename(VALU_PROFILE))
         else:
-            out.update(instructions_per_point=None, achieved=None, peak=None, frac=None,
-                       note="no SQ_INSTS_VALU count committed for this kernel on this workload")
+            out.update(bound=None, achieved=None, peak=None, frac=None, note="no counters committed for this stage on this workload")
         return out
 
     stage_rooflines = {}
@@ -259,13 +263,12 @@ def run_workload(args, workload, torch, want_cpu):
     stage_rooflines["reorder"] = hbm_stage(det["reorder"], (num + reorder_rows) * dim * 4)
     if "build_counters" in res:
         _, rows, grows = res["build_counters"]
-        stage_rooflines["subgraph+boundary"] = valu_stage(det["subgraph"] + det["boundary"],
-                                                          reorder_rows * dim * 4 + grows * knn_degree * 4 + rows * dim * 4 + reorder_rows * degree * 4,
-                                                          "build_kernel", num)   # the boundary launch adds 0.3% to the count
+        stage_rooflines["subgraph+boundary"] = graph_stage(det["subgraph"] + det["boundary"],
+                                                           reorder_rows * dim * 4 + grows * knn_degree * 4 + rows * dim * 4 + reorder_rows * degree * 4,
+                                                           "subgraph+boundary")
     if "refine_counters" in res:
         _, rows, grows = res["refine_counters"]
-        stage_rooflines["refine"] = valu_stage(det["refine"], num * dim * 4 + 2 * num * degree * 4 + grows * degree * 4 + rows * dim * 4,
-                                               "refine_kernel", num)
+        stage_rooflines["refine"] = graph_stage(det["refine"], num * dim * 4 + 2 * num * degree * 4 + grows * degree * 4 + rows * dim * 4, "refine")
 
     out = dict(
         workload=desc, gen_sec=gen_s, build_sec=build_sec, stage_rooflines=stage_rooflines,
