@@ -454,6 +454,11 @@ def main():
             res = run_workload(args, name, torch, want_cpu=not args.no_cpu)
             line["other_configs"][name] = {k: res[k] for k in keys if k in res}
             line["other_configs"][name]["wall_sec"] = time.time() - t0
+        # where the metric's operating point (recall@10 >= 0.95) exists in this run: workload -> (beam, QPS, roofline fraction)
+        line["recall_target_met_on"] = {
+            name: dict(beam=r["beam"], qps=r["qps"], recall_at_10=r["recall_at_10"], roofline_frac=r["roofline"]["frac"])
+            for name, r in [("cfg1", main_res), ("cfg1-navigable", nav)] + [(n, line["other_configs"][n]) for n in ("cfg0", "cfg2", "cfg3")]
+            if r["recall_target_met"]}
     print(json.dumps(line, default=float))
 
 
