@@ -7,8 +7,8 @@
 // What is kept: fp16 rows with fp32 squared norms, <= 32 new + <= 32 old forward samples per node, reverse
 // samples capped at 32, a 64 x 64 distance tile per phase (new x new, new x old) computed on the matrix cores
 // with the norm-trick epilogue, and one offer per row / column (its nearest partner) per phase.
-// What is different: the kNN lists, flags, Bloom filters and samples never leave HBM.  An offer is one 64-bit atomic
-// minimum on a slot of its target's table (no locks, nothing returned); reverse samples go to plain per-node lists with
+// What is different: the kNN lists, flags, Bloom filters and samples never leave HBM.  An offer is a pair of 64-bit
+// atomic minima on two slots of its target's table (no locks, nothing returned); reverse samples go to plain per-node lists with
 // an overflow table that keeps the smallest sources.  What a node holds at the end of a round -- all that the
 // reference's 32-wide device list and its 32 reverse samples would be drawn from -- is the same whatever the order of
 // arrival, so a build is reproducible.  A merge kernel then applies the reference's rules: of a node's offers the
@@ -202,15 +202,15 @@ constexpr uint32_t kRevCap = 64;         // reverse samples per node, kind and r
 // Row stride of the reverse lists, in entries.  Arrivals fill a row from its start, so with a power-of-two stride
 // (256 B) the busy front parts of all rows would sit on the same few memory channels.
 constexpr uint32_t kRevStride = kRevCap + 8;
-// Offers of a round: per node a table of 256 (distance bits : candidate id) keys.  An offer goes to the slot its
-// candidate's id hashes to and stays if it is the smallest key that slot has seen this round (one 64-bit atomic
-// minimum without a return value).  Copies of one offer, found by several joins, are the same key and fall together;
-// two different candidates in one slot leave the nearer one.  What the table holds at the end of the round does not
-// depend on the order of arrival.
+// Offers of a round: per node a table of (distance bits : candidate id) keys, 256 slots for lists of one sub-list, 512
+// for lists of several.  An offer goes to two slots of one 16-slot (128-byte) line of its target's table, both chosen
+// by hashes of the candidate's id, and stays in each if it is the smallest key that slot has seen this round (64-bit
+// atomic minima without a return value).  Copies of one offer, found by several joins, are the same key and fall
+// together; two different candidates in one slot leave the nearer one, and an offer is lost only if both its slots
+// hold nearer candidates (about one of a node's best 32 in ten rounds; with a single slot it was two a round, which
+// showed as a lag of 1.4 points of graph recall in the first rounds).  What the table holds at the end of the round
+// does not depend on the order of arrival.
 constexpr uint32_t kOfferSlotsNarrow = 256, kOfferSlotsWide = 512;   // lists of one sub-list; of several (SLOTS below)
-// With several sub-lists an offer is sent to two slots (two hashes of its candidate) and is lost only if both hold a
-// nearer candidate: those lists are filled 32 offers a round, and each one that a fixed number of rounds loses shows in
-// the graph.  A single sub-list converges to the same graph either way (measured), and one atomic per offer is faster.
 __host__ __device__ constexpr uint32_t offer_slots_for(uint32_t width) { return width > 32 ? kOfferSlotsWide : kOfferSlotsNarrow; }
 constexpr uint32_t kRevSlots = 256;      // overflow table per node and kind: 16 buckets of source ids
 constexpr unsigned long long kNoOffer = ~0ull;
@@ -225,7 +225,10 @@ __device__ __forceinline__ uint32_t first_slot(uint32_t hash) { return __umulhi(
 // Slot of a candidate in an offer table.  The salt changes with the round, so two candidates that share a slot in one
 // round do not share it in the next.
 __device__ __forceinline__ uint32_t offer_slot(uint32_t cand, uint32_t salt, uint32_t shift) { return id_hash(cand ^ salt) >> shift; }
-__device__ __forceinline__ uint32_t offer_slot2(uint32_t cand, uint32_t salt, uint32_t shift) { return ((cand ^ salt) * 0xC2B2AE35u) >> shift; }
+// the second slot in the 16-slot (128-byte) line of the first: another of its 15 positions
+__device__ __forceinline__ uint32_t offer_slot_beside(uint32_t first, uint32_t cand, uint32_t salt) {
+    return (first & ~15u) | ((first + 1u + __umulhi((cand ^ salt) * 0xC2B2AE35u, 15u)) & 15u);
+}
 __device__ __forceinline__ uint32_t round_salt(uint32_t round) { return round * 0x85EBCA6Bu; }
 
 // One source id into a reverse overflow table (256 words).  The bound is read first: a table only comes into play for
@@ -285,7 +288,7 @@ struct JoinArgs {
     uint32_t* rev_thr;             // num x 2: sources not below it stay away in the next scatter (all ones: none)
     uint32_t* counts;              // num x 4: forward new / old, reverse new / old arrivals (restarted by the join)
     unsigned long long* offers;    // num x offer_slots: the offer tables
-    uint32_t offer_slots, slot_shift, two_slots;   // slot_shift = 32 - log2(offer_slots)
+    uint32_t offer_slots, slot_shift;   // slot_shift = 32 - log2(offer_slots)
     const uint32_t* round;         // rounds completed so far (salt of the slot hash)
     unsigned long long* stats;     // striped: [1] offers that stayed away because of their target's threshold (nullable)
     uint32_t num, dim_pad;
@@ -552,7 +555,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         }
     }
     __syncthreads();
-    // An offer is one atomic minimum on its slot of the target's table; nothing comes back, so the wave does not wait.
+    // An offer is two atomic minima on slots of one line of the target's table; nothing comes back, so the wave does not wait.
     const uint32_t salt = round_salt(*a.round);
     uint32_t declined = 0;
     auto send = [&](uint32_t target, uint32_t cand, float dist, uint32_t thr) {
@@ -563,9 +566,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         }
         const unsigned long long key = (static_cast<unsigned long long>(__float_as_uint(dist)) << 32) | cand;
         unsigned long long* row = a.offers + (static_cast<size_t>(seg_start) + target) * a.offer_slots;
-        const uint32_t s1 = offer_slot(cand, salt, a.slot_shift), s2 = offer_slot2(cand, salt, a.slot_shift);
+        const uint32_t s1 = offer_slot(cand, salt, a.slot_shift), s2 = offer_slot_beside(s1, cand, salt);
         __hip_atomic_fetch_min(&row[s1], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (a.two_slots && s2 != s1) __hip_atomic_fetch_min(&row[s2], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_min(&row[s2], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
     {
         float best;
@@ -1278,7 +1281,7 @@ int nnd_join(const NndCtx& c, bool with_stats) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
     JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.offers, offer_slots_for(c.l.width),
-                offer_slots_for(c.l.width) == 512 ? 23u : 24u, c.l.width > 32 ? 1u : 0u, c.round, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
+                offer_slots_for(c.l.width) == 512 ? 23u : 24u, c.round, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
     hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja);
     return launch_status();
 }

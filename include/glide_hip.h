@@ -182,10 +182,11 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *                   reverse_cap (64) reverse samples in order of arrival; counts num x 4 u32 = their lengths (the reverse lengths count every arrival and may exceed
  *                   reverse_cap; the join uses the 32 smallest)
  *   offers     num x offer_slots u64 keys (distance bits << 32 | candidate id, all ones = empty): the offers of the
- *                   round.  offer_slots is 256 when the list is one sub-list (knn_degree <= 32) and 512 otherwise.  An
- *                   offer goes to slot (x * 0x9E3779B1) >> (32 - log2 offer_slots), x = candidate ^ round * 0x85EBCA6B,
- *                   of its target's row -- with 512 slots also to slot (x * 0xC2B2AE35) >> 23 -- and stays where it is
- *                   the smallest key the slot has seen (an atomic minimum): copies of one offer fall together, of two
+ *                   round.  offer_slots is 256 when the list is one sub-list (knn_degree <= 32) and 512 otherwise.  With
+ *                   x = candidate ^ round * 0x85EBCA6B, an offer goes to slot s1 = (x * 0x9E3779B1) >> (32 - log2
+ *                   offer_slots) of its target's row and to a second slot of the same 16-slot line,
+ *                   (s1 & ~15) | ((s1 + 1 + umulhi(x * 0xC2B2AE35, 15)) & 15), and stays in each where it is the
+ *                   smallest key the slot has seen (an atomic minimum): copies of one offer fall together, of two
  *                   candidates that share a slot the nearer one stays.  The merge reads the row, uses its 32 smallest
  *                   distinct keys and empties it.  `round` (one u32, raised by converge) changes the slots from round
  *                   to round.

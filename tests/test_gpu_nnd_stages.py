@@ -16,7 +16,7 @@ INV = 0xFFFFFFFF
 OLD = 0x80000000
 S = 32   # samples per list (NUM_SAMPLES, nn_descent.cuh:391)
 R = 256  # words of a reverse overflow table: 16 buckets of 15 slots + the bucket's bound
-SLOTS = 256  # slots of a node's offer table when the list is one sub-list; 512 with several, where every offer goes to two slots
+SLOTS = 256  # slots of a node's offer table when the list is one sub-list; 512 with several.  Every offer goes to two slots of one line
 RCAP = 64  # reverse samples a list holds before the overflow table takes over
 
 
@@ -85,14 +85,16 @@ def offers_held(st, node, distinct=True):
 
 def model_offer_table(keys, round_, slots=SLOTS):
     """What a node's offer table holds once `keys` (distance bits << 32 | candidate) have all been sent to it: a slot
-    keeps the smallest key it was sent.  A key goes to slot (x * 0x9E3779B1) >> (32 - log2 slots), x = candidate ^
-    round * 0x85EBCA6B, and in a table of 512 also to slot (x * 0xC2B2AE35) >> 23."""
+    keeps the smallest key it was sent.  With x = candidate ^ round * 0x85EBCA6B a key goes to slot
+    s1 = (x * 0x9E3779B1) >> (32 - log2 slots) and to a second slot of the same line of 16,
+    (s1 & ~15) | ((s1 + 1 + ((x * 0xC2B2AE35 mod 2^32) * 15 >> 32)) & 15)."""
     row = np.full(slots, NO_OFFER, np.uint64)
     salt = (round_ * 0x85EBCA6B) & 0xFFFFFFFF
     for key in keys:
         x, shift = (key & 0xFFFFFFFF) ^ salt, 32 - slots.bit_length() + 1
-        for mult in (0x9E3779B1, 0xC2B2AE35)[:2 if slots == 512 else 1]:
-            slot = ((x * mult) & 0xFFFFFFFF) >> shift
+        s1 = ((x * 0x9E3779B1) & 0xFFFFFFFF) >> shift
+        s2 = (s1 & ~15) | ((s1 + 1 + ((((x * 0xC2B2AE35) & 0xFFFFFFFF) * 15) >> 32)) & 15)
+        for slot in (s1, s2):
             if key < int(row[slot]):
                 row[slot] = np.uint64(key)
     return row
