@@ -47,7 +47,10 @@ __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float
                                            uint32_t first, uint32_t count, int lane, IdFn id_of, OutFn out) {
     using Shape = RowShape<DIMV>;
     const int g = Shape::row_of_lane(lane), t = Shape::lane_in_row(lane);
-    constexpr int U = DIMV == 1 ? 2 : (DIMV == 2 ? 2 : (DIMV == 4 ? 2 : 1));
+    // Steps in flight.  Rows of more than 512 dims are 2-4 KB each and a step holds only two of them: with one step in
+    // flight a wavefront had 8 KB on its way, too little to cover the memory latency when a launch has about one
+    // wavefront per SIMD (1 000 queries); four steps took the 960-dim beam-512 search from 16.8 to 13.2 ms.
+    constexpr int U = DIMV == 1 ? 2 : (DIMV == 2 ? 2 : (DIMV == 4 ? 2 : 4));
     for (uint32_t base = first; base < count; base += Shape::ROWS * U) {
         RowRegs<DIMV> rows[U];
 #pragma unroll
