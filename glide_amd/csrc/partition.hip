@@ -19,7 +19,7 @@ struct AssignArgs {
     const float* centroids;
     const float* centroid_norms;   // ||c||^2, fp32
     uint32_t* segment_indexes;     // num x 3: segment, (slot filled later), boundary flag as 0 / 0xffffffff
-    uint32_t* tile_hist;           // tiles x (C + 1)
+    uint32_t* tile_hist;           // (C + 1) x tiles: bin-major, so that the scan over tiles reads each bin as one run
     float* nearest_dists;          // num x 2 or null
     uint32_t num, dim, centroid_num;
     float boundary_factor;
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     }
     __syncthreads();
     for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256)
-        a.tile_hist[static_cast<size_t>(blockIdx.x) * (a.centroid_num + 1) + i] = hist[i];
+        a.tile_hist[static_cast<size_t>(i) * gridDim.x + blockIdx.x] = hist[i];
 }
 
 // Assignment for at most 32 centroids of at most 128 dims, the shape that is bound by reading the points once.
@@ -464,7 +464,7 @@ __global__ __launch_bounds__(256) void assign_resident_kernel(AssignArgs a) {
     }
     __syncthreads();
     for (uint32_t i = threadIdx.x; i <= a.centroid_num; i += 256)
-        a.tile_hist[static_cast<size_t>(blockIdx.x) * (a.centroid_num + 1) + i] = hist[i];
+        a.tile_hist[static_cast<size_t>(i) * gridDim.x + blockIdx.x] = hist[i];
 }
 
 size_t assign_resident_lds_bytes(int nq, uint32_t centroid_num) {
@@ -473,14 +473,15 @@ size_t assign_resident_lds_bytes(int nq, uint32_t centroid_num) {
 
 // exclusive scan over tiles, one workgroup per bin; also emits the bin totals (segment lengths)
 constexpr int kScanThreads = 1024;
-__global__ __launch_bounds__(kScanThreads) void tile_scan_kernel(uint32_t* tile_hist, uint32_t tiles, uint32_t bins, uint32_t* totals) {
+__global__ __launch_bounds__(kScanThreads) void tile_scan_kernel(uint32_t* tile_hist, uint32_t tiles, uint32_t* totals) {
     __shared__ uint32_t wave_total[kScanThreads / 64];
     const uint32_t bin = blockIdx.x;
     const int lane = lane_id(), wave = threadIdx.x >> 6;
     const uint32_t per = ceil_div(tiles, static_cast<uint32_t>(kScanThreads));
     const uint32_t begin = min(threadIdx.x * per, tiles), end = min(begin + per, tiles);
     uint32_t sum = 0;
-    for (uint32_t i = begin; i < end; i++) sum += tile_hist[static_cast<size_t>(i) * bins + bin];
+    uint32_t* const row = tile_hist + static_cast<size_t>(bin) * tiles;
+    for (uint32_t i = begin; i < end; i++) sum += row[i];
     uint32_t inclusive = sum;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -499,8 +500,8 @@ __global__ __launch_bounds__(kScanThreads) void tile_scan_kernel(uint32_t* tile_
     if (threadIdx.x == 0) totals[bin] = total;
     uint32_t run = before + inclusive - sum;
     for (uint32_t i = begin; i < end; i++) {
-        const uint32_t v = tile_hist[static_cast<size_t>(i) * bins + bin];
-        tile_hist[static_cast<size_t>(i) * bins + bin] = run;
+        const uint32_t v = row[i];
+        row[i] = run;
         run += v;
     }
 }
@@ -523,9 +524,9 @@ __global__ __launch_bounds__(kTilePoints) void slot_kernel(uint32_t* segment_ind
         rank += seg[j] == my_seg;
         brank += bnd[j] != kInvalid;
     }
-    const uint32_t* base = tile_base_counts + static_cast<size_t>(blockIdx.x) * (centroid_num + 1);
-    segment_indexes[static_cast<size_t>(p) * 3 + 1] = base[my_seg] + rank;
-    if (my_b != kInvalid) segment_indexes[static_cast<size_t>(p) * 3 + 2] = base[centroid_num] + brank;
+    const uint32_t* base = tile_base_counts + blockIdx.x;   // bin-major: bin b of this tile is base[b * tiles]
+    segment_indexes[static_cast<size_t>(p) * 3 + 1] = base[static_cast<size_t>(my_seg) * gridDim.x] + rank;
+    if (my_b != kInvalid) segment_indexes[static_cast<size_t>(p) * 3 + 2] = base[static_cast<size_t>(centroid_num) * gridDim.x] + brank;
 }
 
 // reorder_kernel (partition_kernel.cuh:68-100).  One wavefront moves kReorderRows consecutive points: their source
@@ -896,7 +897,7 @@ int assign_on_workspace(const float* data, uint32_t num, uint32_t dim, const flo
         }
     }
     // every tile has written all centroid_num + 1 bins of its histogram: nothing in the workspace has to start at zero
-    hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(kScanThreads), 0, s, tile_hist, tiles, centroid_num + 1, segment_lengths);
+    hipLaunchKernelGGL(tile_scan_kernel, dim3(centroid_num + 1), dim3(kScanThreads), 0, s, tile_hist, tiles, segment_lengths);
     hipLaunchKernelGGL(slot_kernel, dim3(tiles), dim3(kTilePoints), 0, s, segment_indexes, tile_hist, num, centroid_num);
     return launch_status();
 }
