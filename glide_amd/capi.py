@@ -359,6 +359,10 @@ def nnd_prepare(reorder_data, reorder_num, dim, segment_starts, segment_lengths,
                                       vp(stream)), "glide_hip_nnd_prepare")
 
 
+def nnd_sample(*args, stream=None):
+    _nnd_stage("glide_hip_nnd_sample", *args, stream)
+
+
 def nnd_reverse_sample(*args, stream=None):
     _nnd_stage("glide_hip_nnd_reverse_sample", *args, stream)
 

@@ -1372,6 +1372,15 @@ int glide_hip_nnd_prepare(const float* reorder_data, uint32_t reorder_num, uint3
     return rc != GLIDE_OK ? rc : nnd_prepare(c, reorder_data, dim, seed);
 }
 
+int glide_hip_nnd_sample(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
+                         uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
+    NndCtx c;
+    int rc = nnd_context(c, reorder_num, dim, segment_starts, segment_lengths, segment_num, knn_degree, workspace, workspace_bytes, stream);
+    if (rc != GLIDE_OK) return rc;
+    hipLaunchKernelGGL(nnd_sample_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.n, c.l.width, c.segs, c.fwd_new, c.fwd_old, c.counts);
+    return launch_status();
+}
+
 int glide_hip_nnd_reverse_sample(uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
                                  uint32_t segment_num, uint32_t knn_degree, void* workspace, size_t workspace_bytes, void* stream) {
     NndCtx c;

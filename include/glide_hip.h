@@ -171,6 +171,7 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *   merge           update_graph :1106-1126 + sample_graph_new :973-1001 + sample_segment_graph :1073-1104
  *   converge        the termination test of update_and_sample :1270-1284 (marks partitions that rest from now on)
  *   finalize        the shrink step :1376-1402
+ *   sample          sample_graph :1040-1071 on its own (prepare and merge include it)
  * glide_hip_nnd_build = prepare, `iterations` x (reverse_sample, local_join, merge, converge), finalize.
  * glide_hip_nnd_layout reports where each array lives in the workspace (byte offsets), so a caller or a test can
  * inspect or replace any of them between stages:
@@ -211,6 +212,13 @@ int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree
 int glide_hip_nnd_prepare(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
                           const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t seed,
                           void *workspace, size_t workspace_bytes, void *stream);
+/* sample_graph (nn_descent.cuh:1040-1071) on the lists as they stand: per list the first <= 32 entries not yet flagged
+ * become its new samples and are flagged, the first <= 32 flagged ones its old samples; the reverse counts restart.
+ * prepare has already done this for the start lists and merge does it for every later round, so the build loop never
+ * calls it; it is there for a caller that replaces the lists between stages. */
+int glide_hip_nnd_sample(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                         const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, void *workspace,
+                         size_t workspace_bytes, void *stream);
 int glide_hip_nnd_reverse_sample(uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
                                  const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree,
                                  void *workspace, size_t workspace_bytes, void *stream);

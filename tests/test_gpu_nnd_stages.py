@@ -423,6 +423,42 @@ def test_crowded_offer_table_announces_a_threshold(hip):
 
 
 @pytest.mark.parametrize("degree", [32, 64])
+def test_sample_stage_on_its_own(hip, degree):
+    """sample_graph (nn_descent.cuh:1040-1071) as a stage: on lists whose first 32 entries prepare has flagged, a second
+    call draws the next 32 unflagged entries in storage order as new samples (all of a 32-wide list is flagged by then:
+    none) and the first 32 flagged ones as old samples."""
+    num, dim = 1200, 128
+    rows = lowdim_data(num, dim, seed=17)
+    seg_start, seg_len = np.array([0, 700], np.uint32), np.array([700, 500], np.uint32)
+    d_rows = hip.DeviceArray.from_numpy(rows)
+    d_ss, d_sl = hip.DeviceArray.from_numpy(seg_start), hip.DeviceArray.from_numpy(seg_len)
+    ws = Workspace(hip, num, dim, degree)
+    args = (num, dim, d_ss, d_sl, 2, degree, ws.buf, ws.bytes)
+    hip.nnd_prepare(d_rows, num, dim, d_ss, d_sl, 2, degree, 4, ws.buf, ws.bytes)
+    hip.synchronize()
+    before = ws.read()
+    hip.nnd_sample(*args)
+    hip.synchronize()
+    after = ws.read()
+    width = ws.l.width
+    for node in range(num):
+        row = before["list_ids"][node]
+        unflagged = [int(v) for v in row if v != INV and not v & OLD][:S]
+        flagged = [int(v) & ~OLD for v in row if v != INV and v & OLD][:S]
+        assert after["counts"][node].tolist() == [len(unflagged), len(flagged), 0, 0]
+        assert after["fwd_new"][node, :len(unflagged)].tolist() == unflagged
+        assert after["fwd_old"][node, :len(flagged)].tolist() == flagged
+        want = row.copy()
+        taken = 0
+        for j in range(width):
+            if want[j] != INV and not want[j] & OLD and taken < S:
+                want[j] |= np.uint32(OLD)
+                taken += 1
+        np.testing.assert_array_equal(after["list_ids"][node], want)
+    assert (after["counts"][:, 0] == (0 if width == 32 else S)).all() and (after["counts"][:, 1] == S).all()
+
+
+@pytest.mark.parametrize("degree", [32, 64])
 def test_small_partitions_hold_no_id_twice(hip, degree):
     """Partitions with fewer points than list slots: the random start lists repeat ids (at distance FLT_MAX), and an offer
     for an id the list holds is rejected whatever distance the held copy carries (insert_to_ordered_list,
