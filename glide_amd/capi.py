@@ -337,7 +337,7 @@ def nnd_build(reorder_data, reorder_num, dim, segment_starts, segment_lengths, s
 class NndLayout(C.Structure):
     """glide_nnd_layout: byte offsets of the NN-descent arrays inside the workspace."""
     _fields_ = [(n, C.c_uint64) for n in ("half_rows", "norms", "list_ids", "list_dists", "fwd_new", "fwd_old", "rev_new", "rev_old",
-                                          "rev_tables", "rev_thr", "counts", "offers", "bloom", "segment_state", "segment_updates", "round", "total")] + \
+                                          "rev_tables", "rev_thr", "counts", "members", "member_counts", "offers", "bloom", "segment_state", "segment_updates", "round", "total")] + \
                [(n, C.c_uint32) for n in ("width", "reverse_cap", "reverse_stride", "offer_slots", "reverse_slots", "row_halfs", "bloom_sets", "reserved")]
 
 

@@ -286,7 +286,9 @@ struct JoinArgs {
     const uint32_t* rev_old;
     uint32_t* rev_tables;          // num x 2 x kRevSlots: where later arrivals went; emptied by the join that reads them
     uint32_t* rev_thr;             // num x 2: sources not below it stay away in the next scatter (all ones: none)
-    uint32_t* counts;              // num x 4: forward new / old, reverse new / old arrivals (restarted by the join)
+    uint32_t* counts;              // num x 4: forward new / old, reverse new / old arrivals (restarted by the members kernel)
+    uint32_t* members;             // num x 128: the lists a join works on, new members first (64 slots), then old ones
+    uint32_t* member_counts;       // num x 2: how many new and old members
     unsigned long long* offers;    // num x offer_slots: the offer tables
     uint32_t offer_slots, slot_shift;   // slot_shift = 32 - log2(offer_slots)
     const uint32_t* round;         // rounds completed so far (salt of the slot hash)
@@ -306,12 +308,14 @@ struct JoinLds {
     };
     __attribute__((aligned(16))) uint32_t new_ids[kBi], old_ids[kBi];   // read four at a time
     __attribute__((aligned(16))) float new_norms[kBi], old_norms[kBi];
-    uint32_t hash_new[128], hash_old[128];
-    __attribute__((aligned(16))) uint32_t rev_raw[2][kRevCap + kRevSlots];   // reverse samples as read: the list, then the overflow table
-    uint32_t rev_sel[2][kSamples];                                 // their 32 smallest entries, ascending
-    uint32_t rev_next_thr[2];
     uint32_t new_thr[kBi], old_thr[kBi];                           // offer thresholds of the members
-    uint32_t n_new, n_old;
+};
+
+struct MembersLds {   // per wavefront = per list; the two kinds of sample use it one after the other
+    __attribute__((aligned(16))) uint32_t rev_raw[4][kRevCap + kRevSlots];   // reverse samples as read: the list, then the overflow table
+    uint32_t rev_sel[4][kSamples];                                 // their 32 smallest entries, ascending
+    uint32_t rev_next_thr[4];
+    uint32_t hash[4][128];
 };
 
 __device__ __forceinline__ bool lds_set_insert(uint32_t* table, uint32_t key) {   // 128-slot open addressing
@@ -374,6 +378,101 @@ __device__ __forceinline__ void line_argmin(const float (*dist)[kDStride], uint3
     }
 }
 
+// ---- who takes part in a join: one wavefront per list, ahead of the join proper.
+// The members of a list are its forward samples and the 32 smallest sources of its reverse arrivals, duplicates
+// removed (reference: sort + binary search, :625-666; forward samples first, so a point that is in both keeps its
+// forward position).  This is light work on scattered reads: a kernel of its own runs it with eight wavefronts per
+// SIMD, where the join, held to six workgroups per CU by its tiles, spent a third of its time on it.
+__global__ __launch_bounds__(256) void nnd_members_kernel(JoinArgs a) {
+    __shared__ MembersLds L;
+    const int lane = lane_id(), wave = threadIdx.x >> 6;
+    const uint32_t node = blockIdx.x * 4 + wave;
+    if (node >= a.num) return;
+    // everything is asked for before anything is known about it (one memory round trip): both reverse lists, the
+    // forward samples (new ones in lanes 0..31, old ones in lanes 32..63), thresholds and counts
+    const uint32_t rev_in[2] = {a.rev_new[static_cast<size_t>(node) * kRevStride + lane], a.rev_old[static_cast<size_t>(node) * kRevStride + lane]};
+    const uint32_t forward_both = (lane < static_cast<int>(kSamples) ? a.fwd_new : a.fwd_old)[static_cast<size_t>(node) * kSamples + (lane & 31)];
+    const uint2 thr_both = *reinterpret_cast<const uint2*>(a.rev_thr + static_cast<size_t>(node) * 2);
+    const uint4 c4 = *reinterpret_cast<const uint4*>(a.counts + static_cast<size_t>(node) * 4);
+    uint32_t seg_start, seg_len, state;
+    locate_uniform(a.segs, node, seg_start, seg_len, &state);
+    if (state == kDone) return;
+    uint32_t* const raw = L.rev_raw[wave];
+    uint32_t* const sel = L.rev_sel[wave];
+    uint32_t* const set = L.hash[wave];
+#pragma unroll
+    for (int kind = 0; kind < 2; kind++) {   // 0: new, 1: old
+        const bool is_old = kind != 0;
+        uint32_t my_id = rev_in[kind];
+        const uint32_t thr_in_force = is_old ? thr_both.y : thr_both.x;
+        const uint32_t forward = static_cast<uint32_t>(__shfl(static_cast<int>(forward_both), (lane & 31) + 32 * kind));
+        __builtin_amdgcn_wave_barrier();   // the kind before is done with the scratch
+        set[lane] = kInvalid;
+        set[lane + 64] = kInvalid;
+
+        // Reverse samples: the 32 smallest sources that arrived, in ascending order.  Up to 64 arrivals sit in the list;
+        // a node that received more also has an overflow table, which is read and emptied (bounds included) here.
+        const uint32_t arrived = is_old ? c4.w : c4.z;
+        if (static_cast<uint32_t>(lane) >= arrived) my_id = kInvalid;
+        uint4 more = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
+        const bool overflowed = arrived > kRevCap;
+        if (overflowed) {
+            uint4* const quad = reinterpret_cast<uint4*>(a.rev_tables + (static_cast<size_t>(node) * 2 + kind) * kRevSlots) + lane;
+            more = *quad;
+            if ((more.x & more.y & more.z & more.w) != kInvalid) *quad = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
+            if ((lane & 3) == 3) more.w = kInvalid;   // word 15 of a bucket is its bound
+            *reinterpret_cast<uint4*>(&raw[kRevCap + 4 * lane]) = more;
+        }
+        raw[lane] = my_id;
+        if (lane < static_cast<int>(kSamples)) sel[lane] = kInvalid;
+        if (lane == 0) L.rev_next_thr[wave] = kInvalid;
+        __builtin_amdgcn_wave_barrier();
+        if (!overflowed) {
+            uint32_t rank = 0;
+            // four slots a step, as far as the arrivals go (the slots behind them hold 0xffffffff and count for nothing)
+            for (uint32_t j = 0; j < arrived; j += 4) {
+                const uint4 q = *reinterpret_cast<const uint4*>(&raw[j]);
+                rank += (q.x < my_id) + (q.y < my_id) + (q.z < my_id) + (q.w < my_id);
+            }
+            if (my_id != kInvalid && rank < kSamples) sel[rank] = my_id;
+        } else {
+            const uint32_t mine[5] = {my_id, more.x, more.y, more.z, more.w};
+            uint32_t rank[5] = {0, 0, 0, 0, 0};
+            for (uint32_t j = 0; j < kRevCap + kRevSlots; j += 4) {
+                const uint4 q = *reinterpret_cast<const uint4*>(&raw[j]);
+#pragma unroll
+                for (int m = 0; m < 5; m++) rank[m] += (q.x < mine[m]) + (q.y < mine[m]) + (q.z < mine[m]) + (q.w < mine[m]);
+            }
+#pragma unroll
+            for (int m = 0; m < 5; m++) {
+                if (mine[m] != kInvalid && rank[m] < kSamples) sel[rank[m]] = mine[m];
+                // after an overflow the 56th smallest source becomes the threshold of the scatter that follows: some 55
+                // sources are then expected, few enough to stay in the list, enough for the smallest 32 to be complete
+                if (mine[m] != kInvalid && rank[m] == kRevThrRank - 1) L.rev_next_thr[wave] = mine[m];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (lane == 0) {
+            // a threshold that is in force stays while at least 40 sources still arrive
+            const uint32_t next = overflowed ? L.rev_next_thr[wave] : (arrived >= kRevKeepArrivals ? thr_in_force : kInvalid);
+            if (next != thr_in_force) a.rev_thr[static_cast<size_t>(node) * 2 + kind] = next;
+            // this list's reverse samples are consumed here and now: the count restarts for the scatter that follows the join
+            a.counts[static_cast<size_t>(node) * 4 + 2 + kind] = 0u;
+        }
+        // Forward samples (lanes 0..31) enter the set first, then the reverse ones (lanes 32..63).
+        const uint32_t k = lane;
+        const uint32_t id = k < kSamples ? (k < (is_old ? c4.y : c4.x) ? forward : kInvalid) : sel[k - kSamples];
+        const bool usable = id != kInvalid && id < seg_len;
+        bool keep = false;
+        if (k < kSamples) keep = usable && lds_set_insert(set, id);
+        __builtin_amdgcn_wave_barrier();
+        if (k >= kSamples) keep = usable && lds_set_insert(set, id);
+        const uint64_t m = ballot(keep);
+        if (keep) a.members[static_cast<size_t>(node) * (2 * kBi) + kBi * kind + prefix_count(m)] = id;
+        if (lane == 0) a.member_counts[static_cast<size_t>(node) * 2 + kind] = __popcll(m);
+    }
+}
+
 // Six workgroups per CU (20 KB of LDS each): the join is bound by the latency of its gather -> matrix -> arg-min ->
 // offer chain, so residency matters more than registers; seven would spill.
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a) {
@@ -382,102 +481,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     const uint32_t node = blockIdx.x;
     if (node >= a.num) return;
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
-    const bool sampler = tid < 128;                  // wave 0 gathers the new members, wave 1 the old ones
-    const bool is_old = (wave & 1) != 0;             // waves 2 and 3 read the reverse tables (new, old)
-    const uint32_t k = tid & 63;                     // sampler: 0..31 forward sample, 32..63 reverse sample
-
-    // sample ids are fetched before the counts are known (one memory round trip instead of two)
-    uint32_t my_id = kInvalid, thr_in_force = kInvalid;
-    if (!sampler) {
-        my_id = (is_old ? a.rev_old : a.rev_new)[static_cast<size_t>(node) * kRevStride + lane];
-        thr_in_force = a.rev_thr[static_cast<size_t>(node) * 2 + is_old];
-    } else if (lane < static_cast<int>(kSamples))
-        my_id = (is_old ? a.fwd_old : a.fwd_new)[static_cast<size_t>(node) * kSamples + lane];
-    if (sampler) {
-        L.hash_new[tid] = kInvalid;
-        L.hash_old[tid] = kInvalid;
-        (is_old ? L.old_norms : L.new_norms)[k] = __builtin_inff();   // replaced below for the rows the lists hold
-    }
-    const uint4 c4 = *reinterpret_cast<const uint4*>(a.counts + static_cast<size_t>(node) * 4);
+    // member ids are fetched before their counts are known (one memory round trip instead of two); slots beyond a
+    // list hold what an earlier round left there, and count for nothing: their norm below is infinite
+    const uint32_t member = tid < static_cast<int>(2 * kBi) ? a.members[static_cast<size_t>(node) * (2 * kBi) + tid] : kInvalid;
+    const uint2 mc = *reinterpret_cast<const uint2*>(a.member_counts + static_cast<size_t>(node) * 2);
     uint32_t seg_start, seg_len;
     uint32_t state;
     locate_uniform(a.segs, node, seg_start, seg_len, &state);
     if (state == kDone) return;
-    // The counts must have arrived in every thread before thread 0 restarts them below; the barrier itself waits
-    // for LDS traffic only, so the registers are consumed here.
-    asm volatile("" ::"v"(c4.x), "v"(c4.y), "v"(c4.z), "v"(c4.w), "v"(my_id), "v"(thr_in_force));
-    if (!sampler) {
-        // Reverse samples: the 32 smallest sources that arrived, in ascending order.  Up to 64 arrivals sit in the list;
-        // a node that received more also has an overflow table, which is read and emptied (bounds included) here.
-        const uint32_t arrived = is_old ? c4.w : c4.z;
-        if (static_cast<uint32_t>(lane) >= arrived) my_id = kInvalid;
-        uint4 more = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
-        const bool overflowed = arrived > kRevCap;
-        if (overflowed) {
-            uint4* const quad = reinterpret_cast<uint4*>(a.rev_tables + (static_cast<size_t>(node) * 2 + is_old) * kRevSlots) + lane;
-            more = *quad;
-            if ((more.x & more.y & more.z & more.w) != kInvalid) *quad = make_uint4(kInvalid, kInvalid, kInvalid, kInvalid);
-            if ((lane & 3) == 3) more.w = kInvalid;   // word 15 of a bucket is its bound
-            *reinterpret_cast<uint4*>(&L.rev_raw[is_old][kRevCap + 4 * lane]) = more;
-        }
-        L.rev_raw[is_old][lane] = my_id;
-        if (lane < static_cast<int>(kSamples)) L.rev_sel[is_old][lane] = kInvalid;
-        if (lane == 0) L.rev_next_thr[is_old] = kInvalid;
-        __builtin_amdgcn_wave_barrier();
-        if (!overflowed) {
-            uint32_t rank = 0;
-            // all 64 slots in four steps of four independent reads (slots beyond the arrivals hold 0xffffffff and count for nothing)
-#pragma unroll
-            for (uint32_t j = 0; j < kRevCap; j += 4) {
-                const uint4 q = *reinterpret_cast<const uint4*>(&L.rev_raw[is_old][j]);
-                rank += (q.x < my_id) + (q.y < my_id) + (q.z < my_id) + (q.w < my_id);
-            }
-            if (my_id != kInvalid && rank < kSamples) L.rev_sel[is_old][rank] = my_id;
-        } else {
-            const uint32_t mine[5] = {my_id, more.x, more.y, more.z, more.w};
-            uint32_t rank[5] = {0, 0, 0, 0, 0};
-            for (uint32_t j = 0; j < kRevCap + kRevSlots; j += 4) {
-                const uint4 q = *reinterpret_cast<const uint4*>(&L.rev_raw[is_old][j]);
-#pragma unroll
-                for (int m = 0; m < 5; m++) rank[m] += (q.x < mine[m]) + (q.y < mine[m]) + (q.z < mine[m]) + (q.w < mine[m]);
-            }
-#pragma unroll
-            for (int m = 0; m < 5; m++) {
-                if (mine[m] != kInvalid && rank[m] < kSamples) L.rev_sel[is_old][rank[m]] = mine[m];
-                // after an overflow the 56th smallest source becomes the threshold of the scatter that follows: some 55
-                // sources are then expected, few enough to stay in the list, enough for the smallest 32 to be complete
-                if (mine[m] != kInvalid && rank[m] == kRevThrRank - 1) L.rev_next_thr[is_old] = mine[m];
-            }
-        }
-        // a threshold that is in force stays while at least 40 sources still arrive
-        __builtin_amdgcn_wave_barrier();
-        if (lane == 0) {
-            const uint32_t next = overflowed ? L.rev_next_thr[is_old] : (arrived >= kRevKeepArrivals ? thr_in_force : kInvalid);
-            if (next != thr_in_force) a.rev_thr[static_cast<size_t>(node) * 2 + is_old] = next;
-        }
-    }
-    __syncthreads();   // the hash sets are clear, the reverse samples chosen, the counts read by everyone
-    // this list's reverse samples are consumed here and now: the counts restart for the scatter that follows the join
-    if (tid == 0) *reinterpret_cast<uint2*>(a.counts + static_cast<size_t>(node) * 4 + 2) = make_uint2(0u, 0u);
-    // Forward then reverse samples, duplicates removed with an LDS hash set (reference: sort + binary search, :625-666).
-    // Forward samples enter the set first, so a point that is in both keeps its forward position.
-    if (sampler) {
-        uint32_t* set = is_old ? L.hash_old : L.hash_new;
-        if (k >= kSamples) my_id = L.rev_sel[is_old][k - kSamples];
-        const bool present = k < kSamples ? k < (is_old ? c4.y : c4.x) : true;
-        const uint32_t id = present ? my_id : kInvalid;
-        const bool usable = id != kInvalid && id < seg_len;
-        bool keep = false;
-        if (k < kSamples) keep = usable && lds_set_insert(set, id);
-        __builtin_amdgcn_wave_barrier();
-        if (k >= kSamples) keep = usable && lds_set_insert(set, id);
-        const uint64_t m = ballot(keep);
-        if (keep) (is_old ? L.old_ids : L.new_ids)[prefix_count(m)] = id;
-        if (lane == 0) (is_old ? L.n_old : L.n_new) = __popcll(m);
+    const uint32_t n_new = mc.x, n_old = mc.y;
+    if (n_new == 0) return;
+    if (tid < static_cast<int>(2 * kBi)) {
+        (tid < static_cast<int>(kBi) ? L.new_ids : L.old_ids)[tid & 63] = member;
+        (tid < static_cast<int>(kBi) ? L.new_norms : L.old_norms)[tid & 63] = __builtin_inff();   // replaced below for the rows the lists hold
     }
     __syncthreads();
-    const uint32_t n_new = L.n_new, n_old = L.n_old;
-    if (n_new == 0) return;
 
     const int rb = wave >> 1, cb = wave & 1;
     float16v acc_nn, acc_no;
@@ -1158,8 +1176,8 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 constexpr uint32_t kMaxWidth = 192;   // six sub-lists: degrees up to 128 (width + 32 offers fit one 256-key network)
 
 struct NndLayout {
-    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts, offers, bloom, stats, seg_state,
-        seg_updates, round, total;
+    size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts, members, member_counts, offers, bloom, stats,
+        seg_state, seg_updates, round, total;
     uint32_t width, dim_pad, bloom_sets;
 };
 NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
@@ -1182,6 +1200,8 @@ NndLayout nnd_layout(uint32_t num, uint32_t dim, uint32_t degree) {
     l.rev_tables = take(n * 2 * kRevSlots * 4);
     l.rev_thr = take(n * 8);
     l.counts = take(n * 16);
+    l.members = take(n * 2 * kBi * 4);
+    l.member_counts = take(n * 8);
     l.offers = take(n * offer_slots_for(l.width) * 8);
     l.bloom = take(n * l.bloom_sets * 64);
     l.stats = take(1024 * 16);
@@ -1206,7 +1226,7 @@ struct NndCtx {
     float2* norms;
     uint32_t* list_ids;
     float* list_dists;
-    uint32_t *fwd_new, *fwd_old, *rev_new, *rev_old, *rev_tables, *rev_thr, *counts, *round;
+    uint32_t *fwd_new, *fwd_old, *rev_new, *rev_old, *rev_tables, *rev_thr, *counts, *members, *member_counts, *round;
     unsigned long long* offers;
     uint32_t* bloom;
     unsigned long long* stats;
@@ -1241,6 +1261,8 @@ int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* s
     c.rev_tables = reinterpret_cast<uint32_t*>(w + c.l.rev_tables);
     c.rev_thr = reinterpret_cast<uint32_t*>(w + c.l.rev_thr);
     c.counts = reinterpret_cast<uint32_t*>(w + c.l.counts);
+    c.members = reinterpret_cast<uint32_t*>(w + c.l.members);
+    c.member_counts = reinterpret_cast<uint32_t*>(w + c.l.member_counts);
     c.offers = reinterpret_cast<unsigned long long*>(w + c.l.offers);
     c.bloom = reinterpret_cast<uint32_t*>(w + c.l.bloom);
     c.stats = reinterpret_cast<unsigned long long*>(w + c.l.stats);
@@ -1280,8 +1302,9 @@ int nnd_reverse(const NndCtx& c) {
 int nnd_join(const NndCtx& c, bool with_stats) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
-    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.offers, offer_slots_for(c.l.width),
+    JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.members, c.member_counts, c.offers, offer_slots_for(c.l.width),
                 offer_slots_for(c.l.width) == 512 ? 23u : 24u, c.round, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
+    hipLaunchKernelGGL(nnd_members_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ja);
     hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja);
     return launch_status();
 }
@@ -1357,7 +1380,7 @@ int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree
     const NndLayout l = nnd_layout(reorder_num, dim, knn_degree);
     out->half_rows = l.half_rows; out->norms = l.norms; out->list_ids = l.list_ids; out->list_dists = l.list_dists;
     out->fwd_new = l.fwd_new; out->fwd_old = l.fwd_old; out->rev_new = l.rev_new; out->rev_old = l.rev_old; out->rev_tables = l.rev_tables; out->rev_thr = l.rev_thr;
-    out->counts = l.counts; out->offers = l.offers; out->bloom = l.bloom;
+    out->counts = l.counts; out->members = l.members; out->member_counts = l.member_counts; out->offers = l.offers; out->bloom = l.bloom;
     out->segment_state = l.seg_state; out->segment_updates = l.seg_updates; out->round = l.round; out->total = l.total;
     out->width = l.width; out->reverse_cap = kRevCap; out->reverse_stride = kRevStride; out->offer_slots = offer_slots_for(l.width); out->reverse_slots = kRevSlots; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
     return GLIDE_OK;

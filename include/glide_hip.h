@@ -182,6 +182,9 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *   fwd_new / fwd_old  num x 32 u32 sample lists, rev_new / rev_old  num rows of reverse_stride (72) u32 holding up to
  *                   reverse_cap (64) reverse samples in order of arrival; counts num x 4 u32 = their lengths (the reverse lengths count every arrival and may exceed
  *                   reverse_cap; the join uses the 32 smallest)
+ *   members    num x 128 u32 and member_counts num x 2 u32: the lists a join works on, written by local_join before its
+ *                   tiles: slots 0..63 the new members (forward samples, then the 32 smallest reverse sources, duplicates
+ *                   removed), slots 64..127 the old ones; slots beyond the counts keep what an earlier round left there
  *   offers     num x offer_slots u64 keys (distance bits << 32 | candidate id, all ones = empty): the offers of the
  *                   round.  offer_slots is 256 when the list is one sub-list (knn_degree <= 32) and 512 otherwise.  With
  *                   x = candidate ^ round * 0x85EBCA6B, an offer goes to slot s1 = (x * 0x9E3779B1) >> (32 - log2
@@ -205,7 +208,7 @@ int glide_hip_nnd_build(const float *reorder_data, uint32_t reorder_num, uint32_
  *   segment_state   u32 per partition: 0 active, 1 last round, 2 resting;  segment_updates  u32 per partition */
 typedef struct {
     uint64_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts,
-        offers, bloom, segment_state, segment_updates, round, total;
+        members, member_counts, offers, bloom, segment_state, segment_updates, round, total;
     uint32_t width, reverse_cap, reverse_stride, offer_slots, reverse_slots, row_halfs, bloom_sets, reserved;
 } glide_nnd_layout;
 int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree, glide_nnd_layout *out);
