@@ -309,6 +309,8 @@ struct JoinLds {
     __attribute__((aligned(16))) uint32_t new_ids[kBi], old_ids[kBi];   // read four at a time
     __attribute__((aligned(16))) float new_norms[kBi], old_norms[kBi];
     uint32_t new_thr[kBi], old_thr[kBi];                           // offer thresholds of the members
+    float part_d[2][2 * kBi];      // column arg-mins of the two row blocks: [new x new | new x old][row block * 64 + column]
+    uint32_t part_i[2][2 * kBi];
 };
 
 struct MembersLds {   // per wavefront = per list; the two kinds of sample use it one after the other
@@ -551,28 +553,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
 
     const int t = lane & 31, kh = lane >> 5;
     const uint32_t line = tid >> 2, part = tid & 3;
-    // ---- phase 1: new x new
-    __syncthreads();   // every wave is done with the rows: the tile may overwrite them
-    // Rows and columns beyond the lists carry an infinite norm (and zero rows), so their entries come out infinite
-    // without a test; the diagonal lies in the two wavefronts whose row and column blocks coincide.
-    {
-        const uint32_t j = cb * 32 + t;
-        const float nj = L.new_norms[j];
-        const bool diagonal_block = rb == cb;
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const uint32_t i0 = rb * 32 + 8 * q + 4 * kh;
-            const float4 ni = *reinterpret_cast<const float4*>(&L.new_norms[i0]);
-            const float n4[4] = {ni.x, ni.y, ni.z, ni.w};
-#pragma unroll
-            for (int m = 0; m < 4; m++) {
-                float d = fmaxf((n4[m] + nj) - 2.f * acc_nn[4 * q + m], 0.f);
-                if (diagonal_block && i0 + m == j) d = FLT_MAX;
-                L.dist[i0 + m][j] = d;
-            }
-        }
-    }
-    __syncthreads();
     // An offer is two atomic minima on slots of one line of the target's table; nothing comes back, so the wave does not wait.
     const uint32_t salt = round_salt(*a.round);
     uint32_t declined = 0;
@@ -588,18 +568,57 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         __hip_atomic_fetch_min(&row[s1], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_fetch_min(&row[s2], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
+    // Nearest partner of a column, in registers.  A lane holds 16 rows of one column of its quadrant, in ascending row
+    // order; its partner lane (the other half of the wavefront) the 16 rows in between; the other row block belongs to
+    // another wavefront and is met through LDS.  Smaller distance first, then the smaller row: what a scan of the
+    // column from the top finds.
+    auto column_partial = [&](float best, uint32_t bi, float* part_d, uint32_t* part_i) {
+        const float od = lane_xor<32>(best);
+        const uint32_t oi = lane_xor<32>(bi);
+        if (od < best || (od == best && oi < bi)) {
+            best = od;
+            bi = oi;
+        }
+        if (kh == 0) {
+            part_d[rb * kBi + cb * 32 + t] = best;
+            part_i[rb * kBi + cb * 32 + t] = bi;
+        }
+    };
+    // ---- new x new.  The matrix is symmetric: the nearest new partner of member j is the arg-min of column j.
+    // Rows and columns beyond the lists carry an infinite norm (and zero rows), so their entries come out infinite
+    // without a test; the diagonal lies in the two wavefronts whose row and column blocks coincide.
     {
-        float best;
-        uint32_t bj;
-        line_argmin<true>(L.dist, line, part, best, bj);
-        if (part == 0 && line < n_new && bj != kInvalid) send(L.new_ids[line], L.new_ids[bj], best, L.new_thr[line]);
+        const uint32_t j = cb * 32 + t;
+        const float nj = L.new_norms[j];
+        const bool diagonal_block = rb == cb;
+        float best = FLT_MAX;
+        uint32_t bi = kInvalid;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t i0 = rb * 32 + 8 * q + 4 * kh;
+            const float4 ni = *reinterpret_cast<const float4*>(&L.new_norms[i0]);
+            const float n4[4] = {ni.x, ni.y, ni.z, ni.w};
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                float d = fmaxf((n4[m] + nj) - 2.f * acc_nn[4 * q + m], 0.f);
+                if (diagonal_block && i0 + m == j) d = FLT_MAX;
+                if (d < best) {
+                    best = d;
+                    bi = i0 + m;
+                }
+            }
+        }
+        column_partial(best, bi, L.part_d[0], L.part_i[0]);
     }
     if (n_old != 0) {
-        // ---- phase 2: new x old (rows: new, columns: old)
-        __syncthreads();
+        // ---- new x old (rows: new, columns: old).  Columns as above (an old member's nearest new one); the rows (a new
+        // member's nearest old one) run across the lanes and go through the distance tile in LDS.
+        __syncthreads();   // every wave is done with the rows: the tile may overwrite them
         const uint32_t j = cb * 32 + t;
         const uint32_t col_id = j < n_old ? L.old_ids[j] : kInvalid;
         const float nj = L.old_norms[j];
+        float best = FLT_MAX;
+        uint32_t bi = kInvalid;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const uint32_t i0 = rb * 32 + 8 * q + 4 * kh;
@@ -612,23 +631,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
                 float d = fmaxf((n4[m] + nj) - 2.f * acc_no[4 * q + m], 0.f);
                 if (id4[m] == col_id) d = FLT_MAX;   // the same point sits in both lists: it is no partner of itself
                 L.dist[i0 + m][j] = d;
+                if (d < best) {
+                    best = d;
+                    bi = i0 + m;
+                }
             }
         }
-        __syncthreads();
-        {
-            float best;
-            uint32_t bj;
-            const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
-            line_argmin<true>(L.dist, line, part, best, bj);
-            if (part == 0 && line < n_new && bj != kInvalid) send(me, L.old_ids[bj], best, L.new_thr[line]);
+        column_partial(best, bi, L.part_d[1], L.part_i[1]);
+    }
+    __syncthreads();
+    // ---- the offers.  Threads 0..63 own the new x new columns, threads 64..127 the new x old columns: the two row
+    // blocks of a column are combined (the upper block wins ties, its rows come first).
+    if (tid < static_cast<int>(2 * kBi) && (tid < static_cast<int>(kBi) || n_old != 0)) {
+        const int which = tid >> 6;
+        const uint32_t j = tid & 63;
+        float best = L.part_d[which][j];
+        uint32_t bi = L.part_i[which][j];
+        const float od = L.part_d[which][kBi + j];
+        if (od < best) {
+            best = od;
+            bi = L.part_i[which][kBi + j];
         }
-        {
-            float best;
-            uint32_t bi;
-            const uint32_t me = line < n_old ? L.old_ids[line] : kInvalid;
-            line_argmin<false>(L.dist, line, part, best, bi);
-            if (part == 0 && line < n_old && bi != kInvalid) send(me, L.new_ids[bi], best, L.old_thr[line]);
-        }
+        if (j < (which ? n_old : n_new) && bi != kInvalid)
+            send((which ? L.old_ids : L.new_ids)[j], L.new_ids[bi], best, (which ? L.old_thr : L.new_thr)[j]);
+    }
+    if (n_old != 0) {
+        float best;
+        uint32_t bj;
+        const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
+        line_argmin<true>(L.dist, line, part, best, bj);
+        if (part == 0 && line < n_new && bj != kInvalid) send(me, L.old_ids[bj], best, L.new_thr[line]);
     }
     if (declined && a.stats) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(declined));
 }
