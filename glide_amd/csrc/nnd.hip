@@ -477,7 +477,7 @@ __global__ __launch_bounds__(256) void nnd_members_kernel(JoinArgs a) {
 
 // Six workgroups per CU (20 KB of LDS each): the join is bound by the latency of its gather -> matrix -> arg-min ->
 // offer chain, so residency matters more than registers; seven would spill.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a, bool wide_only) {
     extern __shared__ __align__(16) unsigned char smem[];
     JoinLds& L = *reinterpret_cast<JoinLds*>(smem);
     const uint32_t node = blockIdx.x;
@@ -492,7 +492,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     locate_uniform(a.segs, node, seg_start, seg_len, &state);
     if (state == kDone) return;
     const uint32_t n_new = mc.x, n_old = mc.y;
-    if (n_new == 0) return;
+    if (n_new == 0 || (wide_only && n_new <= kSamples)) return;   // narrow lists: nnd_join_narrow_kernel
     if (tid < static_cast<int>(2 * kBi)) {
         (tid < static_cast<int>(kBi) ? L.new_ids : L.old_ids)[tid & 63] = member;
         (tid < static_cast<int>(kBi) ? L.new_norms : L.old_norms)[tid & 63] = __builtin_inff();   // replaced below for the rows the lists hold
@@ -663,6 +663,212 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         if (part == 0 && line < n_new && bj != kInvalid) send(me, L.old_ids[bj], best, L.new_thr[line]);
     }
     if (declined && a.stats) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(declined));
+}
+
+// ---- local join of a list with at most 32 new members (rows of up to 128 dims): one wavefront, no barrier ---------
+// From the fourth round on nearly every list has fewer than 32 new members: the 64 x 64 tiles of the kernel above are
+// then three quarters padding, and its four wavefronts hold registers and LDS for work one can do.  Here a wavefront
+// joins one list by itself:
+//  * rows go from memory straight into LDS (global_load_lds, 16 bytes a lane, 16 lanes a row: whole rows in one
+//    round trip, no staging registers); the 16-byte pieces of row r are stored at slot piece ^ (r % 16), so the
+//    matrix-core operand reads (lane t: row t) fall on distinct banks with rows 256 bytes apart;
+//  * the operands of a block of 32 rows are then read into registers once and serve every tile the block takes part
+//    in: new x new, new x old, and old x new.  The last is the transpose of the second; computing it as well (eight
+//    more matrix instructions a tile) turns "a new member's nearest old one" into a column minimum like the other
+//    two, taken over the 16 accumulator registers of a lane and one exchange between the halves of the wavefront, so
+//    no distance ever leaves the registers;
+//  * the second block of old members is fetched into the buffer of the new ones while the first tiles are computed.
+constexpr uint32_t kNarrowJoinMaxDim = 128;
+typedef const __attribute__((address_space(1))) void* global_ptr;
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// Running column minimum over one 32 x 32 tile: rows row_base .. + 31 (their norms and ids in LDS), the lane's column
+// with norm nj and id col_id.  A point is no partner of itself: the diagonal of new x new, and a point that sits in
+// both lists.  Rows and columns beyond the lists carry an infinite norm (and zero rows) and never win.
+__device__ __forceinline__ void tile_column_min(const float16v& acc, const float* row_norms, const uint32_t* row_ids, uint32_t row_base, float nj,
+                                                uint32_t col_id, int kh, float& best, uint32_t& bi) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const uint32_t i0 = row_base + 8 * q + 4 * kh;
+        const float4 ni = *reinterpret_cast<const float4*>(&row_norms[i0]);
+        const uint4 idi = *reinterpret_cast<const uint4*>(&row_ids[i0]);
+        const float n4[4] = {ni.x, ni.y, ni.z, ni.w};
+        const uint32_t id4[4] = {idi.x, idi.y, idi.z, idi.w};
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            float d = fmaxf((n4[m] + nj) - 2.f * acc[4 * q + m], 0.f);
+            if (id4[m] == col_id) d = FLT_MAX;
+            if (d < best) {
+                best = d;
+                bi = i0 + m;
+            }
+        }
+    }
+}
+
+constexpr int kWaitVm0 = 0x0F70, kWaitLgkm0 = 0xC07F;   // s_waitcnt vmcnt(0) / lgkmcnt(0), the other counters left alone
+
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void nnd_join_narrow_kernel(JoinArgs a) {
+    // separate arrays, so that the compiler can tell reads of the small ones from the row buffers that fetches write
+    __shared__ __attribute__((aligned(16))) _Float16 rows[32][kNarrowJoinMaxDim];   // one block of 32 members at a time
+    __shared__ __attribute__((aligned(16))) uint32_t lds_new_ids[kSamples], lds_old_ids[kBi];
+    __shared__ __attribute__((aligned(16))) float lds_new_norms[kSamples], lds_old_norms[kBi];
+    const uint32_t node = blockIdx.x;
+    const int lane = lane_id(), t = lane & 31, kh = lane >> 5;
+    // ids before counts (one round trip); slots beyond a list hold what an earlier round left there
+    const uint32_t got_new = a.members[static_cast<size_t>(node) * (2 * kBi) + t];
+    const uint32_t got_old = a.members[static_cast<size_t>(node) * (2 * kBi) + kBi + lane];
+    const uint2 mc = *reinterpret_cast<const uint2*>(a.member_counts + static_cast<size_t>(node) * 2);
+    uint32_t seg_start, seg_len, state;
+    locate_uniform(a.segs, node, seg_start, seg_len, &state);
+    if (state == kDone) return;
+    const uint32_t n_new = mc.x, n_old = mc.y;
+    if (n_new == 0 || n_new > kSamples) return;   // wider lists belong to nnd_join_kernel
+    const uint32_t new_id = static_cast<uint32_t>(t) < n_new ? got_new : kInvalid, old_id = static_cast<uint32_t>(lane) < n_old ? got_old : kInvalid;
+    lds_new_ids[t] = new_id;
+    lds_old_ids[lane] = old_id;
+    __builtin_amdgcn_wave_barrier();
+
+    // Sixteen lanes fetch one row; eight instructions fill a block of 32.  A lane whose row or piece does not exist
+    // stores zeros in its place -- all such stores of a block before its first fetch, because an ordinary LDS store
+    // waits for the fetches issued before it.
+    const uint32_t my_row = lane >> 4, slot = lane & 15;
+    auto row_ids = [&](uint32_t (&ids)[8], const uint32_t* from) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) ids[i] = from[4 * i + my_row];
+    };
+    auto clear = [&](_Float16 (*buf)[kNarrowJoinMaxDim], const uint32_t (&ids)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t r = 4 * i + my_row, piece = slot ^ (r & 15);
+            if (ids[i] == kInvalid || piece * 8 >= a.dim_pad) *reinterpret_cast<float4*>(&buf[r][slot * 8]) = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto fetch = [&](_Float16 (*buf)[kNarrowJoinMaxDim], const uint32_t (&ids)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t r = 4 * i + my_row, piece = slot ^ (r & 15);
+            if (ids[i] != kInvalid && piece * 8 < a.dim_pad)
+                __builtin_amdgcn_global_load_lds((global_ptr)(a.half_rows + static_cast<size_t>(seg_start + ids[i]) * a.dim_pad + piece * 8), (lds_ptr)(&buf[4 * i][0]), 16, 0, 0);
+        }
+    };
+    auto operands = [&](half8v (&X)[8], const _Float16 (*buf)[kNarrowJoinMaxDim]) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) X[s] = *reinterpret_cast<const half8v*>(&buf[t][((2 * s + kh) ^ (t & 15)) * 8]);
+    };
+    const bool second_block = n_old > 32;
+    uint32_t ids[8];
+    row_ids(ids, lds_new_ids);
+    clear(rows, ids);
+    fetch(rows, ids);
+    // norm and offer threshold of the lane's own members, in the same round trip
+    float2 nw = make_float2(__builtin_inff(), __uint_as_float(kInvalid)), od = nw;
+    if (new_id != kInvalid) nw = a.norms[seg_start + new_id];
+    if (old_id != kInvalid) od = a.norms[seg_start + old_id];
+    half8v A[8], B[8];
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+    __builtin_amdgcn_wave_barrier();
+    lds_new_norms[t] = nw.x;
+    lds_old_norms[lane] = od.x;
+    operands(A, rows);
+    // The buffer is free once its rows are in registers: the next block sets out while tiles are computed.
+    auto next_block = [&](const uint32_t* from) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+        __builtin_amdgcn_wave_barrier();
+        row_ids(ids, from);
+        clear(rows, ids);
+        fetch(rows, ids);
+    };
+    auto arrived = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(kWaitVm0);
+        __builtin_amdgcn_wave_barrier();
+        operands(B, rows);
+    };
+    if (n_old) next_block(lds_old_ids);
+    const float x_od = lane_xor<32>(od.x);
+    const uint32_t x_old = lane_xor<32>(old_id);
+    const float b_norm[2] = {kh ? x_od : od.x, kh ? od.x : x_od};   // column t of old block 0 / 1, for both halves
+    const uint32_t b_id[2] = {kh ? x_old : old_id, kh ? old_id : x_old};
+
+    const uint32_t steps = (a.dim_pad + 15) / 16;
+    auto tile = [&](const half8v (&X)[8], const half8v (&Y)[8]) __attribute__((always_inline)) {
+        float16v acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+            if (static_cast<uint32_t>(s) < steps) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(X[s], Y[s], acc, 0, 0, 0);
+        return acc;
+    };
+    // the two halves of a wavefront hold alternate groups of four rows of a column: smaller distance, then smaller row
+    auto settle = [&](float& best, uint32_t& bi) __attribute__((always_inline)) {
+        const float other_d = lane_xor<32>(best);
+        const uint32_t other_i = lane_xor<32>(bi);
+        if (other_d < best || (other_d == best && other_i < bi)) {
+            best = other_d;
+            bi = other_i;
+        }
+    };
+    float nn_d = FLT_MAX, on_d = FLT_MAX, no_d[2] = {FLT_MAX, FLT_MAX};
+    uint32_t nn_i = kInvalid, on_i = kInvalid, no_i[2] = {kInvalid, kInvalid};
+    {   // new x new: the nearest new partner of new member t
+        const float16v acc = tile(A, A);
+        tile_column_min(acc, lds_new_norms, lds_new_ids, 0, nw.x, new_id, kh, nn_d, nn_i);
+        settle(nn_d, nn_i);
+    }
+    if (n_old) {
+        arrived();
+        if (second_block) next_block(lds_old_ids + 32);
+        {   // new x old: the nearest new partner of old member t
+            const float16v acc = tile(A, B);
+            tile_column_min(acc, lds_new_norms, lds_new_ids, 0, b_norm[0], b_id[0], kh, no_d[0], no_i[0]);
+            settle(no_d[0], no_i[0]);
+        }
+        {   // old x new: the nearest old partner of new member t, first block of rows
+            const float16v acc = tile(B, A);
+            tile_column_min(acc, lds_old_norms, lds_old_ids, 0, nw.x, new_id, kh, on_d, on_i);
+        }
+        if (second_block) {
+            arrived();
+            {
+                const float16v acc = tile(A, B);
+                tile_column_min(acc, lds_new_norms, lds_new_ids, 0, b_norm[1], b_id[1], kh, no_d[1], no_i[1]);
+                settle(no_d[1], no_i[1]);
+            }
+            {
+                const float16v acc = tile(B, A);
+                tile_column_min(acc, lds_old_norms, lds_old_ids, 32, nw.x, new_id, kh, on_d, on_i);
+            }
+        }
+        settle(on_d, on_i);
+    }
+
+    // ---- the offers: two atomic minima on slots of one line of the target's table; nothing comes back
+    const uint32_t salt = round_salt(*a.round);
+    uint32_t declined = 0;
+    auto send = [&](uint32_t target, uint32_t cand, float dist, uint32_t thr) {
+        bool stays_away = false;
+        if (target != kInvalid && cand != kInvalid && cand != target && cand < seg_len && dist < FLT_MAX) {
+            if (__float_as_uint(dist) >= thr) {
+                stays_away = true;   // the target has asked offers from this distance on to stay away
+            } else {
+                const unsigned long long key = (static_cast<unsigned long long>(__float_as_uint(dist)) << 32) | cand;
+                unsigned long long* row = a.offers + (static_cast<size_t>(seg_start) + target) * a.offer_slots;
+                const uint32_t s1 = offer_slot(cand, salt, a.slot_shift), s2 = offer_slot_beside(s1, cand, salt);
+                __hip_atomic_fetch_min(&row[s1], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_min(&row[s2], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (a.stats) declined += static_cast<uint32_t>(__popcll(ballot(stays_away)));
+    };
+    // lower half: the nearest new partner of new member t; upper half: its nearest old partner
+    const uint32_t from_new = lds_new_ids[nn_i & 31u], from_old = lds_old_ids[on_i & 63u];
+    const uint32_t partner = kh ? (on_i == kInvalid ? kInvalid : from_old) : (nn_i == kInvalid ? kInvalid : from_new);
+    send(new_id, partner, kh ? on_d : nn_d, __float_as_uint(nw.y));
+    // old member `lane`: its nearest new partner
+    const uint32_t pick_old = kh ? no_i[1] : no_i[0];
+    send(old_id, pick_old == kInvalid ? kInvalid : lds_new_ids[pick_old & 31u], kh ? no_d[1] : no_d[0], __float_as_uint(od.y));
+    if (declined && lane == 0) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(declined));
 }
 
 // ---- merge ------------------------------------------------------------------------------------------------------
@@ -1337,7 +1543,11 @@ int nnd_join(const NndCtx& c, bool with_stats) {
     JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.members, c.member_counts, c.offers, offer_slots_for(c.l.width),
                 offer_slots_for(c.l.width) == 512 ? 23u : 24u, c.round, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
     hipLaunchKernelGGL(nnd_members_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ja);
-    hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja);
+    // lists with at most 32 new members go to the one-wavefront kernel, the others to the workgroup kernel; each passes
+    // over the other's lists
+    const bool narrow = c.l.dim_pad <= kNarrowJoinMaxDim;
+    hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja, narrow);
+    if (narrow) hipLaunchKernelGGL(nnd_join_narrow_kernel, dim3(c.n), dim3(64), 0, c.s, ja);
     return launch_status();
 }
 
