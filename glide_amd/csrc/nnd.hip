@@ -477,12 +477,17 @@ __global__ __launch_bounds__(256) void nnd_members_kernel(JoinArgs a) {
 
 // Six workgroups per CU (20 KB of LDS each): the join is bound by the latency of its gather -> matrix -> arg-min ->
 // offer chain, so residency matters more than registers; seven would spill.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a, bool wide_only) {
+// `lists`: which lists are this kernel's.  kAllLists: every one.  kWideLists: those with more than 32 new members, the
+// others being nnd_join_narrow_kernel's; kWideListsFew: the same when they are expected to be few -- the counts are
+// then read first, and a workgroup that passes over its list has asked for 8 bytes instead of the whole member list.
+constexpr int kAllLists = 0, kWideLists = 1, kWideListsFew = 2;
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a, int lists) {
     extern __shared__ __align__(16) unsigned char smem[];
     JoinLds& L = *reinterpret_cast<JoinLds*>(smem);
     const uint32_t node = blockIdx.x;
     if (node >= a.num) return;
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    if (lists == kWideListsFew && a.member_counts[static_cast<size_t>(node) * 2] <= kSamples) return;
     // member ids are fetched before their counts are known (one memory round trip instead of two); slots beyond a
     // list hold what an earlier round left there, and count for nothing: their norm below is infinite
     const uint32_t member = tid < static_cast<int>(2 * kBi) ? a.members[static_cast<size_t>(node) * (2 * kBi) + tid] : kInvalid;
@@ -492,7 +497,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     locate_uniform(a.segs, node, seg_start, seg_len, &state);
     if (state == kDone) return;
     const uint32_t n_new = mc.x, n_old = mc.y;
-    if (n_new == 0 || (wide_only && n_new <= kSamples)) return;   // narrow lists: nnd_join_narrow_kernel
+    if (n_new == 0 || (lists != kAllLists && n_new <= kSamples)) return;
     if (tid < static_cast<int>(2 * kBi)) {
         (tid < static_cast<int>(kBi) ? L.new_ids : L.old_ids)[tid & 63] = member;
         (tid < static_cast<int>(kBi) ? L.new_norms : L.old_norms)[tid & 63] = __builtin_inff();   // replaced below for the rows the lists hold
@@ -1537,7 +1542,8 @@ int nnd_reverse(const NndCtx& c) {
     return launch_status();
 }
 
-int nnd_join(const NndCtx& c, bool with_stats) {
+// few_wide: most lists are expected to have at most 32 new members (the rule once the first rounds are over)
+int nnd_join(const NndCtx& c, bool with_stats, bool few_wide = false) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
     JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.members, c.member_counts, c.offers, offer_slots_for(c.l.width),
@@ -1546,7 +1552,7 @@ int nnd_join(const NndCtx& c, bool with_stats) {
     // lists with at most 32 new members go to the one-wavefront kernel, the others to the workgroup kernel; each passes
     // over the other's lists
     const bool narrow = c.l.dim_pad <= kNarrowJoinMaxDim;
-    hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja, narrow);
+    hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja, !narrow ? kAllLists : few_wide ? kWideListsFew : kWideLists);
     if (narrow) hipLaunchKernelGGL(nnd_join_narrow_kernel, dim3(c.n), dim3(64), 0, c.s, ja);
     return launch_status();
 }
@@ -1598,7 +1604,7 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
     if ((rc = nnd_prepare(c, reorder_data, dim, seed)) != GLIDE_OK) return rc;
     for (uint32_t it = 0; it < iterations; it++) {
         if (it == 0 && (rc = nnd_reverse(c)) != GLIDE_OK) return rc;   // later rounds: the merge of the round before has done it
-        if ((rc = nnd_join(c, stats_out != nullptr)) != GLIDE_OK) return rc;
+        if ((rc = nnd_join(c, stats_out != nullptr, it >= 3)) != GLIDE_OK) return rc;
         if ((rc = nnd_merge(c, stats_out != nullptr, it + 1 < iterations)) != GLIDE_OK) return rc;
         if ((rc = nnd_converge(c, dim, termination_threshold)) != GLIDE_OK) return rc;
         // GNND::build leaves its loop when the update count falls below the limit (nn_descent.cuh:1270-1284).  Here the
