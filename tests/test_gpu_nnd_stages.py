@@ -489,3 +489,72 @@ def test_small_partitions_hold_no_id_twice(hip, degree):
     hip.nnd_finalize(num, dim, d_ss, d_sl, 4, degree, d_knn, None, ws.buf, ws.bytes)
     hip.synchronize()
     assert (d_knn.numpy() < limit[:, None]).all()
+
+
+def fast_model_join(st, rows, seg_start, seg_len):
+    """model_join with the arg-mins taken by numpy (first minimum = earlier position); also returns how many lists had
+    (at most 32 new members, of those more than 32 old ones, more than 32 new members)."""
+    offers, shapes = {}, [0, 0, 0]
+    half = rows.astype(np.float16).astype(np.float32)
+    norms = (rows.astype(np.float32) ** 2).sum(1, dtype=np.float32)
+    for node in range(seg_start, seg_start + seg_len):
+        c = st["counts"][node]
+        new = _dedupe(st["fwd_new"][node, :c[0]], reverse_samples(st, node, 0), seg_len)
+        old = _dedupe(st["fwd_old"][node, :c[1]], reverse_samples(st, node, 1), seg_len)
+        if not new:
+            continue
+        shapes[0 if len(new) <= S else 2] += 1
+        shapes[1] += len(new) <= S and len(old) > S
+        new_a, old_a = np.array(new), np.array(old, dtype=np.int64)
+        xn, nn_ = half[seg_start + new_a], norms[seg_start + new_a]
+        d = np.maximum(nn_[:, None] + nn_[None, :] - 2.0 * (xn @ xn.T), 0.0).astype(np.float32)
+        np.fill_diagonal(d, np.inf)
+        if len(new) > 1:
+            for i, j in enumerate(d.argmin(1)):
+                offers.setdefault(new[i], []).append((float(d[i, j]), new[j]))
+        if old:
+            xo, no_ = half[seg_start + old_a], norms[seg_start + old_a]
+            d = np.maximum(nn_[:, None] + no_[None, :] - 2.0 * (xn @ xo.T), 0.0).astype(np.float32)
+            d[new_a[:, None] == old_a[None, :]] = np.inf        # a point in both lists is no partner of itself
+            for i, j in enumerate(d.argmin(1)):
+                if np.isfinite(d[i, j]):
+                    offers.setdefault(new[i], []).append((float(d[i, j]), old[j]))
+            for j, i in enumerate(d.argmin(0)):
+                if np.isfinite(d[i, j]):
+                    offers.setdefault(old[j], []).append((float(d[i, j]), new[i]))
+    kept = {k: sorted(o for o in v if offer_key(*o) >> 32 < int(st["offer_thr"][seg_start + k])) for k, v in offers.items()}
+    return kept, shapes
+
+
+@pytest.mark.parametrize("dim", [40, 96, 128, 136])
+def test_both_join_kernels_match_model(hip, dim):
+    """Six rounds, so that lists with few new members (one wavefront each, rows of up to 128 dims) and lists with many (one
+    workgroup each) both occur, with one and with two blocks of old members; row lengths that are no multiple of 16
+    (the last matrix step half empty), below 128 and above it.  Every node's offer table must be the model's."""
+    num, degree = 1800, 32
+    rows = lowdim_data(num, dim, seed=11)
+    seg_start, seg_len = np.array([0, 1500, 1780], np.uint32), np.array([1500, 280, 20], np.uint32)
+    d_rows = hip.DeviceArray.from_numpy(rows)
+    d_ss, d_sl = hip.DeviceArray.from_numpy(seg_start), hip.DeviceArray.from_numpy(seg_len)
+    ws = Workspace(hip, num, dim, degree)
+    args = (num, dim, d_ss, d_sl, 3, degree, ws.buf, ws.bytes)
+    hip.nnd_prepare(d_rows, num, dim, d_ss, d_sl, 3, degree, 7, ws.buf, ws.bytes)
+    seen = np.zeros(3, np.int64)
+    for it in range(6):
+        print("dim", dim, "round", it, flush=True)
+        hip.nnd_reverse_sample(*args)
+        hip.synchronize()
+        st = ws.read()
+        hip.nnd_local_join(*args)
+        hip.synchronize()
+        after = ws.read()
+        for s0, l0 in zip(seg_start.tolist(), seg_len.tolist()):
+            offers, shapes = fast_model_join(st, rows, s0, l0)
+            seen += shapes
+            for t in range(l0):
+                exp = model_offer_table([offer_key(d, c) for d, c in offers.get(t, [])], it, ws.l.offer_slots)
+                np.testing.assert_array_equal(after["offers"][s0 + t], exp, err_msg="round %d, offer table of node %d" % (it, s0 + t))
+        hip.nnd_merge(*args)
+        hip.nnd_converge(num, dim, d_ss, d_sl, 3, degree, 0.0, ws.buf, ws.bytes)
+    print("lists with at most 32 new members %d (%d of them with more than 32 old ones), with more %d" % tuple(seen), flush=True)
+    assert seen.min() > 0
