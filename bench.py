@@ -31,6 +31,10 @@ SWEEP_BEAMS = (32, 64, 128, 256, 512)       # the reference accepts beams up to 
 NAMED_BEAMS = {"cfg1": (32, 64, 128, 256)}  # the medium configuration names its beams; 512 is swept there as an extra
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "search_kernels_hbm_traffic.md")
 VALU_PROFILE = os.path.join(ROOT, "profiles", "build_refine_kernels_counters.md")
+NND_OFFERS_NOTE = ("nnd_offers: distinct offers the merge steps found in the offer tables, all rounds.  nnd_offers_declined_by_threshold: offers a "
+                   "join did not send because their distance was not below the threshold their target announced (the distance of its 64th "
+                   "best offer of the round before, announced only by nodes whose table was five eighths full).  Nothing depends on the order "
+                   "of arrival: two builds with one seed give the same graph (tests/test_gpu_nnd.py::test_nnd_same_seed_same_graph).")
 
 
 def measured_traffic(workload, beam):
@@ -286,7 +290,8 @@ def run_workload(args, workload, torch, want_cpu):
         workload=desc, gen_sec=gen_s, build_sec=build_sec, stage_rooflines=stage_rooflines,
         build_stages=dict(pre=res["pre_time"], knn=res["knn_time"], index=res["index_time"], refine=res["refine_time"],
                           detail={**res["pre_stages"], **res["build_stages"]}),
-        nnd_iterations=nnd_iters, nnd_offers=res["nnd_stats"][0], nnd_offers_dropped=res["nnd_stats"][1],
+        nnd_iterations=nnd_iters, nnd_offers=res["nnd_stats"][0], nnd_offers_declined_by_threshold=res["nnd_stats"][1],
+        nnd_offers_note=NND_OFFERS_NOTE,
         graph_recall_at_32=graph_recall_partition, graph_recall_at_32_global=graph_recall_global,
         partition_sizes=[int(x) for x in h_len], empty_slots_fraction=holes,
         sweep=sweep, beam=chosen["beam"], recall_at_10=chosen["recall_at_10"], recall_target_met=bool(ok),
@@ -451,7 +456,7 @@ def main():
         "qps_at_max_beam": None if met else main_res["qps"],
     }
     for k in ("build_sec", "build_stages", "graph_recall_at_32", "graph_recall_at_32_global", "recall_at_10", "recall_target_met",
-              "empty_slots_fraction", "sweep", "kernel_ms", "nnd_offers", "nnd_offers_dropped", "stage_rooflines", "roofline"):
+              "empty_slots_fraction", "sweep", "kernel_ms", "nnd_offers", "nnd_offers_declined_by_threshold", "nnd_offers_note", "stage_rooflines", "roofline"):
         line[k] = main_res[k]
     if "cpu_baseline" in main_res:
         line["cpu_baseline"] = main_res["cpu_baseline"]

@@ -59,7 +59,7 @@ def test_nnd_structure_and_recall(hip):
     r_gpu = partition_recall(knn, data, seg_start, seg_len, k)
     cpu = O.nnd_build(data, seg_start, seg_len, k, 10).astype(np.uint32)
     r_cpu = partition_recall(cpu, data, seg_start, seg_len, k)
-    print("graph recall@32 after 10 iterations: gpu %.4f cpu-restatement %.4f; offers %d dropped %d" % (r_gpu, r_cpu, stats[0], stats[1]))
+    print("graph recall@32 after 10 iterations: gpu %.4f cpu-restatement %.4f; offers %d, declined by their target's threshold %d" % (r_gpu, r_cpu, stats[0], stats[1]))
     assert r_gpu >= 0.95
     assert r_gpu >= r_cpu - 0.005      # within half a point of the reference algorithm at equal degree / iterations
 
