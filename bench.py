@@ -85,6 +85,8 @@ def parse():
                     help="only run the plain copy kernel on 1 GiB x steps (yardstick for rocprofv3 byte counters) and exit")
     ap.add_argument("--valu-calibration", action="store_true",
                     help="only run the register-only multiply-add kernel (yardstick for the vector-ALU issue rate) and exit")
+    ap.add_argument("--atomic-calibration", action="store_true",
+                    help="only run the scattered-atomics kernel (yardstick for the NN-descent offers and slot reservations) and exit")
     ap.add_argument("--partition-only", type=int, default=0, metavar="C",
                     help="only time partition assignment of 1M x 128 rows against C centroids (fp32 matrix-core tile) and exit")
     return ap.parse_args()
@@ -391,6 +393,27 @@ def main():
             insts = 2048 * 4 * rounds * 16 * per_step
             res[name] = {"wave_instructions": insts, "ms": ms, "G_wave_instructions_per_s": insts / ms / 1e6}
         print(json.dumps({"kernel": "valu_probe_kernel", "compute_units": info["compute_units"], "modes": res}))
+        return
+
+    if args.atomic_calibration:
+        import numpy as np
+        out = capi.DeviceArray(4, np.uint32)
+        rounds, res = 256, {}
+        ops = 2048 * 256 * rounds
+        for name, slots in (("2 MB of slots (stays in L2)", 1 << 18), ("2 GB of slots (an offer table of 1M nodes)", 1 << 28)):
+            for mode, kind in enumerate(("64-bit minimum, no result", "32-bit add, result used", "64-bit minimum, pairs of adjacent lanes on one 128-byte line",
+                                         "64-bit minimum, 16 adjacent lanes on one 128-byte line")):
+                table = capi.DeviceArray.full(2 * slots, 0xFFFFFFFF if mode == 0 else 0, np.uint32)
+                capi.atomic_probe(mode, table, slots, rounds, out)
+                e0, e1 = capi.Event(), capi.Event()
+                e0.record()
+                for _ in range(args.steps):
+                    capi.atomic_probe(mode, table, slots, rounds, out)
+                e1.record()
+                ms = e0.elapsed_ms(e1) / args.steps
+                res["%s; %s" % (kind, name)] = {"lane_operations": ops, "ms": ms, "G_lane_operations_per_s": ops / ms / 1e6}
+                del table
+        print(json.dumps({"kernel": "atomic_probe_kernel", "compute_units": info["compute_units"], "modes": res}))
         return
 
     if args.partition_only:

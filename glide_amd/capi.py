@@ -397,6 +397,10 @@ def valu_probe(mode, rounds, out, stream=None):
     check(lib().glide_hip_valu_probe(C.c_int(mode), u32(rounds), _ptr(out), vp(stream)), "glide_hip_valu_probe")
 
 
+def atomic_probe(mode, table, slots, rounds, out, stream=None):
+    check(lib().glide_hip_atomic_probe(C.c_int(mode), _ptr(table), u32(slots), u32(rounds), _ptr(out), vp(stream)), "glide_hip_atomic_probe")
+
+
 def copy_bytes(dst, src, nbytes, stream=None):
     check(lib().glide_hip_copy_bytes(_ptr(dst), _ptr(src), C.c_size_t(nbytes), vp(stream)), "glide_hip_copy_bytes")
 

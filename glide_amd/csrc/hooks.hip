@@ -46,6 +46,33 @@ __global__ __launch_bounds__(256) void valu_probe_kernel(uint32_t rounds, float 
     if (sum == 12345.678f) out[0] = sum;   // keeps the loop alive; practically never taken
 }
 
+// The rate of atomic operations on scattered words: every thread issues `rounds` of them on slots of `table` drawn by
+// a hash of (thread, round).  MODE 0: 64-bit minimum, nothing returned (what an NN-descent offer is made of); 1: 32-bit
+// add whose result is used (what reserves a slot of a reverse list); 2 and 3: as 0, with 2 / 16 adjacent lanes on slots of
+// one 128-byte line.
+template <int MODE>
+__global__ __launch_bounds__(256) void atomic_probe_kernel(unsigned long long* table, uint32_t slot_mask, uint32_t rounds, uint32_t* out) {
+    const uint32_t tid = blockIdx.x * 256 + threadIdx.x;
+    uint32_t x = tid * 0x9E3779B1u + 0x7F4A7C15u, sum = 0;
+    for (uint32_t r = 0; r < rounds; r++) {
+        x ^= x << 13;
+        x ^= x >> 17;
+        x ^= x << 5;
+        uint32_t slot = (x * 0x85EBCA6Bu >> 7) & slot_mask;
+        if constexpr (MODE >= 2) {   // groups of 2 (MODE 2) or 16 (MODE 3) adjacent lanes share a 128-byte line
+            constexpr uint32_t G = MODE == 2 ? 2 : 16;
+            const uint32_t leader = static_cast<uint32_t>(__shfl(static_cast<int>(slot), static_cast<int>(threadIdx.x & 63u & ~(G - 1))));
+            slot = ((leader & ~15u) | ((leader + (threadIdx.x & (G - 1))) & 15u)) & slot_mask;
+        }
+        if constexpr (MODE != 1) {
+            __hip_atomic_fetch_min(&table[slot], (static_cast<unsigned long long>(x) << 32) | tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            sum += atomicAdd(reinterpret_cast<uint32_t*>(table) + 2 * slot, 1u);
+        }
+    }
+    if (sum == 0xFFFFFFF1u) out[0] = sum;   // keeps the results alive; practically never taken
+}
+
 __global__ __launch_bounds__(64) void distance_batch_kernel(const float* a, const float* b, uint32_t n, uint32_t dim,
                                                             int metric, float* out) {
     const int lane = lane_id();
@@ -184,6 +211,17 @@ int glide_hip_valu_probe(int mode, uint32_t rounds, float* out, void* stream) {
         case 1: hipLaunchKernelGGL(valu_probe_kernel<1>, dim3(2048), dim3(256), 0, as_stream(stream), rounds, 1.0f, out); break;
         case 2: hipLaunchKernelGGL(valu_probe_kernel<2>, dim3(2048), dim3(256), 0, as_stream(stream), rounds, 1.0f, out); break;
         default: hipLaunchKernelGGL(valu_probe_kernel<3>, dim3(2048), dim3(256), 0, as_stream(stream), rounds, 1.0f, out); break;
+    }
+    return launch_status();
+}
+
+int glide_hip_atomic_probe(int mode, unsigned long long* table, uint32_t slots, uint32_t rounds, uint32_t* out, void* stream) {
+    if (!table || !out || mode < 0 || mode > 3 || slots < 16 || (slots & (slots - 1)) != 0) return GLIDE_ERR_BAD_ARGUMENT;
+    switch (mode) {
+        case 0: hipLaunchKernelGGL(atomic_probe_kernel<0>, dim3(2048), dim3(256), 0, as_stream(stream), table, slots - 1, rounds, out); break;
+        case 1: hipLaunchKernelGGL(atomic_probe_kernel<1>, dim3(2048), dim3(256), 0, as_stream(stream), table, slots - 1, rounds, out); break;
+        case 2: hipLaunchKernelGGL(atomic_probe_kernel<2>, dim3(2048), dim3(256), 0, as_stream(stream), table, slots - 1, rounds, out); break;
+        default: hipLaunchKernelGGL(atomic_probe_kernel<3>, dim3(2048), dim3(256), 0, as_stream(stream), table, slots - 1, rounds, out); break;
     }
     return launch_status();
 }
