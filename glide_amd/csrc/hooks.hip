@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void atomic_probe_kernel(unsigned long long* t
         x ^= x << 13;
         x ^= x >> 17;
         x ^= x << 5;
-        uint32_t slot = (x * 0x85EBCA6Bu >> 7) & slot_mask;
+        uint32_t slot = (x * 0x85EBCA6Bu >> 4) & slot_mask;
         if constexpr (MODE >= 2) {   // groups of 2 (MODE 2) or 16 (MODE 3) adjacent lanes share a 128-byte line
             constexpr uint32_t G = MODE == 2 ? 2 : 16;
             const uint32_t leader = static_cast<uint32_t>(__shfl(static_cast<int>(slot), static_cast<int>(threadIdx.x & 63u & ~(G - 1))));
