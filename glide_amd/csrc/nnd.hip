@@ -563,16 +563,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     // operations a second, and nearly twice as many when adjacent lanes aim at one 128-byte line.
     const uint32_t salt = round_salt(*a.round);
     uint32_t declined = 0;
-    auto send = [&](uint32_t target, uint32_t cand, float dist, uint32_t thr, bool second_slot) {
-        if (cand == kInvalid || cand == target || cand >= seg_len || !(dist < FLT_MAX)) return;
+    // A slot is read before anything is sent to it (the reads of a thread's two offers are under way while the row scan
+    // runs): within a round a slot only ever gets smaller, so a minimum that would not get below what the read has found
+    // changes nothing and is left out.  In the first rounds, where the wide lists are, that is every second one.
+    struct Offer {
+        unsigned long long* where;
+        unsigned long long what, there;
+    };
+    auto address = [&](uint32_t target, uint32_t cand, float dist, uint32_t thr, bool second_slot) {
+        Offer o{nullptr, 0, 0};
+        if (cand == kInvalid || cand == target || cand >= seg_len || !(dist < FLT_MAX)) return o;
         if (__float_as_uint(dist) >= thr) {   // the target has asked offers from this distance on to stay away
             declined += !second_slot;
-            return;
+            return o;
         }
-        const unsigned long long key = (static_cast<unsigned long long>(__float_as_uint(dist)) << 32) | cand;
         unsigned long long* row = a.offers + (static_cast<size_t>(seg_start) + target) * a.offer_slots;
         const uint32_t s1 = offer_slot(cand, salt, a.slot_shift);
-        __hip_atomic_fetch_min(&row[second_slot ? offer_slot_beside(s1, cand, salt) : s1], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        o.where = &row[second_slot ? offer_slot_beside(s1, cand, salt) : s1];
+        o.what = (static_cast<unsigned long long>(__float_as_uint(dist)) << 32) | cand;
+        o.there = __hip_atomic_load(o.where, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return o;
+    };
+    auto send = [&](const Offer& o) {
+        if (o.where && o.what < o.there) __hip_atomic_fetch_min(o.where, o.what, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
     // Nearest partner of a column, in registers.  A lane holds 16 rows of one column of its quadrant, in ascending row
     // order; its partner lane (the other half of the wavefront) the 16 rows in between; the other row block belongs to
@@ -648,6 +661,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     __syncthreads();
     // ---- the offers.  Threads 2 j and 2 j + 1 own new x new column j (j < 64) or new x old column j - 64: the two row
     // blocks of a column are combined (the upper block wins ties, its rows come first), then each takes a slot.
+    Offer of_column{nullptr, 0, 0}, of_row{nullptr, 0, 0};
     {
         const int which = tid >> 7;
         const uint32_t j = (tid >> 1) & 63;
@@ -660,7 +674,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
                 bi = L.part_i[which][kBi + j];
             }
             if (j < (which ? n_old : n_new) && bi != kInvalid)
-                send((which ? L.old_ids : L.new_ids)[j], L.new_ids[bi], best, (which ? L.old_thr : L.new_thr)[j], tid & 1);
+                of_column = address((which ? L.old_ids : L.new_ids)[j], L.new_ids[bi], best, (which ? L.old_thr : L.new_thr)[j], tid & 1);
         }
     }
     if (n_old != 0) {
@@ -669,8 +683,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
         uint32_t bj;
         const uint32_t me = line < n_new ? L.new_ids[line] : kInvalid;
         line_argmin<true>(L.dist, line, part, best, bj);
-        if (part < 2 && line < n_new && bj != kInvalid) send(me, L.old_ids[bj], best, L.new_thr[line], part);
+        if (part < 2 && line < n_new && bj != kInvalid) of_row = address(me, L.old_ids[bj], best, L.new_thr[line], part);
     }
+    send(of_column);
+    send(of_row);
     if (declined && a.stats) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(declined));
 }
 
@@ -717,7 +733,7 @@ __device__ __forceinline__ void tile_column_min(const float16v& acc, const float
 
 constexpr int kWaitVm0 = 0x0F70, kWaitLgkm0 = 0xC07F;   // s_waitcnt vmcnt(0) / lgkmcnt(0), the other counters left alone
 
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void nnd_join_narrow_kernel(JoinArgs a) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void nnd_join_narrow_kernel(JoinArgs a, bool read_first) {
     // separate arrays, so that the compiler can tell reads of the small ones from the row buffers that fetches write
     __shared__ __attribute__((aligned(16))) _Float16 rows[32][kNarrowJoinMaxDim];   // one block of 32 members at a time
     __shared__ __attribute__((aligned(16))) uint32_t lds_new_ids[kSamples], lds_old_ids[kBi];
@@ -853,38 +869,51 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
     }
 
     // ---- the offers: two atomic minima on slots of one line of the target's table; nothing comes back.  Every lane
-    // has at most one offer.  The chip carries out some 27 G scattered atomic operations a second, and nearly twice as
-    // many when adjacent lanes aim at one 128-byte line: so the two slots of an offer are taken by two adjacent lanes
-    // in one instruction -- first the offers of the lower 32 lanes, then those of the upper 32.
+    // has at most one offer of each kind.  The chip carries out some 27 G scattered atomic operations a second, and
+    // nearly twice as many when adjacent lanes aim at one 128-byte line: so the two slots of an offer are taken by two
+    // adjacent lanes in one instruction -- first the offers of the lower 32 lanes, then those of the upper 32.  And a
+    // in the first rounds (read_first) a slot is read before anything is sent to it: within a round a slot only ever gets
+    // smaller, so a minimum that would not get below what the read has found changes nothing and is left out.  In
+    // those rounds half of them are -- copies of an offer another list has delivered, offers that lose their slot to a
+    // nearer one -- and reads are an order of magnitude cheaper than atomics; later few are, and the read only adds a
+    // round trip.
     const uint32_t salt = round_salt(*a.round);
     uint32_t declined = 0;
-    auto send = [&](uint32_t target, uint32_t cand, float dist, uint32_t thr) __attribute__((always_inline)) {
+    unsigned long long* where[4];
+    unsigned long long what[4], there[4];
+    auto address = [&](int first, uint32_t target, uint32_t cand, float dist, uint32_t thr) __attribute__((always_inline)) {
         const bool wanted = target != kInvalid && cand != kInvalid && cand != target && cand < seg_len && dist < FLT_MAX;
         const bool stays_away = wanted && __float_as_uint(dist) >= thr;   // the target has asked offers from this distance on to stay away
         const uint64_t go = ballot(wanted && !stays_away);
         if (a.stats) declined += static_cast<uint32_t>(__popcll(ballot(stays_away)));
 #pragma unroll
         for (int h = 0; h < 2; h++) {
+            where[first + h] = nullptr;
+            what[first + h] = 0;
+            there[first + h] = 0;
             if (static_cast<uint32_t>(go >> (32 * h)) == 0u) continue;
             const int from = 32 * h + (lane >> 1);
             const uint32_t t_ = static_cast<uint32_t>(__shfl(static_cast<int>(target), from)), c_ = static_cast<uint32_t>(__shfl(static_cast<int>(cand), from));
             const uint32_t d_ = static_cast<uint32_t>(__shfl(static_cast<int>(__float_as_uint(dist)), from));
             if ((go >> from) & 1ull) {
-                const unsigned long long key = (static_cast<unsigned long long>(d_) << 32) | c_;
                 unsigned long long* row = a.offers + (static_cast<size_t>(seg_start) + t_) * a.offer_slots;
                 const uint32_t s1 = offer_slot(c_, salt, a.slot_shift);
-                const uint32_t slot = (lane & 1) ? offer_slot_beside(s1, c_, salt) : s1;
-                __hip_atomic_fetch_min(&row[slot], key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                where[first + h] = &row[(lane & 1) ? offer_slot_beside(s1, c_, salt) : s1];
+                what[first + h] = (static_cast<unsigned long long>(d_) << 32) | c_;
+                there[first + h] = read_first ? __hip_atomic_load(where[first + h], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : kNoOffer;
             }
         }
     };
     // lower half: the nearest new partner of new member t; upper half: its nearest old partner
     const uint32_t from_new = lds_new_ids[nn_i & 31u], from_old = lds_old_ids[on_i & 63u];
     const uint32_t partner = kh ? (on_i == kInvalid ? kInvalid : from_old) : (nn_i == kInvalid ? kInvalid : from_new);
-    send(new_id, partner, kh ? on_d : nn_d, __float_as_uint(nw.y));
+    address(0, new_id, partner, kh ? on_d : nn_d, __float_as_uint(nw.y));
     // old member `lane`: its nearest new partner
     const uint32_t pick_old = kh ? no_i[1] : no_i[0];
-    send(old_id, pick_old == kInvalid ? kInvalid : lds_new_ids[pick_old & 31u], kh ? no_d[1] : no_d[0], __float_as_uint(od.y));
+    address(2, old_id, pick_old == kInvalid ? kInvalid : lds_new_ids[pick_old & 31u], kh ? no_d[1] : no_d[0], __float_as_uint(od.y));
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (where[i] && what[i] < there[i]) __hip_atomic_fetch_min(where[i], what[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (declined && lane == 0) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(declined));
 }
 
@@ -1555,7 +1584,8 @@ int nnd_reverse(const NndCtx& c) {
 }
 
 // few_wide: most lists are expected to have at most 32 new members (the rule once the first rounds are over)
-int nnd_join(const NndCtx& c, bool with_stats, bool few_wide = false) {
+// early: one of the first rounds, in which many offers are copies of one another
+int nnd_join(const NndCtx& c, bool with_stats, bool few_wide = false, bool early = true) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
     JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.members, c.member_counts, c.offers, offer_slots_for(c.l.width),
@@ -1565,7 +1595,7 @@ int nnd_join(const NndCtx& c, bool with_stats, bool few_wide = false) {
     // over the other's lists
     const bool narrow = c.l.dim_pad <= kNarrowJoinMaxDim;
     hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja, !narrow ? kAllLists : few_wide ? kWideListsFew : kWideLists);
-    if (narrow) hipLaunchKernelGGL(nnd_join_narrow_kernel, dim3(c.n), dim3(64), 0, c.s, ja);
+    if (narrow) hipLaunchKernelGGL(nnd_join_narrow_kernel, dim3(c.n), dim3(64), 0, c.s, ja, early);
     return launch_status();
 }
 
@@ -1616,7 +1646,7 @@ int glide_hip_nnd_build(const float* reorder_data, uint32_t reorder_num, uint32_
     if ((rc = nnd_prepare(c, reorder_data, dim, seed)) != GLIDE_OK) return rc;
     for (uint32_t it = 0; it < iterations; it++) {
         if (it == 0 && (rc = nnd_reverse(c)) != GLIDE_OK) return rc;   // later rounds: the merge of the round before has done it
-        if ((rc = nnd_join(c, stats_out != nullptr, it >= 3)) != GLIDE_OK) return rc;
+        if ((rc = nnd_join(c, stats_out != nullptr, it >= 3, it < 4)) != GLIDE_OK) return rc;
         if ((rc = nnd_merge(c, stats_out != nullptr, it + 1 < iterations)) != GLIDE_OK) return rc;
         if ((rc = nnd_converge(c, dim, termination_threshold)) != GLIDE_OK) return rc;
         // GNND::build leaves its loop when the update count falls below the limit (nn_descent.cuh:1270-1284).  Here the
