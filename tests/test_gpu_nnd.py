@@ -190,3 +190,32 @@ def test_nnd_same_seed_same_graph(hip):
         assert np.array_equal(a, b) and st_a[0] == st_b[0]
         assert not np.array_equal(a, c)
         print("degree %d: offers merged %d, dropped by full buckets %d" % (k, st_a[0], st_a[1]))
+
+
+@pytest.mark.parametrize("k,dim", [(32, 128), (64, 96), (32, 200)])
+def test_nnd_build_equals_its_stages(hip, k, dim):
+    """glide_hip_nnd_build takes shortcuts its stage entry points do not: the merge kernel scatters the next round's
+    reverse samples itself, from the fourth round on the workgroup join looks at a list's counts before its members,
+    and from the fifth the joins no longer read a slot before sending to it.  None of this may show: eight rounds run
+    stage by stage must end in the very graph the fused build gives (dims with and without the one-wavefront join)."""
+    from glide_amd import datasets as D
+    data = D.gmm_clipped(12000, dim, seed=21)
+    seg_start, seg_len = np.array([0, 7000], np.uint32), np.array([7000, 5000], np.uint32)
+    rounds, seed = 8, 5
+    fused, _ = gpu_nnd(hip, data, seg_start, seg_len, k, rounds, seed=seed)
+    n = data.shape[0]
+    d_data = hip.DeviceArray.from_numpy(data, np.float32)
+    d_ss, d_sl = hip.DeviceArray.from_numpy(seg_start, np.uint32), hip.DeviceArray.from_numpy(seg_len, np.uint32)
+    wb = hip.nnd_workspace_bytes(n, dim, k)
+    ws = hip.DeviceArray(wb // 16 + 1, np.dtype("V16"))
+    args = (n, dim, d_ss, d_sl, 2, k, ws, wb)
+    hip.nnd_prepare(d_data, n, dim, d_ss, d_sl, 2, k, seed, ws, wb)
+    for _ in range(rounds):
+        hip.nnd_reverse_sample(*args)
+        hip.nnd_local_join(*args)
+        hip.nnd_merge(*args)
+        hip.nnd_converge(n, dim, d_ss, d_sl, 2, k, 0.0, ws, wb)
+    knn = hip.DeviceArray((n, k), np.uint32)
+    hip.nnd_finalize(n, dim, d_ss, d_sl, 2, k, knn, None, ws, wb)
+    hip.synchronize()
+    assert np.array_equal(knn.numpy(), fused)
