@@ -31,6 +31,7 @@ SWEEP_BEAMS = (32, 64, 128, 256, 512)       # the reference accepts beams up to 
 NAMED_BEAMS = {"cfg1": (32, 64, 128, 256)}  # the medium configuration names its beams; 512 is swept there as an extra
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "search_kernels_hbm_traffic.md")
 VALU_PROFILE = os.path.join(ROOT, "profiles", "build_refine_kernels_counters.md")
+NND_PROFILE = os.path.join(ROOT, "profiles", "nnd_kernels_cfg1_rounds_and_counters.md")
 NND_OFFERS_NOTE = ("nnd_offers: distinct offers the merge steps found in the offer tables, all rounds.  nnd_offers_declined_by_threshold: offers a "
                    "join did not send because their distance was not below the threshold their target announced (the distance of its 64th "
                    "best offer of the round before, announced only by nodes whose table was five eighths full).  Nothing depends on the order "
@@ -67,6 +68,21 @@ def measured_stage(stage, workload):
     for m in re.finditer(r"^\|\s*([\w+]+)\s*\|\s*([\w-]+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*$", text, re.M):
         if m.group(1) == stage and m.group(2) == workload:
             return float(m.group(3)), float(m.group(4)), float(m.group(5)), float(m.group(6))
+    return None
+
+
+def measured_knn(workload):
+    """(atomic lane operations issued by pairs of adjacent lanes on one line, issued by single lanes, yardstick rates of the
+    two in G/s) of the NN-descent stage of one workload, from the committed counter summary: TCP_TCC_ATOMIC_*_REQ summed
+    over the launches of a build (`rocprofv3 --pmc` run of this script), the rates from --atomic-calibration.  The build
+    is reproducible, so the counts belong to the workload.  None for a workload the file does not hold."""
+    try:
+        text = open(NND_PROFILE).read()
+    except OSError:
+        return None
+    for m in re.finditer(r"^\|\s*knn\s*\|\s*([\w-]+)\s*\|\s*(\d+)\s*\|\s*(\d+)\s*\|\s*([\d.]+)\s*\|\s*([\d.]+)\s*\|\s*$", text, re.M):
+        if m.group(1) == workload:
+            return float(m.group(2)), float(m.group(3)), float(m.group(4)), float(m.group(5))
     return None
 
 
@@ -279,6 +295,17 @@ def run_workload(args, workload, torch, want_cpu):
     stage_rooflines["assign"] = dict(hbm_stage(det["assign"], num * dim * 4 + num * 12),
                                      mfma_tflops=assign_flops / det["assign"] / 1e12 if det["assign"] > 0 else 0.0, mfma_peak_tflops=157.3)
     stage_rooflines["reorder"] = hbm_stage(det["reorder"], (num + reorder_rows) * dim * 4)
+    # The NN-descent stage is bound by what a CU's memory pipeline charges per distinct cache line, atomic operations above
+    # all: the time its atomics take at the rates of the probe kernel, as a fraction of the stage.
+    mk = measured_knn(workload)
+    if mk and res["knn_time"] > 0:
+        paired, single, rate_pairs, rate_single = mk
+        at_yardstick = paired / rate_pairs / 1e9 + single / rate_single / 1e9
+        stage_rooflines["knn"] = dict(bound="scattered atomics", seconds=res["knn_time"], atomic_lane_operations_in_pairs=int(paired),
+                                      atomic_lane_operations_single=int(single), peak_pairs=rate_pairs, peak_single=rate_single,
+                                      unit="G lane operations/s", achieved=(paired + single) / res["knn_time"] / 1e9,
+                                      seconds_at_the_yardstick_rates=at_yardstick, frac=at_yardstick / res["knn_time"],
+                                      source="profiles/" + os.path.basename(NND_PROFILE))
     if "build_counters" in res:
         _, rows, grows = res["build_counters"]
         stage_rooflines["subgraph+boundary"] = graph_stage(det["subgraph"] + det["boundary"],
