@@ -475,19 +475,11 @@ __global__ __launch_bounds__(256) void nnd_members_kernel(JoinArgs a) {
     }
 }
 
-// Six workgroups per CU (20 KB of LDS each): the join is bound by the latency of its gather -> matrix -> arg-min ->
-// offer chain, so residency matters more than registers; seven would spill.
-// `lists`: which lists are this kernel's.  kAllLists: every one.  kWideLists: those with more than 32 new members, the
-// others being nnd_join_narrow_kernel's; kWideListsFew: the same when they are expected to be few -- the counts are
-// then read first, and a workgroup that passes over its list has asked for 8 bytes instead of the whole member list.
-constexpr int kAllLists = 0, kWideLists = 1, kWideListsFew = 2;
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a, int lists) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    JoinLds& L = *reinterpret_cast<JoinLds*>(smem);
-    const uint32_t node = blockIdx.x;
-    if (node >= a.num) return;
+// The join of one list by a workgroup of four wavefronts.  `lists`: which lists are the caller's.  kAllLists: every
+// one; kWideLists: those with more than 32 new members, the others being nnd_join_narrow_kernel's.
+constexpr int kAllLists = 0, kWideLists = 1;
+__device__ __forceinline__ void join_list(const JoinArgs& a, JoinLds& L, const uint32_t node, const int lists) {
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
-    if (lists == kWideListsFew && a.member_counts[static_cast<size_t>(node) * 2] <= kSamples) return;
     // member ids are fetched before their counts are known (one memory round trip instead of two); slots beyond a
     // list hold what an earlier round left there, and count for nothing: their norm below is infinite
     const uint32_t member = tid < static_cast<int>(2 * kBi) ? a.members[static_cast<size_t>(node) * (2 * kBi) + tid] : kInvalid;
@@ -688,6 +680,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) voi
     send(of_column);
     send(of_row);
     if (declined && a.stats) atomicAdd(&a.stats[2 * (blockIdx.x & 1023u) + 1], static_cast<unsigned long long>(declined));
+}
+
+// Six workgroups per CU (20 KB of LDS each): the join is bound by the latency of its gather -> matrix -> arg-min ->
+// offer chain, so residency matters more than registers; seven would spill.  One workgroup per list.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 6))) void nnd_join_kernel(JoinArgs a, int lists) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (blockIdx.x < a.num) join_list(a, *reinterpret_cast<JoinLds*>(smem), blockIdx.x, lists);
+}
+
+// The same for the rounds in which few lists are wide: a workgroup looks at the counts of a run of 16 lists (one cache
+// line) and joins the wide ones among them, one after the other.  A million workgroups that look at one list each and
+// leave would cost 0.4 ms a round.  Four workgroups per CU: the loop would spill at six, and the few lists there are do
+// not fill them.
+constexpr uint32_t kWideRun = 16;
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void nnd_join_runs_kernel(JoinArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t first = blockIdx.x * kWideRun, mine = first + (threadIdx.x & 63u);
+    const bool wide = (threadIdx.x & 63u) < kWideRun && mine < a.num && a.member_counts[static_cast<size_t>(mine) * 2] > kSamples;
+    uint32_t todo = static_cast<uint32_t>(ballot(wide));   // the same in all four wavefronts
+    while (todo) {
+        const uint32_t j = static_cast<uint32_t>(__ffs(static_cast<int>(todo)) - 1);
+        todo &= todo - 1;
+        join_list(a, *reinterpret_cast<JoinLds*>(smem), first + j, kWideLists);
+        __syncthreads();   // the next list overwrites what this one kept in LDS
+    }
 }
 
 // ---- local join of a list with at most 32 new members (rows of up to 128 dims): one wavefront, no barrier ---------
@@ -1588,13 +1605,18 @@ int nnd_reverse(const NndCtx& c) {
 int nnd_join(const NndCtx& c, bool with_stats, bool few_wide = false, bool early = true) {
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(sizeof(JoinLds))));
+    GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&nnd_join_runs_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(sizeof(JoinLds))));
     JoinArgs ja{c.half_rows, c.norms, c.fwd_new, c.fwd_old, c.rev_new, c.rev_old, c.rev_tables, c.rev_thr, c.counts, c.members, c.member_counts, c.offers, offer_slots_for(c.l.width),
                 offer_slots_for(c.l.width) == 512 ? 23u : 24u, c.round, with_stats ? c.stats : nullptr, c.n, c.l.dim_pad, c.segs};
     hipLaunchKernelGGL(nnd_members_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ja);
     // lists with at most 32 new members go to the one-wavefront kernel, the others to the workgroup kernel; each passes
     // over the other's lists
     const bool narrow = c.l.dim_pad <= kNarrowJoinMaxDim;
-    hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja, !narrow ? kAllLists : few_wide ? kWideListsFew : kWideLists);
+    if (narrow && few_wide)
+        hipLaunchKernelGGL(nnd_join_runs_kernel, dim3(ceil_div(c.n, kWideRun)), dim3(256), sizeof(JoinLds), c.s, ja);
+    else
+        hipLaunchKernelGGL(nnd_join_kernel, dim3(c.n), dim3(256), sizeof(JoinLds), c.s, ja, narrow ? kWideLists : kAllLists);
     if (narrow) hipLaunchKernelGGL(nnd_join_narrow_kernel, dim3(c.n), dim3(64), 0, c.s, ja, early);
     return launch_status();
 }

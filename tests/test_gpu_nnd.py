@@ -195,7 +195,7 @@ def test_nnd_same_seed_same_graph(hip):
 @pytest.mark.parametrize("k,dim", [(32, 128), (64, 96), (32, 200)])
 def test_nnd_build_equals_its_stages(hip, k, dim):
     """glide_hip_nnd_build takes shortcuts its stage entry points do not: the merge kernel scatters the next round's
-    reverse samples itself, from the fourth round on the workgroup join looks at a list's counts before its members,
+    reverse samples itself, from the fourth round on the workgroup join takes runs of 16 lists per workgroup,
     and from the fifth the joins no longer read a slot before sending to it.  None of this may show: eight rounds run
     stage by stage must end in the very graph the fused build gives (dims with and without the one-wavefront join)."""
     from glide_amd import datasets as D
