@@ -77,7 +77,7 @@ def cpu_leg():
 def run(args, info):
     import torch
     from glide_amd import datasets as D
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    root = os.path.dirname(os.path.abspath(__file__))
     bindir = os.path.join(root, "glide_amd", "bin")
     for exe in ("large_preprocess", "large_knn", "large_build", "large_search"):
         if not os.path.exists(os.path.join(bindir, exe)):

@@ -393,18 +393,6 @@ def widen_u8(src, count, dst, stream=None):
     check(lib().glide_hip_widen_u8(_ptr(src), C.c_size_t(count), _ptr(dst), vp(stream)), "glide_hip_widen_u8")
 
 
-def valu_probe(mode, rounds, out, stream=None):
-    check(lib().glide_hip_valu_probe(C.c_int(mode), u32(rounds), _ptr(out), vp(stream)), "glide_hip_valu_probe")
-
-
-def atomic_probe(mode, table, slots, rounds, out, stream=None):
-    check(lib().glide_hip_atomic_probe(C.c_int(mode), _ptr(table), u32(slots), u32(rounds), _ptr(out), vp(stream)), "glide_hip_atomic_probe")
-
-
-def copy_bytes(dst, src, nbytes, stream=None):
-    check(lib().glide_hip_copy_bytes(_ptr(dst), _ptr(src), C.c_size_t(nbytes), vp(stream)), "glide_hip_copy_bytes")
-
-
 def build_segment(segment_data, num, dim, knn_graph, knn_degree, start_point, graph_degree, beam, max_iterations,
                   min_iterations, hash_bit, hash_reset_interval, relaxant, metric, graph, counters=None, stream=None):
     check(lib().glide_hip_build_segment(_ptr(segment_data), u32(num), u32(dim), _ptr(knn_graph), u32(knn_degree),

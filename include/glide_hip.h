@@ -412,21 +412,6 @@ int glide_hip_stream_wait_event(void *stream, void *event);
 int glide_hip_widen_u8(const unsigned char *src, size_t count, float *dst, void *stream);
 
 /* ---- test hooks for the device primitives (subsystems 5, 6 and the hash set) ------------------------------ */
-/* A plain copy kernel (bytes % 16 == 0, 16-byte aligned): no counterpart in the reference; it is the transfer
- * of known size against which hardware byte counters (FETCH_SIZE / WRITE_SIZE) are calibrated. */
-int glide_hip_copy_bytes(void *dst, const void *src, size_t bytes, void *stream);
-/* A register-only kernel of 2048 x 256 threads, each running rounds x 16 independent steps: no counterpart in the
- * reference; it is the yardstick for the vector-ALU issue rate against which the instruction counters of the build and
- * search kernels are read.  mode 0: fused multiply-add, 1: integer add, 2: compare + select (two instructions a step),
- * 3: DPP cross-lane move + add (two a step).  out: one float. */
-int glide_hip_valu_probe(int mode, uint32_t rounds, float *out, void *stream);
-/* 2048 x 256 threads, each issuing `rounds` atomic operations on pseudo-random 8-byte slots of `table` (`slots` of
- * them, a power of two; the caller sets the table's contents): no counterpart in the reference; it is the yardstick for
- * the rate of scattered atomics against which the NN-descent kernels' offers and slot reservations are read.
- * mode 0: 64-bit minimum without a returned value, 1: 32-bit add whose result is used, 2 / 3: as 0 with 2 / 16 adjacent
- * lanes on slots of one 128-byte line.  out: one u32. */
-int glide_hip_atomic_probe(int mode, unsigned long long *table, uint32_t slots, uint32_t rounds, uint32_t *out,
-                           void *stream);
 /* compute_similarity_warp (distance.cuh:9-27): out[i] = dist(a[i], b[i]) for n row pairs */
 int glide_hip_distance_batch(const float *a, const float *b, uint32_t n, uint32_t dim, int metric, float *out,
                              void *stream);

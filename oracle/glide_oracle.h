@@ -20,7 +20,15 @@
  *   prune                  RNG invariant over kept pairs, brute force on tiny pools (pinned)
  *   boundary merge         hand-worked rows for both branches                       (pinned)
  *   reverse edges          invariants + brute force                                 (pinned)
- *   beam search            recall vs exact brute force; bit-exactness is GPU-vs-oracle only
+ *   beam search            recall vs exact brute force; the visited-set reset + restore by a hand-derived run
+ *                          on a path graph (results, iterations, rows scored for six reset intervals, a table
+ *                          that overflows unless it is cleared) and by equality with a reset-free search (pinned)
+ *   refine                 hand-worked rows on a 12-point line graph + a float64 model written from the
+ *                          definition (first admissible head, heads before it dropped, holes in slot order),
+ *                          every row of random graphs with holes                    (pinned)
+ *   segment choice         numpy: float64 distances, stable argsort, ratio test, top-up (pinned)
+ *   large-path result merge  sorted union of the partitions' own top-k (from the small path's search),
+ *                          any partition order, unlisted partitions and list gaps     (pinned)
  *   NN-descent             parity unpinned bit-wise (the reference is unseeded and racy);
  *                          statistical: graph recall vs exact kNN
  *   k-means (cuVS)         parity unpinned (third-party, absent from the reference tree); the stand-in

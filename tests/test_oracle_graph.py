@@ -180,3 +180,216 @@ def test_bruteforce_matches_numpy():
     full = ((data[None].astype(np.float64) - q[:, None].astype(np.float64)) ** 2).sum(-1)
     assert np.array_equal(ids, np.argsort(full, 1)[:, :5])
     assert np.allclose(d, np.sqrt(np.sort(full, 1)[:, :5]), rtol=1e-5)
+
+
+# ---------------------------------------------------------------- large-path segment choice (reference search_kernel.cuh:546-607)
+def test_select_segments_against_numpy():
+    """Ranked centroid ids while d_i / d_0 <= boundary_factor, topped up to min_segment_num, the rest 0xffffffff --
+    written here from float64 distances and a stable argsort."""
+    rng = np.random.default_rng(11)
+    for C, dim, metric in ((7, 16, 0), (24, 32, 0), (40, 8, 0), (12, 16, 1)):
+        cent = rng.standard_normal((C, dim)).astype(np.float32) * 3
+        q = rng.standard_normal((200, dim)).astype(np.float32) * 3
+        d = ((q[:, None].astype(np.float64) - cent[None].astype(np.float64)) ** 2).sum(-1)
+        if metric == 0:
+            d = np.sqrt(d)                                   # Euclidean distances are square roots everywhere (distance.cuh:22-26)
+        order = np.argsort(d, 1, kind="stable")
+        ds = np.take_along_axis(d, order, 1)
+        for min_seg, bf in ((1, 1.0), (1, 1.3), (3, 1.15), (C, 1.05), (2, 50.0)):
+            got = O.select_segments(q, cent, min_seg, bf, metric)
+            ratio = ds / ds[:, :1]
+            clear = (np.abs(ratio[:, 1:] - bf) > 1e-5).all(1) & (np.diff(ds, axis=1) > 1e-6 * ds[:, 1:]).all(1)   # away from ties of the two roundings
+            assert clear.sum() > 150
+            take = np.maximum((ratio <= bf).sum(1), min_seg)
+            want = np.where(np.arange(C)[None] < take[:, None], order, INV).astype(np.uint32)
+            assert np.array_equal(got[clear], want[clear]), (C, metric, min_seg, bf)
+            assert (got[:, 0] == order[:, 0])[clear].all()   # the nearest partition is always listed first
+
+
+# ---------------------------------------------------------------- large-path result merge (reference search_kernel.cuh:609-765)
+def test_search_sub_merges_partitions_like_a_sorted_union():
+    """Three partitions searched one after another into one running top-k: the result is the sorted union of each
+    partition's own top-k, ids through the partition's map, whatever the order of the partitions; a partition a query does
+    not list leaves its row alone, and the scan of the list stops at the first 0xffffffff.  The partitions' own top-k
+    come from the small path's search (one centroid, the same start point: `get_init` with no excluded id is
+    `result_init` with one centroid), so the merge is held against numpy, not against itself."""
+    rng = np.random.default_rng(12)
+    dim, deg, top_k, nq = 16, 8, 10, 40
+    sp = O.search_params(32, deg)
+    parts = []
+    for s, n in enumerate((300, 180, 420)):
+        data = rng.standard_normal((n, dim)).astype(np.float32) + s       # generic floats: distances are distinct
+        knn, _ = O.bruteforce_knn(data, data, deg, exclude_self=True)
+        mp = (rng.permutation(5000)[:n] + 10_000 * s).astype(np.uint32)
+        parts.append((data, knn, mp, int(rng.integers(0, n))))
+    queries = rng.standard_normal((nq, dim)).astype(np.float32) + 1
+    own = []
+    for data, knn, mp, start in parts:
+        ids, dists, _ = O.search(data, knn, data[:1].copy(), np.array([start], np.uint32), queries, top_k, **sp)
+        own.append((mp[ids], dists))
+    # lists: queries 0..9 list all three, 10..19 only partitions 2 and 0, 20..29 only partition 1,
+    # 30..39 list partition 1, then 0xffffffff, then partition 2 behind it (never seen: the scan stops at the gap)
+    seg = np.full((nq, 3), INV, np.uint32)
+    seg[:10] = [0, 1, 2]
+    seg[10:20, :2] = [2, 0]
+    seg[20:30, 0] = 1
+    seg[30:, 0], seg[30:, 2] = 1, 2
+    listed = [(0, 1, 2)] * 10 + [(0, 2)] * 10 + [(1,)] * 20
+    for order in ((0, 1, 2), (2, 0, 1), (1, 2, 0)):
+        fi = np.full((nq, top_k), INV, np.uint32)
+        fd = np.full((nq, top_k), np.finfo(np.float32).max, np.float32)
+        for s in order:
+            data, knn, mp, start = parts[s]
+            O.search_sub(data, knn, mp, queries, seg, s, start, top_k, sp, fi, fd)
+        for q in range(nq):
+            ids = np.concatenate([own[s][0][q] for s in listed[q]])
+            ds = np.concatenate([own[s][1][q] for s in listed[q]])
+            assert np.unique(ds).size == ds.size
+            o = np.argsort(ds)[:top_k]
+            assert np.array_equal(fi[q], ids[o]) and np.array_equal(fd[q], ds[o]), (order, q)
+
+
+# ---------------------------------------------------------------- refine (reference graph_kernel.cuh:455-673)
+def refine_model(data, graph, start, relax, p):
+    """`refine_kernel` for one point, written from its definition in float64 for a beam that holds every reachable node:
+    then the beam is the set reachable from the start point's neighbours (the point itself is not expanded into, but may
+    sit among the start point's neighbours), sorted by distance."""
+    row = graph[p]
+    holes = np.nonzero(row == INV)[0]
+    if holes.size == 0:
+        return row.copy()
+    dist = lambda a, b: np.sqrt(((data[a].astype(np.float64) - data[b].astype(np.float64)) ** 2).sum())
+    seen = [int(x) for x in graph[start] if x != INV]
+    todo = list(seen)
+    while todo:
+        u = todo.pop()
+        for v in graph[u]:
+            v = int(v)
+            if v != INV and v != p and v not in seen:
+                seen.append(v)
+                todo.append(v)
+    pool = sorted(seen, key=lambda x: dist(p, x))
+    fills = []
+    while len(fills) < holes.size and pool:
+        ok = [i for i, x in enumerate(pool) if x != p and x not in row.tolist()]      # select_point: the first admissible entry
+        if not ok:
+            break
+        h = pool[ok[0]]
+        fills.append(h)
+        pool = [x for x in pool[ok[0]:] if not (relax * dist(h, x) < dist(p, x))]       # entries before the head are dropped too
+    out = row.copy()
+    out[holes[:len(fills)]] = fills
+    return out
+
+
+BIG_BEAM = dict(beam=64, max_iterations=4000, min_iterations=0, hash_bit=12, hash_reset_interval=1 << 20)
+
+
+def test_refine_hand_built_line_graph():
+    """Twelve points on a line with growing gaps.  With relaxant 1 a chosen neighbour removes everything behind it on its
+    side of the point and nothing on the other side, so a row gets the nearest admissible point, then the nearest
+    admissible farther point on the other side, and nothing more."""
+    x = np.cumsum([0, 1, 1.1, 1.2, 1.3, 1.4, 1.5, 1.6, 1.7, 1.8, 1.9, 2.0])
+    data = np.zeros((12, 4), np.float32)
+    data[:, 0] = x
+    g = np.full((12, 4), INV, np.uint32)
+    for i in range(12):
+        g[i, 0] = i + 1 if i < 11 else 10
+        g[i, 1] = i - 1 if i > 0 else 5          # row 0 (the start point) also names 5: point 5 meets itself in its beam
+    full = g.copy()
+    full[:, 2], full[:, 3] = (np.arange(12) + 2) % 12, (np.arange(12) + 3) % 12   # rows without holes
+    g[3] = full[3]
+    g[5] = [6, INV, 4, INV]                      # holes at slots 1 and 3
+    g[8] = [9, 7, 10, INV]                       # one hole
+    g[2, 1] = INV                                # row 2 = [3, INV, INV, INV]: three holes, only two points can be chosen
+    cent, sps = data[:1].copy(), np.array([0], np.uint32)
+    got, _ = O.refine(data, g, cent, sps, BIG_BEAM, 1.0)
+    assert np.array_equal(got[3], g[3])                                   # no hole: untouched
+    # point 5 (x = 6.0): by distance 4 (1.4, in the row), 6 (1.5, in the row), 3 (2.7) <- first admissible; behind it on
+    # the left 2, 1, 0 fall, on the right 7 (3.1) is the next head; after it nothing is left.  5 itself (distance 0, from
+    # the start point's row) is skipped.
+    assert got[5].tolist() == [6, 3, 4, 7]
+    # point 8 (x = 10.8): 7 and 9 are in the row, 10 is in the row, 6 (3.3) is the first admissible; one hole, one pick
+    assert got[8].tolist() == [9, 7, 10, 6]
+    # point 2 (x = 2.1): 1 (1.1) first, then 3 (1.2) is in the row -> 4 (2.5); the third hole stays empty
+    assert got[2].tolist() == [3, 1, 4, INV]
+    for p in range(12):
+        assert np.array_equal(got[p], refine_model(data, g, 0, 1.0, p)), p
+
+
+def test_refine_against_definition_on_random_graphs():
+    rng = np.random.default_rng(13)
+    for n, deg, relax in ((60, 4, 1.05), (150, 8, 1.05), (150, 8, 1.3)):
+        data = rng.standard_normal((n, 8)).astype(np.float32)
+        g, _ = O.bruteforce_knn(data, data, deg, exclude_self=True)
+        g = np.ascontiguousarray(g[:, rng.permutation(deg)])
+        g[rng.random((n, deg)) < 0.35] = INV
+        g[0, 0] = 7                                                       # the start point's row is not empty
+        sp = dict(BIG_BEAM, beam=256)
+        got, _ = O.refine(data, g, data[:1].copy(), np.array([0], np.uint32), sp, relax)
+        dist = lambda a, b: np.sqrt(((data[a].astype(np.float64) - data[b].astype(np.float64)) ** 2).sum())
+        for p in range(n):
+            assert np.array_equal(got[p], refine_model(data, g, 0, relax, p)), (n, p)
+            old, new = g[p], got[p]
+            assert ((new == old) | (old == INV)).all()                    # only holes change
+            added = new[(old == INV) & (new != INV)].tolist()
+            assert p not in added and not set(added) & set(old.tolist()) and len(set(added)) == len(added)
+            for i, a in enumerate(added):                                 # no chosen neighbour occludes a later one
+                for b in added[i + 1:]:
+                    assert relax * dist(a, b) >= dist(p, b) * (1 - 1e-6)
+            holes = np.nonzero(old == INV)[0]
+            assert (new[holes[len(added):]] == INV).all()                 # filled in slot order, front first
+
+
+# ---------------------------------------------------------------- visited-set reset and restore (reference search_kernel.cuh:327-334,438-469)
+def path_with_far_node(n):
+    """Nodes 0..n-1 at x = 0..n-1, node i -> (i + 1, F); F = node n far away on the other side.  Query beyond the last node."""
+    data = np.zeros((n + 1, 4), np.float32)
+    data[:n, 0] = np.arange(n)
+    data[n, 0] = -1000.0
+    g = np.full((n + 1, 2), INV, np.uint32)
+    g[:n, 0] = np.arange(1, n + 1)
+    g[n - 1, 0] = INV
+    g[:n, 1] = n
+    q = np.zeros((1, 4), np.float32)
+    q[0, 0] = n - 1 + 0.25
+    return data, g, q
+
+
+def test_hash_reset_and_restore_on_a_path():
+    """Hand-derived run.  The search enters at node 1 and F (the neighbours of start point 0) and walks one node per
+    iteration: iteration j expands node j + 1.  The beam (32) holds F until 32 path nodes are known, i.e. until the merge
+    at the top of iteration 31.  A reset empties the visited set and the restore puts the beam back, so from then on F is
+    forgotten by every reset and scored once more by the expansion that follows it; path nodes in the beam never are.
+    Rows scored = n path nodes... minus the start point (never scored) + F once + one per reset in iterations 31..n-2.
+    The table has 64 slots: without the clearing it overflows after 64 nodes and the walk stops; without the restore the
+    node behind the parent would be scored again on every step."""
+    n = 120
+    data, g, q = path_with_far_node(n)
+    cent, sps = data[:1].copy(), np.array([0], np.uint32)
+    want_ids = np.arange(n - 1, n - 11, -1)
+    want_d = (q[0, 0] - np.arange(n - 1, n - 11, -1)).astype(np.float32)
+    for reset in (1, 2, 3, 5, 7, 1 << 20):
+        hash_bit = 6 if reset <= 7 else 10
+        ids, dists, st = O.search(data, g, cent, sps, q, 10, 32, 1000, 0, hash_bit, reset)
+        assert ids[0].tolist() == want_ids.tolist() and np.array_equal(dists[0], want_d), reset
+        resets_after_eviction = sum(1 for j in range(31, n - 1) if (j + 1) % reset == 0)
+        assert st["iterations"] == n, (reset, st)
+        assert st["graph_rows"] == n, (reset, st)                       # the start point's row + one row per expanded node 1..n-1
+        assert st["rows_scored"] == (n - 1) + 1 + resets_after_eviction, (reset, st)
+
+
+def test_hash_reset_every_iteration_returns_no_id_twice():
+    rng = np.random.default_rng(14)
+    data = rng.standard_normal((3000, 16)).astype(np.float32)
+    knn, _ = O.bruteforce_knn(data, data, 16, exclude_self=True)
+    queries = rng.standard_normal((100, 16)).astype(np.float32)
+    cent, sps = data[:1].copy(), np.array([17], np.uint32)
+    base = O.search(data, knn, cent, sps, queries, 32, 64, 400, 0, 13, 1 << 20)
+    for reset in (1, 2, 3):
+        ids, dists, st = O.search(data, knn, cent, sps, queries, 32, 64, 400, 0, 8, reset)
+        for row in ids:
+            assert np.unique(row).size == row.size
+        # a forgotten node is farther than everything the beam held when it left, so scoring it again changes nothing
+        assert np.array_equal(ids, base[0]) and np.array_equal(dists, base[1])
+        assert st["rows_scored"] > base[2]["rows_scored"] and st["iterations"] == base[2]["iterations"]
