@@ -277,6 +277,13 @@ def partition_assign(data, num, dim, centroids, centroid_num, boundary_factor, m
                                            C.c_size_t(workspace_bytes), vp(stream)), "glide_hip_partition_assign")
 
 
+def mem_info():
+    """(free, total) bytes of device memory on the current device."""
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    check(lib().glide_hip_mem_info(C.byref(free), C.byref(total)), "glide_hip_mem_info")
+    return free.value, total.value
+
+
 def partition_assign_fixed_max_points():
     f = lib().glide_hip_partition_assign_fixed_max_points
     f.restype = C.c_uint32

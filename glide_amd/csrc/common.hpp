@@ -18,7 +18,8 @@ constexpr int kWave = 64;
 enum Metric : int { kEuclidean = 0, kCosine = 1 };  // reference params.cuh:5-8
 
 __host__ __device__ constexpr uint32_t round_up32(uint32_t p) { return (p + 31u) & ~31u; }  // utils.cuh:21-23
-__host__ __device__ constexpr uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+// a / b rounded up, without the wrap of (a + b - 1) when a is within b of 2^32
+__host__ __device__ constexpr uint32_t ceil_div(uint32_t a, uint32_t b) { return a / b + (a % b != 0); }
 
 __device__ __forceinline__ int lane_id() { return static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))); }
 

@@ -1595,7 +1595,7 @@ int nnd_prepare(const NndCtx& c, const float* data, uint32_t dim, uint32_t seed)
 }
 
 int nnd_reverse(const NndCtx& c) {
-    hipLaunchKernelGGL(nnd_reverse_kernel, dim3(ceil_div(c.n * 64, 256)), dim3(256), 0, c.s, c.fwd_new, c.fwd_old, c.counts, c.rev_new, c.rev_old,
+    hipLaunchKernelGGL(nnd_reverse_kernel, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.fwd_new, c.fwd_old, c.counts, c.rev_new, c.rev_old,
                        c.rev_tables, c.rev_thr, c.n, c.segs);
     return launch_status();
 }
@@ -1694,7 +1694,7 @@ int glide_hip_nnd_layout(uint32_t reorder_num, uint32_t dim, uint32_t knn_degree
     out->fwd_new = l.fwd_new; out->fwd_old = l.fwd_old; out->rev_new = l.rev_new; out->rev_old = l.rev_old; out->rev_tables = l.rev_tables; out->rev_thr = l.rev_thr;
     out->counts = l.counts; out->members = l.members; out->member_counts = l.member_counts; out->offers = l.offers; out->bloom = l.bloom;
     out->segment_state = l.seg_state; out->segment_updates = l.seg_updates; out->round = l.round; out->total = l.total;
-    out->width = l.width; out->reverse_cap = kRevCap; out->reverse_stride = kRevStride; out->offer_slots = offer_slots_for(l.width); out->reverse_slots = kRevSlots; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets;
+    out->width = l.width; out->reverse_cap = kRevCap; out->reverse_stride = kRevStride; out->offer_slots = offer_slots_for(l.width); out->reverse_slots = kRevSlots; out->row_halfs = l.dim_pad; out->bloom_sets = l.bloom_sets; out->reserved = 0;
     return GLIDE_OK;
 }
 

@@ -47,6 +47,14 @@ int glide_hip_device_info(char* name, size_t name_len, int* compute_units, size_
     return GLIDE_OK;
 }
 
+int glide_hip_mem_info(size_t* free_bytes, size_t* total_bytes) {
+    size_t f = 0, t = 0;
+    GLIDE_HIP_TRY(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return GLIDE_OK;
+}
+
 int glide_hip_malloc(void** ptr, size_t bytes) {
     if (!ptr) return GLIDE_ERR_BAD_ARGUMENT;
     GLIDE_HIP_TRY(hipMalloc(ptr, bytes ? bytes : 1));

@@ -109,3 +109,30 @@ def recall(result_ids, truth_ids, k):
     for r, t in zip(result_ids[:, :k], truth_ids[:, :k]):
         hit += len(set(r.tolist()) & set(t.tolist()))
     return hit / float(result_ids.shape[0] * k)
+
+
+def reachable_recall_bound(graph, centroids, start_points, queries, gt, metric=0):
+    """Upper bound on recall@k of ANY beam width on a finished index, from the reference's entry rule alone: a search enters
+    through the single start point of the query's nearest centroid (search_kernel.cuh:270-271; one random start point per
+    partition, glide_impl.cuh:43-75) and only ever scores neighbours of nodes it has scored, so a true neighbour outside the
+    set reachable from that start point over directed graph edges cannot be returned.  Returns (bound, fraction of the
+    points reachable from the average start point).  Host-side breadth-first search over the N x D id table."""
+    from scipy.sparse import csr_matrix
+    from scipy.sparse.csgraph import breadth_first_order
+    n, deg = graph.shape
+    valid = graph != 0xFFFFFFFF
+    indptr = np.concatenate([[0], np.cumsum(valid.sum(1))]).astype(np.int64)
+    adj = csr_matrix((np.ones(int(indptr[-1]), np.int8), graph[valid].astype(np.int64), indptr), shape=(n, n))
+    q64, c64 = queries.astype(np.float64), centroids.astype(np.float64)
+    nearest = ((q64 * q64).sum(1)[:, None] - 2.0 * q64 @ c64.T + (c64 * c64).sum(1)[None]).argmin(1)
+    hits, sizes = np.zeros(queries.shape[0]), []
+    for c in np.unique(nearest):
+        sp = int(start_points[c])
+        order = breadth_first_order(adj, sp, directed=True, return_predecessors=False)
+        reach = np.zeros(n, bool)
+        reach[order] = True
+        reach[sp] = bool((graph[order] == sp).any())   # the start point itself is only scored if an edge leads back to it
+        sizes.append(reach.mean())
+        mine = np.nonzero(nearest == c)[0]
+        hits[mine] = reach[gt[mine].astype(np.int64)].mean(1)
+    return float(hits.mean()), float(np.mean(sizes)), hits

@@ -38,6 +38,9 @@ const char *glide_hip_error_string(int code);
 /* replaces the hard-coded cudaSetDevice(1) of the reference mains (small_build.cu:33) */
 int glide_hip_set_device(int device);
 int glide_hip_device_info(char *name, size_t name_len, int *compute_units, size_t *total_mem);
+/* free and total device memory of the current device (hipMemGetInfo); no counterpart in the reference: lets a host
+ * size its staging buffers and lets a test see that an entry point allocates nothing */
+int glide_hip_mem_info(size_t *free_bytes, size_t *total_bytes);
 
 /* memory / stream / event helpers for hosts that have no HIP runtime of their own
  * (replace raft::make_device_matrix / raft::copy / rmm stream pool / cudaEvent use, glide_impl.cuh:15-41,53-72) */

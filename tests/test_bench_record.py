@@ -64,7 +64,9 @@ def test_reachable_recall_bound_on_a_hand_built_graph():
     start_points = np.array([0, 4], np.uint32)
     queries = np.array([[1.0, 0.0], [9.0, 0.0], [9.0, 1.0]], np.float32)
     gt = np.array([[0, 1], [4, 3], [7, 6]], np.uint32)   # query 0: start point 0 is never scored (no edge back), 1 is reachable
-    bound, frac = bench.reachable_recall_bound(graph, centroids, start_points, queries, gt)
+    from glide_amd import datasets as Ds
+    bound, frac, per_query = Ds.reachable_recall_bound(graph, centroids, start_points, queries, gt)
+    assert per_query.tolist() == [0.5, 0.5, 1.0]
     # query 0: {1} of {0, 1} -> 0.5; query 1: 4 reachable (edge back), 3 on the other chain -> 0.5; query 2: both -> 1.0
     assert abs(bound - (0.5 + 0.5 + 1.0) / 3) < 1e-12
     assert abs(frac - (3 / 8 + 4 / 8) / 2) < 1e-12

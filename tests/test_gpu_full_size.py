@@ -223,3 +223,32 @@ def test_search_properties(hip, world, beam):
     print("beam", beam, "recall@10", r, flush=True)
     if world["kind"] == "lowdim_integer":
         assert r >= (0.96 if beam == 32 else 0.99)
+
+
+def test_recall_is_bounded_by_what_the_entry_point_reaches(hip, world):
+    """A search enters through the one start point of the query's nearest centroid (search_kernel.cuh:270-271,
+    glide_impl.cuh:43-75) and only scores neighbours of nodes it has scored: a true neighbour that no directed path from
+    that start point reaches cannot be returned at any beam.  The bound is computed on the host by breadth-first search
+    over the finished 1M x 32 graph; every beam of the reference's range must stay below it query by query, and the widest
+    beam must come close to it -- which is what makes the low recall of the mixtures a property of the algorithm on that
+    data (components the kNN graph does not connect) and not of this implementation."""
+    from glide_amd import datasets as Ds, index as G
+    gt = _truth(world)
+    m = gt.shape[0]
+    bound, reach_frac, per_query = Ds.reachable_recall_bound(world["graph"], world["centroids"], world["start_points"], world["queries"][:m], gt,
+                                                             world["metric"])
+    print(world["kind"], "reachable bound on recall@10: %.4f; an average start point reaches %.3f of the points" % (bound, reach_frac), flush=True)
+    recalls = {}
+    for beam in (32, 64, 128, 256, 512):
+        sp = G.make_search_parameter(beam, D, 10)
+        ids, _ = world["index"].search(sp, world["d_queries"])
+        found = np.array([np.isin(ids[q], gt[q]).sum() / 10.0 for q in range(m)])
+        assert (found <= per_query + 1e-9).all(), "beam %d returned a true neighbour the entry point cannot reach" % beam
+        recalls[beam] = float(found.mean())
+    print(world["kind"], "recall@10 by beam", {b: round(r, 4) for b, r in recalls.items()}, flush=True)
+    assert all(recalls[a] <= recalls[b] + 0.005 for a, b in zip((32, 64, 128, 256), (64, 128, 256, 512)))
+    assert recalls[512] <= bound and bound - recalls[512] <= 0.05
+    if world["kind"] == "lowdim_integer":
+        assert bound >= 0.999 and recalls[32] >= 0.96
+    else:
+        assert bound < 0.5, "the mixtures' components are not connected: no beam can reach recall@10 0.95"

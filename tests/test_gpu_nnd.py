@@ -185,11 +185,12 @@ def test_nnd_same_seed_same_graph(hip):
         a, st_a = gpu_nnd(hip, data, seg_start, seg_len, k, rounds, seed=3)
         b, st_b = gpu_nnd(hip, data, seg_start, seg_len, k, rounds, seed=3)
         c, _ = gpu_nnd(hip, data, seg_start, seg_len, k, rounds, seed=4)
-        # st[1] counts arrivals turned away by a full bucket: copies of one offer may be counted once or twice, depending on
-        # whether the second copy still finds the first; what the tables end up holding (st[0]) does not depend on that
-        assert np.array_equal(a, b) and st_a[0] == st_b[0]
+        # st[0]: distinct offers the merge steps found in the tables; st[1]: offers a join did not send because they were not
+        # below the threshold their target had announced.  A join decides that per offer from values fixed before the round
+        # starts, so both counts repeat with the graph
+        assert np.array_equal(a, b) and st_a[0] == st_b[0] and st_a[1] == st_b[1]
         assert not np.array_equal(a, c)
-        print("degree %d: offers merged %d, dropped by full buckets %d" % (k, st_a[0], st_a[1]))
+        print("degree %d: offers merged %d, declined by a target's threshold %d" % (k, st_a[0], st_a[1]))
 
 
 @pytest.mark.parametrize("k,dim", [(32, 128), (64, 96), (32, 200)])

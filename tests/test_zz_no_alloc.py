@@ -77,3 +77,32 @@ def test_fixed_scratch_rejects_oversize_and_bad_arguments(hip):
     hip.partition_assign_fixed(d_data, 0, dim, d_cent, c, 1.04, 0, seg_idx, seg_len, None)
     hip.synchronize()
     assert np.array_equal(seg_len.numpy(), np.zeros(c + 1, np.uint32))
+
+
+def test_fixed_scratch_calls_allocate_nothing(hip):
+    """What the entry point is for: once its first call on the device has looked up the scratch array, further calls of
+    any size leave the device's free memory where it was (every input and output is allocated beforehand)."""
+    from oracle import oracle as O
+    cases = []
+    for n, dim, c in ((4096, 128, 16), (65536, 128, 256), (333, 64, 5), (20000, 96, 40)):
+        data = lowdim_data(n, dim, seed=n)
+        cent = O.kmeans(data[:: max(1, n // 1000)], c, iterations=2)
+        cases.append((n, dim, c, hip.DeviceArray.from_numpy(data), hip.DeviceArray.from_numpy(cent), hip.DeviceArray((n, 3), np.uint32),
+                      hip.DeviceArray(c + 1, np.uint32), hip.DeviceArray((n, 2), np.float32)))
+    n, dim, c, d_data, d_cent, seg_idx, seg_len, nearest = cases[0]
+    hip.partition_assign_fixed(d_data, n, dim, d_cent, c, 1.04, 0, seg_idx, seg_len, nearest)      # first call: symbol lookup
+    hip.synchronize()
+    free_before, total = hip.mem_info()
+    assert 0 < free_before <= total
+    for _ in range(3):
+        for n, dim, c, d_data, d_cent, seg_idx, seg_len, nearest in cases:
+            print("fixed call", n, dim, c, flush=True)
+            hip.partition_assign_fixed(d_data, n, dim, d_cent, c, 1.04, 0, seg_idx, seg_len, nearest)
+            assert hip.mem_info()[0] == free_before, "a call changed the device's free memory while it was in flight"
+    hip.synchronize()
+    assert hip.mem_info()[0] == free_before
+    # the workspace form needs memory the caller brings: the same figure moves when that workspace is allocated
+    wb = hip.partition_assign_workspace_bytes(65536, 256)
+    ws = hip.DeviceArray(max(wb // 4 + 1, 1 << 20), np.uint32)
+    assert hip.mem_info()[0] < free_before
+    ws.free()
