@@ -119,6 +119,9 @@ def parse():
                     help="only run the register-only multiply-add kernel (yardstick for the vector-ALU issue rate) and exit")
     ap.add_argument("--atomic-calibration", action="store_true",
                     help="only run the scattered-atomics kernel (yardstick for the NN-descent offers and slot reservations) and exit")
+    ap.add_argument("--gather-calibration", action="store_true",
+                    help="only run the scattered-row read kernel (yardstick for the search kernels' row gathers) and exit")
+    ap.add_argument("--queries", type=int, default=0, help="use only the first N queries of the workload (small-batch measurements)")
     ap.add_argument("--partition-only", type=int, default=0, metavar="C",
                     help="only time partition assignment of 1M x 128 rows against C centroids (fp32 matrix-core tile) and exit")
     return ap.parse_args()
@@ -171,6 +174,9 @@ def run_workload(args, workload, torch, want_cpu):
     top_k = 10
     t0 = time.time()
     data, queries = make_data(workload, num, nq)
+    if args.queries:
+        nq = min(nq, args.queries)
+        queries = np.ascontiguousarray(queries[:nq])
     gen_s = time.time() - t0
 
     d_data = capi.DeviceArray.from_numpy(data)
@@ -471,6 +477,35 @@ def main():
                 res["%s; %s" % (kind, name)] = {"lane_operations": ops, "ms": ms, "G_lane_operations_per_s": ops / ms / 1e6}
                 del table
         print(json.dumps({"kernel": "atomic_probe_kernel", "compute_units": info["compute_units"], "modes": res}))
+        return
+
+    if args.gather_calibration:
+        import numpy as np
+        out = capi.DeviceArray(4, np.float32)
+        res = {}
+        # (label, row bytes, row stride, rows per wave-wide step, table rows)
+        for label, row_bytes, stride, rps, rows in (("512-byte rows (128 dims), 8 lanes a row, 16 rows in flight per wavefront", 512, 512, 8, 1 << 20),
+                                                    ("3840-byte rows (960 dims), 32 lanes a row, 8 rows in flight per wavefront", 3840, 3840, 2, 1 << 20),
+                                                    ("3840-byte rows (960 dims), 64 lanes a row, 8 rows in flight per wavefront", 3840, 3840, 1, 1 << 20),
+                                                    ("3840-byte rows 4096 bytes apart, 32 lanes a row, 8 rows in flight per wavefront", 3840, 4096, 2, 1 << 20),
+                                                    ("3840-byte rows 3968 bytes apart, 32 lanes a row, 8 rows in flight per wavefront", 3840, 3968, 2, 1 << 20),
+                                                    ("4096-byte rows (1024 dims), 32 lanes a row, 8 rows in flight per wavefront", 4096, 4096, 2, 1 << 20),
+                                                    ("2048-byte rows (512 dims), 32 lanes a row, 8 rows in flight per wavefront", 2048, 2048, 2, 1 << 20)):
+            table = capi.DeviceArray.full(rows * stride // 4, 0x3F800000, np.uint32)
+            for waves_per_simd in (1, 2, 4, 8):
+                waves = info["compute_units"] * 4 * waves_per_simd           # all resident at once: that many wavefronts per SIMD
+                rows_per_wave = max(64, (4 << 30) // row_bytes // waves // 64 * 64)   # about 4 GiB per launch
+                probes.gather_probe(table, rows, row_bytes, stride, waves, rows_per_wave, rps, out)
+                e0, e1 = capi.Event(), capi.Event()
+                e0.record()
+                for _ in range(args.steps):
+                    probes.gather_probe(table, rows, row_bytes, stride, waves, rows_per_wave, rps, out)
+                e1.record()
+                ms = e0.elapsed_ms(e1) / args.steps
+                nbytes = waves * rows_per_wave * row_bytes
+                res["%s; %d wavefronts" % (label, waves)] = {"bytes": nbytes, "ms": ms, "GBps": nbytes / ms / 1e6, "frac_of_8TBps": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+            del table
+        print(json.dumps({"kernel": "gather_probe_kernel", "compute_units": info["compute_units"], "modes": res}))
         return
 
     if args.partition_only:

@@ -29,3 +29,8 @@ def valu_probe(mode, rounds, out, stream=None):
 def atomic_probe(mode, table, slots, rounds, out, stream=None):
     capi.check(lib().glide_probe_atomic(C.c_int(mode), capi._ptr(table), C.c_uint32(slots), C.c_uint32(rounds), capi._ptr(out), C.c_void_p(stream)),
                "glide_probe_atomic")
+
+
+def gather_probe(table, row_count, row_bytes, row_stride_bytes, waves, rows_per_wave, rows_per_step, out, stream=None):
+    capi.check(lib().glide_probe_gather(capi._ptr(table), C.c_uint32(row_count), C.c_uint32(row_bytes), C.c_uint32(row_stride_bytes), C.c_uint32(waves), C.c_uint32(rows_per_wave),
+                                        C.c_int(rows_per_step), capi._ptr(out), C.c_void_p(stream)), "glide_probe_gather")

@@ -39,19 +39,44 @@ inline size_t beam_lds_bytes(uint32_t degree) {
 inline size_t beam_stage_bytes(uint32_t beam) { return beam > 256 ? (2 * 512 + 4) * sizeof(uint32_t) : 0; }
 
 __device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
+// The same point in a wavefront that shares its workgroup with others (TEAM): a workgroup barrier would wait for them.
+// LDS instructions of one wavefront execute in program order; what is needed between a store and a dependent load of
+// another lane is that the compiler keeps that order, which a wavefront-scope fence does.
+template <bool TEAM>
+__device__ __forceinline__ void wave_sync_in() {
+    if constexpr (TEAM) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    } else {
+        __syncthreads();
+    }
+}
 
-// Distances from `ref` to `count` listed rows, RowShape<DIMV>::ROWS rows per step (one per lane group), U steps in
-// flight.  id_of(idx) -> row id of list entry idx; out(idx, dist) is called by one lane per scored row.
-template <int DIMV, class IdFn, class OutFn>
-__device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float* data, uint32_t dim, int metric,
-                                           uint32_t first, uint32_t count, int lane, IdFn id_of, OutFn out) {
+// Where score_list reads the reference row from: registers (one copy per wavefront) ...
+template <int DIMV>
+struct RefInRegs {
+    const RowRegs<DIMV>& r;
+    __device__ __forceinline__ float4 chunk(int c, int) const { return r.v[c]; }
+};
+// ... or LDS, laid out as the loads of one lane group would hold it (chunk c of lane t at [c * LPR + t]): the wavefronts
+// of a team share one copy and keep their registers for rows in flight.  The two lane groups of a wide row read the same
+// addresses (a broadcast), adjacent lanes adjacent 16-byte words: no bank conflicts.
+template <int DIMV>
+struct RefInLds {
+    const float4* q;
+    __device__ __forceinline__ float4 chunk(int c, int t) const { return q[c * RowShape<DIMV>::LPR + t]; }
+};
+
+// Distances from a reference row to `count` listed rows, RowShape<DIMV>::ROWS rows per step (one per lane group), U steps
+// in flight.  id_of(idx) -> row id of list entry idx; out(idx, dist) is called by one lane per scored row.  A team of
+// `members` wavefronts splits the list in runs of ROWS * U entries, member `member` taking every members-th run; the sum
+// of a row is formed in the same order whoever forms it.
+template <int DIMV, int U, class Ref, class IdFn, class OutFn>
+__device__ __forceinline__ void score_share(const Ref ref, const float* data, uint32_t dim, int metric, uint32_t first, uint32_t count,
+                                            int lane, uint32_t member, uint32_t members, IdFn id_of, OutFn out) {
     using Shape = RowShape<DIMV>;
     const int g = Shape::row_of_lane(lane), t = Shape::lane_in_row(lane);
-    // Steps in flight.  Rows of more than 512 dims are 2-4 KB each and a step holds only two of them: with one step in
-    // flight a wavefront had 8 KB on its way, too little to cover the memory latency when a launch has about one
-    // wavefront per SIMD (1 000 queries); four steps took the 960-dim beam-512 search from 16.8 to 13.2 ms.
-    constexpr int U = DIMV == 1 ? 2 : (DIMV == 2 ? 2 : (DIMV == 4 ? 2 : 4));
-    for (uint32_t base = first; base < count; base += Shape::ROWS * U) {
+    for (uint32_t base = first + member * Shape::ROWS * U; base < count; base += Shape::ROWS * U * members) {
         RowRegs<DIMV> rows[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -62,14 +87,29 @@ __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const uint32_t idx = base + Shape::ROWS * u + g;
-            const float d = finish_distance(row_sum<DIMV>(partial_sqdist<DIMV>(ref, rows[u])), metric);
+            float acc = 0.f;
+#pragma unroll
+            for (int c = 0; c < Shape::NV; c++) acc = sqdist4(ref.chunk(c, t), rows[u].v[c], acc);
+            const float d = finish_distance(row_sum<DIMV>(acc), metric);
             if (t == 0 && idx < count) out(idx, d);
         }
     }
 }
 
-template <int MAX_CAND, int MAX_BEAM, int DIMV>
+template <int DIMV, class IdFn, class OutFn>
+__device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float* data, uint32_t dim, int metric,
+                                           uint32_t first, uint32_t count, int lane, IdFn id_of, OutFn out) {
+    // Steps in flight.  Rows of more than 512 dims are 2-4 KB each and a step holds only two of them: with one step in
+    // flight a wavefront had 8 KB on its way, too little to cover the memory latency when a launch has about one
+    // wavefront per SIMD (1 000 queries); four steps took the 960-dim beam-512 search from 16.8 to 13.2 ms.
+    constexpr int U = DIMV == 8 ? 4 : 2;
+    score_share<DIMV, U>(RefInRegs<DIMV>{ref}, data, dim, metric, first, count, lane, 0u, 1u, id_of, out);
+}
+
+// TEAM: the beam's wavefront is one of several in its workgroup (the others only score rows, see search_team_kernel).
+template <int MAX_CAND, int MAX_BEAM, int DIMV, bool TEAM = false>
 struct Beam {
+    static __device__ __forceinline__ void wave_sync() { wave_sync_in<TEAM>(); }
     static constexpr int NB = MAX_BEAM / 64;
     static constexpr int NC = MAX_CAND / 64;
     static constexpr int NC32 = MAX_CAND / 32;  // items per lane in the reference's 32-lane layout
@@ -100,11 +140,34 @@ struct Beam {
         wave_sync();
     }
 
+    // One pass of the main loop up to the next expansion's candidate list (what `run` does between two score phases).
+    // Returns false when the search is over; otherwise `nv` rows wait to be scored.
+    __device__ __forceinline__ bool step_to_list(uint32_t& iter, bool& terminate, const uint32_t* graph, uint32_t self_id, uint32_t& nv) {
+        absorb(iter == 0);
+        cnt.iterations++;
+        const bool reset_now = ((iter + 1) % p.reset_interval) == 0;
+        if (reset_now) {
+            hash_clear(hash, p.hash_bit, lane);
+            wave_sync();
+        }
+        if (iter + 1 == p.max_iterations) return false;
+        const uint32_t parent = select_parent();
+        if (parent == kInvalid) terminate = true;
+        if (reset_now) {
+            restore_hash();
+            wave_sync();
+        }
+        if (terminate && iter >= p.min_iterations) return false;
+        nv = expand_list(parent, graph, self_id, kInvalid);
+        iter++;
+        return true;
+    }
+
     // Expansion of `parent` (reference compute_distance / get_init / result_init second half):
     // every neighbour not yet in the visited set becomes a candidate; `exclude_insert` is never inserted,
     // `exclude_score` is inserted and kept as a candidate id but gets distance FLT_MAX.
-    __device__ __forceinline__ void expand(uint32_t parent, const uint32_t* graph, const float* data,
-                                           uint32_t exclude_insert, uint32_t exclude_score) {
+    // First half: the candidate slots and the list of slots to score (returns its length).
+    __device__ __forceinline__ uint32_t expand_list(uint32_t parent, const uint32_t* graph, uint32_t exclude_insert, uint32_t exclude_score) {
         uint32_t nv = 0;
         if (parent != kInvalid) cnt.graph_rows++;
 #pragma unroll
@@ -124,6 +187,12 @@ struct Beam {
         wave_sync();
         cnt.rows_scored += nv;
         last_scored = nv;
+        return nv;
+    }
+
+    __device__ __forceinline__ void expand(uint32_t parent, const uint32_t* graph, const float* data,
+                                           uint32_t exclude_insert, uint32_t exclude_score) {
+        const uint32_t nv = expand_list(parent, graph, exclude_insert, exclude_score);
         BeamLds<MAX_CAND>* l = lds;
         score_list<DIMV>(q, data, p.dim, p.metric, 0, nv, lane,
                          [l](uint32_t idx) { return l->cand_id[l->vlist[idx]]; },
@@ -431,7 +500,7 @@ struct Beam {
 
 // Nearest centroid by the reference's sort network (search_kernel.cuh:259-268, distance.cuh:29-60):
 // strided load, blocked store, element 0 is the winner.  One wavefront; scratch holds `centroid_num` pairs.
-template <int MAX_CENTROID, int DIMV>
+template <int MAX_CENTROID, int DIMV, bool TEAM = false>
 __device__ __forceinline__ uint32_t nearest_centroid(const RowRegs<DIMV>& q, const float* centroids, uint32_t centroid_num,
                                                      uint32_t dim, int metric, float* cent_dist, int lane) {
     using Shape = RowShape<DIMV>;
@@ -447,7 +516,7 @@ __device__ __forceinline__ uint32_t nearest_centroid(const RowRegs<DIMV>& q, con
         const float d = finish_distance(row_sum<DIMV>(partial_sqdist<DIMV>(q, row)), metric);
         if (t == 0 && c < centroid_num) cent_dist[c] = d;
     }
-    wave_sync();
+    wave_sync_in<TEAM>();
     constexpr int NR = WaveNet<MAX_CENTROID>::NR;
     constexpr int N32 = MAX_CENTROID / 32;
     float k[NR];
@@ -461,7 +530,7 @@ __device__ __forceinline__ uint32_t nearest_centroid(const RowRegs<DIMV>& q, con
         v[r] = ok ? j : kInvalid;
     }
     WaveNet<MAX_CENTROID>::sort(k, v, lane);
-    wave_sync();
+    wave_sync_in<TEAM>();
     return read_lane(v[0], 0);
 }
 

@@ -70,6 +70,43 @@ __global__ __launch_bounds__(256) void atomic_probe_kernel(unsigned long long* t
     if (sum == 0xFFFFFFF1u) out[0] = sum;   // keeps the results alive; practically never taken
 }
 
+// The rate at which rows scattered over a table can be read, whatever is done with them: every wavefront walks its own
+// pseudo-random sequence of rows and reads each one with 16-byte loads of adjacent lanes, `rows_in_flight` rows requested
+// before the first is consumed (ROWS_PER_STEP rows per wave-wide step: a row takes 64 / ROWS_PER_STEP lanes and as many
+// loads per lane as its length needs).  This is the memory side of a graph search's scoring loop without its distances,
+// its sorting networks and its dependent graph-row fetch.
+template <int ROWS_PER_STEP, int STEPS>
+__global__ __launch_bounds__(64) void gather_probe_kernel(const float4* table, uint32_t row_count, uint32_t quads_per_row, uint32_t stride_quads,
+                                                          uint32_t rows_per_wave, float* out) {
+    constexpr int LPR = 64 / ROWS_PER_STEP;
+    const int lane = threadIdx.x, g = lane / LPR, t = lane % LPR;
+    uint32_t x = (blockIdx.x * 64 + 1) * 0x9E3779B1u + 0x7F4A7C15u;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (uint32_t r = 0; r < rows_per_wave; r += ROWS_PER_STEP * STEPS) {
+        uint32_t row[STEPS];
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            x ^= x << 13;
+            x ^= x >> 17;
+            x ^= x << 5;
+            row[s] = static_cast<uint32_t>((static_cast<unsigned long long>((x + g * 0x85EBCA6Bu) * 0xC2B2AE35u) * row_count) >> 32);
+        }
+        for (uint32_t c = t; c < quads_per_row; c += LPR) {
+            float4 v[STEPS];
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) v[s] = table[static_cast<size_t>(row[s]) * stride_quads + c];
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                acc.x += v[s].x;
+                acc.y += v[s].y;
+                acc.z += v[s].z;
+                acc.w += v[s].w;
+            }
+        }
+    }
+    if (acc.x + acc.y + acc.z + acc.w == 12345.678f) out[0] = acc.x;   // keeps the loads alive; practically never taken
+}
+
 }  // namespace glide
 
 using namespace glide;
@@ -101,6 +138,22 @@ int glide_probe_atomic(int mode, unsigned long long* table, uint32_t slots, uint
         case 1: hipLaunchKernelGGL(atomic_probe_kernel<1>, dim3(2048), dim3(256), 0, as_stream(stream), table, slots - 1, rounds, out); break;
         case 2: hipLaunchKernelGGL(atomic_probe_kernel<2>, dim3(2048), dim3(256), 0, as_stream(stream), table, slots - 1, rounds, out); break;
         default: hipLaunchKernelGGL(atomic_probe_kernel<3>, dim3(2048), dim3(256), 0, as_stream(stream), table, slots - 1, rounds, out); break;
+    }
+    return launch_status();
+}
+
+int glide_probe_gather(const void* table, uint32_t row_count, uint32_t row_bytes, uint32_t row_stride_bytes, uint32_t waves, uint32_t rows_per_wave, int rows_per_step,
+                       float* out, void* stream) {
+    if (!table || !out || row_count == 0 || row_bytes == 0 || row_bytes % 16 != 0 || row_stride_bytes % 16 != 0 || row_stride_bytes < row_bytes || waves == 0)
+        return GLIDE_ERR_BAD_ARGUMENT;
+    const float4* t = static_cast<const float4*>(table);
+    const uint32_t quads = row_bytes / 16, stride = row_stride_bytes / 16;
+    hipStream_t s = as_stream(stream);
+    switch (rows_per_step) {
+        case 8: hipLaunchKernelGGL((gather_probe_kernel<8, 2>), dim3(waves), dim3(64), 0, s, t, row_count, quads, stride, rows_per_wave, out); break;
+        case 2: hipLaunchKernelGGL((gather_probe_kernel<2, 4>), dim3(waves), dim3(64), 0, s, t, row_count, quads, stride, rows_per_wave, out); break;
+        case 1: hipLaunchKernelGGL((gather_probe_kernel<1, 8>), dim3(waves), dim3(64), 0, s, t, row_count, quads, stride, rows_per_wave, out); break;
+        default: return GLIDE_ERR_UNSUPPORTED;
     }
     return launch_status();
 }

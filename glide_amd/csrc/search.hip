@@ -18,14 +18,14 @@ struct SearchArgs {
     BeamParams p;
 };
 
-template <int DIMV>
+template <int DIMV, bool TEAM = false>
 __device__ __forceinline__ uint32_t pick_centroid(uint32_t max_centroid, const RowRegs<DIMV>& q, const float* centroids,
                                                   uint32_t centroid_num, uint32_t dim, int metric, float* scratch, int lane) {
     switch (max_centroid) {  // bucket chosen like reference kernel_config.cuh:161-171
-        case 32: return nearest_centroid<32, DIMV>(q, centroids, centroid_num, dim, metric, scratch, lane);
-        case 64: return nearest_centroid<64, DIMV>(q, centroids, centroid_num, dim, metric, scratch, lane);
-        case 128: return nearest_centroid<128, DIMV>(q, centroids, centroid_num, dim, metric, scratch, lane);
-        default: return nearest_centroid<256, DIMV>(q, centroids, centroid_num, dim, metric, scratch, lane);
+        case 32: return nearest_centroid<32, DIMV, TEAM>(q, centroids, centroid_num, dim, metric, scratch, lane);
+        case 64: return nearest_centroid<64, DIMV, TEAM>(q, centroids, centroid_num, dim, metric, scratch, lane);
+        case 128: return nearest_centroid<128, DIMV, TEAM>(q, centroids, centroid_num, dim, metric, scratch, lane);
+        default: return nearest_centroid<256, DIMV, TEAM>(q, centroids, centroid_num, dim, metric, scratch, lane);
     }
 }
 
@@ -68,6 +68,86 @@ __global__ __launch_bounds__(64) void search_kernel(SearchArgs a) {
 template <int MAX_CAND, int MAX_BEAM, int DIMV>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(5, 5))) void search_kernel_dense(SearchArgs a) {
     search_body<MAX_CAND, MAX_BEAM, DIMV>(a);
+}
+
+// Small batches of long rows (more than 256 dims): a team of kTeam wavefronts per query.  Wavefront 0 owns the search
+// (beam, visited set, sorting networks) exactly as in search_kernel; between two of its passes every wavefront of the
+// team scores a share of the expansion's candidate rows.  One wavefront can keep only a few 2-4 KB rows in flight in its
+// registers, and a search is a chain of dependent expansions: while the batch leaves SIMDs idle, a team gives a query
+// kTeam times the bytes on their way and an expansion takes one or two memory round trips instead of six (64 queries of
+// 960 dims: 1.9 times the throughput at beams up to 256, 1.3 times above).  Once a batch fills the chip on its own
+// (about two wavefronts per SIMD) the row gathers run at the rate the memory system sustains for scattered rows either
+// way and the team only adds its barriers, so larger batches keep one wavefront per query.  The query row sits in LDS
+// once per team (RefInLds) so that the registers hold rows in flight; every distance is summed in the order
+// search_kernel sums it, so results are identical.
+constexpr int kTeam = 4;
+
+template <int DIMV>
+struct TeamShape {
+    static constexpr int U = DIMV == 8 ? 2 : 4;   // row steps in flight per wavefront: 64 row registers either way
+    static constexpr size_t query_bytes = sizeof(float4) * RowShape<DIMV>::NV * RowShape<DIMV>::LPR;
+};
+
+template <int MAX_CAND, int MAX_BEAM, int DIMV>
+__global__ __launch_bounds__(64 * kTeam) void search_team_kernel(SearchArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    using Shape = RowShape<DIMV>;
+    auto* lds = reinterpret_cast<BeamLds<MAX_CAND>*>(smem);
+    float* cent = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>));
+    float4* qlds = reinterpret_cast<float4*>(cent + round_up32(a.centroid_num));
+    uint32_t* ctl = reinterpret_cast<uint32_t*>(qlds + Shape::NV * Shape::LPR);   // [0] rows to score, [1] search over
+    uint32_t* hash = ctl + 4;
+    const uint32_t wave = threadIdx.x >> 6;
+    const int lane = lane_id();
+    for (uint32_t qid = blockIdx.x; qid < a.query_num; qid += gridDim.x) {
+        Beam<MAX_CAND, MAX_BEAM, DIMV, true> b;
+        uint32_t iter = 0;
+        bool terminate = false;
+        if (wave == 0) {
+            b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
+            if (Shape::row_of_lane(lane) == 0) {
+#pragma unroll
+                for (int c = 0; c < Shape::NV; c++) qlds[c * Shape::LPR + Shape::lane_in_row(lane)] = b.q.v[c];
+            }
+            const uint32_t c0 = pick_centroid<DIMV, true>(a.max_centroid, b.q, a.centroids, a.centroid_num, a.p.dim, a.p.metric, cent, lane);
+            const uint32_t nv = b.expand_list(a.start_points[c0], a.graph, kInvalid, kInvalid);   // result_init: the entry node itself is never scored
+            if (lane == 0) {
+                ctl[0] = nv;
+                ctl[1] = 0;
+            }
+        }
+        __syncthreads();
+        while (true) {
+            const uint32_t nv = ctl[0];
+            score_share<DIMV, TeamShape<DIMV>::U>(RefInLds<DIMV>{qlds}, a.data, a.p.dim, a.p.metric, 0, nv, lane, wave, kTeam,
+                                                  [lds](uint32_t idx) { return lds->cand_id[lds->vlist[idx]]; },
+                                                  [lds](uint32_t idx, float d) { lds->cand_dist[lds->vlist[idx]] = d; });
+            __syncthreads();
+            if (wave == 0) {
+                uint32_t next = 0;
+                const bool more = b.step_to_list(iter, terminate, a.graph, kInvalid, next);
+                if (lane == 0) {
+                    ctl[0] = next;
+                    ctl[1] = more ? 0u : 1u;
+                }
+            }
+            __syncthreads();
+            if (ctl[1] != 0) break;
+        }
+        if (wave == 0) {
+            constexpr int NB = MAX_BEAM / 64;
+#pragma unroll
+            for (int r = 0; r < NB; r++) {
+                const uint32_t e = NB * lane + r;
+                if (e < a.top_k) {
+                    a.result_ids[static_cast<size_t>(qid) * a.top_k + e] = b.bv[r] & kClean;
+                    a.result_dists[static_cast<size_t>(qid) * a.top_k + e] = b.bk[r];
+                }
+            }
+            b.flush_counters(a.counters);
+        }
+        __syncthreads();   // the next query reuses the LDS
+    }
 }
 
 // ---- large path: one staged partition at a time ---------------------------------------------------------------
@@ -417,6 +497,18 @@ search_fn pick_dim(uint32_t dim) {
     if (dim <= 512) return search_kernel<MAX_CAND, MAX_BEAM, 4>;
     return search_kernel<MAX_CAND, MAX_BEAM, 8>;
 }
+template <int MAX_CAND, int MAX_BEAM>
+search_fn pick_team_dim(uint32_t dim) {
+    if (dim <= 512) return search_team_kernel<MAX_CAND, MAX_BEAM, 4>;
+    return search_team_kernel<MAX_CAND, MAX_BEAM, 8>;
+}
+template <int MAX_CAND>
+search_fn pick_team_beam(uint32_t beam, uint32_t dim) {
+    if (beam <= 64) return pick_team_dim<MAX_CAND, 64>(dim);
+    if (beam <= 128) return pick_team_dim<MAX_CAND, 128>(dim);
+    if (beam <= 256) return pick_team_dim<MAX_CAND, 256>(dim);
+    return pick_team_dim<MAX_CAND, 512>(dim);
+}
 template <int MAX_CAND>
 search_fn pick_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_dim<MAX_CAND, 64>(dim);
@@ -430,6 +522,12 @@ search_fn pick_beam(uint32_t beam, uint32_t dim) {
 // hardware dispatch runs one full round and a thin, latency-bound tail.  Equal rounds are faster: the grid is the
 // batch divided by the number of rounds and every wavefront loops over its share.  Larger beams are bound by the
 // sorting networks and keep one workgroup per query.
+size_t simd_count() {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 0;
+    return static_cast<size_t>(cus) * 4;
+}
+
 uint32_t balanced_grid(uint32_t items, uint32_t beam, size_t lds_bytes) {
     if (beam > 64) return items;
     int dev = 0, cus = 0;
@@ -488,11 +586,16 @@ int launch_search(const float* data, uint32_t num, uint32_t dim, const uint32_t*
     a.p.min_iterations = min_iterations;
     a.p.metric = metric;
 
-    search_fn fn = graph_degree <= 64 ? pick_beam<64>(beam, dim) : graph_degree <= 128 ? pick_beam<128>(beam, dim) : pick_beam<256>(beam, dim);
+    const bool team = dim > 256 && static_cast<size_t>(query_num) * kTeam <= 2 * simd_count();   // see search_team_kernel
+    search_fn fn;
+    if (team) fn = graph_degree <= 64 ? pick_team_beam<64>(beam, dim) : graph_degree <= 128 ? pick_team_beam<128>(beam, dim) : pick_team_beam<256>(beam, dim);
+    else fn = graph_degree <= 64 ? pick_beam<64>(beam, dim) : graph_degree <= 128 ? pick_beam<128>(beam, dim) : pick_beam<256>(beam, dim);
     const size_t lds_bytes = beam_lds_bytes(graph_degree) + round_up32(centroid_num) * sizeof(float) +
-                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam) +
+                             (team ? (dim <= 512 ? TeamShape<4>::query_bytes : TeamShape<8>::query_bytes) + 16 : 0);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-    hipLaunchKernelGGL(fn, dim3(balanced_grid(query_num, beam, lds_bytes)), dim3(64), lds_bytes, as_stream(stream), a);
+    if (team) hipLaunchKernelGGL(fn, dim3(query_num), dim3(64 * kTeam), lds_bytes, as_stream(stream), a);
+    else hipLaunchKernelGGL(fn, dim3(balanced_grid(query_num, beam, lds_bytes)), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
 }
 }  // namespace

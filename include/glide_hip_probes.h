@@ -25,6 +25,14 @@ int glide_probe_valu(int mode, uint32_t rounds, float *out, void *stream);
 int glide_probe_atomic(int mode, unsigned long long *table, uint32_t slots, uint32_t rounds, uint32_t *out,
                        void *stream);
 
+/* `waves` wavefronts, each reading `rows_per_wave` pseudo-random rows of `row_bytes` (a multiple of 16) out of a table of
+ * `row_count` rows that start `row_stride_bytes` apart, with 16-byte loads of adjacent lanes and nothing else to do: the rate at which scattered rows can be
+ * fetched at all, the yardstick for the search kernels' row gathers.  rows_per_step 8 / 2 / 1: a row is read by 8 / 32 /
+ * 64 lanes (the search kernels' shapes for 128-dim and 960-dim rows; one row per wavefront), with 16 / 8 / 8 rows requested
+ * before the first is consumed.  out: one float. */
+int glide_probe_gather(const void *table, uint32_t row_count, uint32_t row_bytes, uint32_t row_stride_bytes, uint32_t waves,
+                       uint32_t rows_per_wave, int rows_per_step, float *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -159,6 +159,12 @@ int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, uint32_t di
 /* The same build with the host loop as the reference ships it (length passed as end, partition-local id compared with the
  * global row index, no merge across sub-lists before truncation; nn_descent.cuh:1276-1283, :1117, :1376-1402).  Only
  * for quoting what the shipped executable would score; nothing is held to it. */
+/* go_nnd_build_ex from start lists the caller brings (reorder_num x extended degree partition-local ids, a row's sub-lists
+ * one after the other, negative = empty) instead of the shuffled ones of init_random_graph (nn_descent.cuh:1003-1038):
+ * lets a test start both sides of a comparison from one random graph. */
+int go_nnd_build_from(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                      const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
+                      float termination_threshold, const int32_t *start_lists, int32_t *knn_graph, int threads);
 int go_nnd_build_shipped(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
                          const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
                          float termination_threshold, uint32_t seed, int32_t *knn_graph, int threads);

@@ -268,7 +268,8 @@ struct Shipped {
     uint32_t last_join;         // out: the iteration of this partition's last join
 };
 void build_partition(const float *data, const float *norms_in, uint32_t n, uint32_t dim, uint32_t K, uint32_t iterations, uint32_t seed,
-                     int32_t *out /* n x K local ids */, uint32_t row_index_base, float termination_limit, Shipped *shipped = nullptr) {
+                     int32_t *out /* n x K local ids */, uint32_t row_index_base, float termination_limit, Shipped *shipped = nullptr,
+                     const int32_t *start_lists = nullptr /* n x W local ids, sub-list after sub-list, replacing the shuffled lists */) {
     Partition P;
     P.n = n;
     P.dim = dim;
@@ -288,8 +289,13 @@ void build_partition(const float *data, const float *norms_in, uint32_t n, uint3
     for (auto &l : P.locks) omp_init_lock(&l);
     Bloom bloom(n, ext_inter / kSeg);
 
-    // init_random_graph nn_descent.cuh:1003-1038 (local ids)
-    for (uint32_t sub = 0; sub < P.num_sub; sub++) {
+    // init_random_graph nn_descent.cuh:1003-1038 (local ids); a caller that brings its own start lists (a test that wants
+    // both sides of a comparison to start from the same random graph) replaces the shuffle, nothing else
+    if (start_lists) {
+        for (size_t i = 0; i < static_cast<size_t>(n) * P.W; i++)
+            P.lists[i] = (start_lists[i] >= 0 && static_cast<uint32_t>(start_lists[i]) < n) ? start_lists[i] : INT_MAX;
+    }
+    for (uint32_t sub = 0; sub < P.num_sub && !start_lists; sub++) {
         uint32_t m = std::max<uint32_t>(n / P.num_sub, 1);
         std::vector<int> seq(m);
         std::iota(seq.begin(), seq.end(), 0);
@@ -429,6 +435,38 @@ extern "C" int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, 
         const float limit = termination_threshold * static_cast<float>(reorder_num) * static_cast<float>(dim) / 100.0f;
         build_partition(half.data() + static_cast<size_t>(start) * dim, norms.data() + start, len, dim, knn_degree, iterations, seed,
                         knn_graph + static_cast<size_t>(start) * knn_degree, start, limit);
+    }
+    return 0;
+}
+
+// go_nnd_build_ex from given start lists: reorder_num x extended degree partition-local ids, a row's sub-lists one after
+// the other (sub-list s holds ids with id % num_sub == s), negative = empty slot.
+extern "C" int go_nnd_build_from(const float *reorder_data, uint32_t reorder_num, uint32_t dim, const uint32_t *segment_starts,
+                                 const uint32_t *segment_lengths, uint32_t segment_num, uint32_t knn_degree, uint32_t iterations,
+                                 float termination_threshold, const int32_t *start_lists, int32_t *knn_graph, int threads) {
+#ifdef _OPENMP
+    if (threads > 0) omp_set_num_threads(threads);
+#endif
+    if (knn_degree == 0 || knn_degree > 128 || !start_lists) return -1;
+    const uint32_t W = go_nnd_extended_degree(knn_degree);
+    std::vector<float> half(static_cast<size_t>(reorder_num) * dim), norms(reorder_num);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < static_cast<int64_t>(reorder_num); i++) {
+        float acc = 0.0f;
+        for (uint32_t t = 0; t < dim; t++) {
+            float v = reorder_data[static_cast<size_t>(i) * dim + t];
+            acc += v * v;
+            half[static_cast<size_t>(i) * dim + t] = round_half(v);
+        }
+        norms[i] = acc;
+    }
+    for (uint32_t s = 0; s < segment_num; s++) {
+        uint32_t start = segment_starts[s], len = segment_lengths[s];
+        if (len == 0) continue;
+        if (start + len > reorder_num) return -2;
+        const float limit = termination_threshold * static_cast<float>(reorder_num) * static_cast<float>(dim) / 100.0f;
+        build_partition(half.data() + static_cast<size_t>(start) * dim, norms.data() + start, len, dim, knn_degree, iterations, 0,
+                        knn_graph + static_cast<size_t>(start) * knn_degree, start, limit, nullptr, start_lists + static_cast<size_t>(start) * W);
     }
     return 0;
 }

@@ -321,6 +321,21 @@ def nnd_build(reorder_data, seg_start, seg_len, knn_degree, iterations, seed=0, 
     return out
 
 
+def nnd_build_from(reorder_data, seg_start, seg_len, knn_degree, iterations, start_lists, threads=0, termination_threshold=0.0):
+    """nnd_build from the caller's start lists: (rows, extended degree) int32 partition-local ids, a row's sub-lists one
+    after the other (sub-list s holds ids with id % num_sub == s), negative = empty slot."""
+    reorder_data, seg_start, seg_len = _f32(reorder_data), _u32(seg_start), _u32(seg_len)
+    start_lists = np.ascontiguousarray(start_lists, dtype=np.int32)
+    assert start_lists.shape == (reorder_data.shape[0], nnd_extended_degree(knn_degree))
+    out = np.empty((reorder_data.shape[0], knn_degree), dtype=np.int32)
+    rc = lib().go_nnd_build_from(_p(reorder_data), u32(reorder_data.shape[0]), u32(reorder_data.shape[1]), _p(seg_start), _p(seg_len),
+                                 u32(seg_start.size), u32(knn_degree), u32(iterations), C.c_float(termination_threshold),
+                                 start_lists.ctypes.data_as(C.c_void_p), _p(out), C.c_int(threads))
+    if rc != 0:
+        raise ValueError("oracle nnd_build_from failed: %d" % rc)
+    return out
+
+
 def bruteforce_knn(data, queries, k, metric=EUCLIDEAN, exclude_self=False, threads=0):
     data, queries = _f32(data), _f32(queries)
     ids = np.empty((queries.shape[0], k), dtype=np.uint32)

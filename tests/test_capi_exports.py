@@ -26,7 +26,7 @@ def test_every_header_has_its_library():
     """include/ holds the product boundary and the measurement yardsticks, nothing else; each is exported by its own library."""
     assert sorted(os.listdir(os.path.join(ROOT, "include"))) == ["glide_hip.h", "glide_hip_probes.h"]
     names = declared_symbols("glide_hip_probes.h", "glide_probe_")
-    assert names == ["glide_probe_atomic", "glide_probe_copy_bytes", "glide_probe_valu"]
+    assert names == ["glide_probe_atomic", "glide_probe_copy_bytes", "glide_probe_gather", "glide_probe_valu"]
     path = os.path.join(ROOT, "glide_amd", "libglide_probes.so")
     assert os.path.exists(path), "build the libraries first (make -C glide_amd/csrc)"
     probes = ctypes.CDLL(path)

@@ -286,3 +286,99 @@ def test_large_pipeline_cli_uint8(tmp_path):
     for key in ("rdata", "map", "starts", "lengths", "centroids", "graph", "sp"):
         assert np.array_equal(a[key], b[key]), key
     assert a["recall"] == b["recall"] and b["recall"] >= 0.9
+
+
+def test_large_merged_pipeline_cli_256_partitions(tmp_path):
+    """The large-build configuration at its real partition count: 1M rows of the benchmark's mixture in 256 locality
+    partitions with a boundary segment, every stage staged from pinned host memory by the large_* executables
+    (large_preprocess -> large_knn -> large_build with merge and refinement -> large_search on the merged index;
+    glide_large_impl.cuh:109-166,347-507).  At this size the stages are held to what does not depend on the size -- the
+    partition files are a partition, kNN lists are local and distinct and find the true neighbours, graph rows are valid,
+    distinct and cross partitions only where boundary copies link them, the run repeats bit for bit -- and the search of
+    the finished files is compared with the oracle's search of the same files, query by query."""
+    from glide_amd import datasets as D
+    from oracle import oracle as O
+    n, dim, c, nq, bf = 1_000_000, 128, 256, 500, 1.002      # the boundary factor of the 50M run (256 centroids split every component)
+    data, queries = D.gmm_clipped(n, dim, seed=1234), D.gmm_clipped(nq, dim, seed=4321)
+    truth, _ = O.bruteforce_knn(data, queries, 100)
+    f = lambda name: str(tmp_path / name)
+    D.write_fbin(f("base.fbin"), data)
+    D.write_fbin(f("query.fbin"), queries)
+    D.write_fbin(f("truth"), truth.astype(np.uint32))
+    pre, knn_file, graph_base, result = f("pre"), f("knn"), f("graph"), f("result.csv")
+    print("files written", flush=True)
+
+    run(os.path.join(BIN, "large_preprocess"), f("base.fbin"), pre, result, c, 0.01, "Euclidean", bf)
+    centroids = D.read_fbin(pre + ".centroid")
+    starts, lengths = D.read_segment(pre + ".segment")
+    mp = D.read_vector(pre + ".map")
+    rdata = D.read_fbin(pre + ".reorder")
+    copies = int(lengths[c])
+    print("partitioned:", copies, "boundary copies, largest partition", int(lengths[:c].max()), flush=True)
+    assert centroids.shape == (c, dim) and starts.size == c + 1 and lengths[:c].sum() == n and starts[c] == n and 0 < copies < n // 2
+    assert np.array_equal(starts[:c + 1], np.concatenate([[0], np.cumsum(lengths[:c])]).astype(np.uint32))
+    assert rdata.shape == (n + copies, dim) and mp.size == n + copies
+    assert np.array_equal(rdata, data[mp]) and np.array_equal(np.sort(mp[:n]), np.arange(n, dtype=np.uint32))
+    assert np.unique(mp[n:]).size == copies
+    # membership and boundary flag of a sample against a float64 arg-min over the 256 centroids
+    pick = np.random.default_rng(3).choice(n, 5000, replace=False)
+    d = np.sqrt(((data[pick, None, :].astype(np.float64) - centroids[None].astype(np.float64)) ** 2).sum(-1))
+    order = np.argsort(d, axis=1)
+    d0, d1 = d[np.arange(pick.size), order[:, 0]], d[np.arange(pick.size), order[:, 1]]
+    owner = np.empty(n, np.int64)
+    owner[mp[:n]] = np.searchsorted(starts[1:c + 1], np.arange(n), side="right")
+    boundary = np.zeros(n, bool)
+    boundary[mp[n:]] = True
+    clear = d1 - d0 > 1e-4 * d1
+    assert clear.mean() > 0.98 and np.array_equal(owner[pick][clear], order[:, 0][clear])
+    sure = np.abs(d1 / d0 - bf) > 1e-4
+    assert np.array_equal(boundary[pick][sure], (d1 / d0 <= bf)[sure])
+
+    run(os.path.join(BIN, "large_knn"), pre, knn_file, result, 32)
+    knn = D.read_fbin(knn_file, np.uint32)
+    assert knn.shape == (n + copies, 32)
+    recalls = []
+    for i, (s, l) in enumerate(zip(starts.tolist(), lengths.tolist())):
+        rows = knn[s:s + l].astype(np.int64)
+        assert rows.max() < l
+        if l > 64:      # a partition smaller than a list fills up with repeats, as in the reference (nn_descent.cuh:1392-1398)
+            assert not (rows == np.arange(l)[:, None]).any(), "a kNN list holds its own node"
+            assert (np.diff(np.sort(rows, axis=1), axis=1) > 0).all(), "a kNN list holds an id twice"
+        if i % 32 == 0 and l > 200:
+            gt, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + 100], 32, exclude_self=True)
+            recalls.append(D.recall(knn[s:s + 100], gt, 32))
+    print("kNN recall@32 of sampled partitions", np.round(recalls, 4), flush=True)
+    assert np.mean(recalls) >= 0.95
+
+    out = run(os.path.join(BIN, "large_build"), pre, knn_file, graph_base, result, "Euclidean", 32, 32, 1.05, 64, 128)
+    assert "index build time" in out
+    graph = D.read_fbin(graph_base + ".graph", np.uint32)
+    sp = D.read_vector(graph_base + ".sp")
+    INV = 0xFFFFFFFF
+    assert graph.shape == (n, 32) and sp.size == c + 1
+    valid = graph != INV
+    assert graph[valid].max() < n and valid.any(axis=1).all()
+    srt = np.sort(graph.astype(np.int64), axis=1)
+    assert not ((np.diff(srt, axis=1) == 0) & (srt[:, 1:] != INV)).any(), "a row names a point twice"
+    part_of = np.searchsorted(starts[1:c + 1], np.arange(n), side="right")
+    cross = (part_of[np.where(valid, graph, 0)] != part_of[:, None]) & valid
+    print("edges that cross partitions: %.4f of all" % (cross.sum() / valid.sum()), flush=True)
+    assert cross.any()
+    # a second build from the same files gives the same graph
+    run(os.path.join(BIN, "large_build"), pre, knn_file, f("graph_again"), f("result_again.csv"), "Euclidean", 32, 32, 1.05, 64, 128)
+    assert np.array_equal(D.read_fbin(f("graph_again") + ".graph", np.uint32), graph)
+
+    entries = (starts[:c] + sp[:c]).astype(np.uint32)
+    for beam in (32, 128):
+        out = run(os.path.join(BIN, "large_search"), pre, f("query.fbin"), f("truth"), graph_base, result, "Euclidean", 10, beam, 2, 1.1)
+        recall = float(out.split("total_recall:")[1].split()[0])
+        assert "index upload time" in out
+        # the merged search ranks all 256 centroids for its entry point (the small path's bucket rule would look at 64)
+        qd = np.sqrt(((queries[:, None, :].astype(np.float64) - centroids[None].astype(np.float64)) ** 2).sum(-1))
+        e_ids = np.empty((nq, 10), np.uint32)
+        for cid in np.unique(qd.argmin(1)):
+            mine = np.nonzero(qd.argmin(1) == cid)[0]
+            ids, _, _ = O.search(rdata[:n], graph, centroids[cid:cid + 1], entries[cid:cid + 1], queries[mine], 10, **O.search_params(beam, 32))
+            e_ids[mine] = np.where(ids < n, mp[np.minimum(ids, n - 1)], ids)
+        print("beam", beam, "recall@10", recall, flush=True)
+        assert abs(D.recall(e_ids, truth, 10) - recall) < 1e-6

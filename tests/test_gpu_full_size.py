@@ -1,5 +1,6 @@
-"""The 1M-point configurations at their real size: 16 partitions, graph degree 32, 10 000 queries, top-10 (128 dims
-Euclidean on the benchmark's mixture and on data of low intrinsic dimension, 96 dims cosine on the normalised mixture).
+"""The 1M-point configurations at their real size: 16 partitions, top-10; graph degree 32 and 10 000 queries for 128 dims
+Euclidean on the benchmark's mixture and on data of low intrinsic dimension and for 96 dims cosine on the normalised
+mixture; graph degree 64, kNN degree 64 and 1 000 queries for the 960-dim configuration.
 
 What the CPU oracle can finish in seconds at this size is compared bit for bit (the sub-graph rows of the first
 points, searches of a sample of the queries on the finished index); everything else is held to properties that do
@@ -14,10 +15,13 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-N, C, D, K, NQ = 1_000_000, 16, 32, 32, 10_000
-# name: generator, dims, metric, integer-valued (sums exact in fp32)
-CONFIGS = {"lowdim_integer": ("lowdim_integer", 128, 0, True), "gmm_clipped": ("gmm_clipped", 128, 0, True),
-           "gmm_normalized_cosine": ("gmm_normalized", 96, 1, False)}
+N, C = 1_000_000, 16
+# name: generator, dims, metric, integer-valued (sums exact in fp32), graph degree, kNN degree, queries, graph recall@32 expected
+CONFIGS = {"lowdim_integer": ("lowdim_integer", 128, 0, True, 32, 32, 10_000, 0.95), "gmm_clipped": ("gmm_clipped", 128, 0, True, 32, 32, 10_000, 0.95),
+           "gmm_normalized_cosine": ("gmm_normalized", 96, 1, False, 32, 32, 10_000, 0.95),
+           # the termination limit of NN-descent grows with the row length (nn_descent.cuh:1280), so the 960-dim build stops
+           # after fewer rounds: recall@32 0.89 here, on the GPU and in the CPU restatement alike
+           "beta_scaled_960": ("beta_scaled", 960, 0, False, 64, 64, 1_000, 0.85)}
 INVALID = 0xFFFFFFFF
 
 
@@ -34,7 +38,7 @@ def hip():
 def world(hip, request):
     """Data, queries, the partitioning, the kNN graph and the finished index, all made on the GPU."""
     from glide_amd import datasets as Ds, index as G
-    gen_name, DIM, metric, exact = CONFIGS[request.param]
+    gen_name, DIM, metric, exact, D, K, NQ, knn_recall = CONFIGS[request.param]
     gen = getattr(Ds, gen_name)
     data, queries = gen(N, DIM, seed=1234), gen(NQ, DIM, seed=4321)
     print("data", request.param, data.shape, flush=True)
@@ -51,7 +55,7 @@ def world(hip, request):
     assert np.array_equal(d_cent2.numpy(), centroids) and np.array_equal(d_map2.numpy(), h_map) and np.array_equal(h_len2, h_len)
     for d in (d_re2, d_map2, d_cent2):
         d.free()
-    w = dict(kind=request.param, metric=metric, exact=exact, data=data, queries=queries, rdata=rdata, map=h_map, seg_start=h_start.copy(), seg_len=h_len.copy(), centroids=centroids, knn=knn)
+    w = dict(kind=request.param, metric=metric, exact=exact, D=D, K=K, NQ=NQ, knn_recall=knn_recall, data=data, queries=queries, rdata=rdata, map=h_map, seg_start=h_start.copy(), seg_len=h_len.copy(), centroids=centroids, knn=knn)
 
     # the sub-graph stage alone, for the comparison with the oracle
     index = G.GLIDE(D, d_data, d_cent, metric)
@@ -83,7 +87,7 @@ def world(hip, request):
 def _truth(world):
     if "truth" not in world:
         from oracle import oracle as O
-        world["truth"] = O.bruteforce_knn(world["data"], world["queries"][:1000], 10, world["metric"])[0].astype(np.uint32)
+        world["truth"] = O.bruteforce_knn(world["data"], world["queries"][:min(1000, world["NQ"])], 10, world["metric"])[0].astype(np.uint32)
     return world["truth"]
 
 
@@ -124,6 +128,7 @@ def test_partition_assignment_on_a_sample(world):
 
 
 def test_knn_graph_lists(world):
+    D, K, NQ = world["D"], world["K"], world["NQ"]
     from glide_amd import datasets as Ds
     from oracle import oracle as O
     knn, seg_start, seg_len, rdata = world["knn"], world["seg_start"], world["seg_len"], world["rdata"]
@@ -135,18 +140,19 @@ def test_knn_graph_lists(world):
         assert not (rows == np.arange(l)[:, None]).any(), "no list holds its own node"
         srt = np.sort(rows, axis=1)
         assert (np.diff(srt, axis=1) > 0).all(), "no list holds an id twice"
-        m = 100
-        ids, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + m], K + 1, world["metric"])
-        truth = np.array([[x for x in ids[i].tolist() if x != i][:K] for i in range(m)], dtype=np.uint32)
-        recalls.append(Ds.recall(knn[s:s + m], truth, K))
-    print("graph recall@%d per partition" % K, np.round(recalls, 4), flush=True)
-    assert np.mean(recalls) >= 0.95
+        m, ke = 100, 32
+        ids, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + m], ke + 1, world["metric"])
+        truth = np.array([[x for x in ids[i].tolist() if x != i][:ke] for i in range(m)], dtype=np.uint32)
+        recalls.append(Ds.recall(knn[s:s + m, :ke], truth, ke))
+    print("graph recall@32 per partition", np.round(recalls, 4), flush=True)
+    assert np.mean(recalls) >= world["knn_recall"]
 
 
 def test_subgraph_rows_equal_the_oracle(world):
     """The first points in partition order, searched over their whole partition of the full-size kNN graph."""
+    D, K, NQ = world["D"], world["K"], world["NQ"]
     from oracle import oracle as O
-    m = 1500
+    m = 1500 if world["data"].shape[1] <= 128 else 400
     sp = O.search_params(64, K)
     assert (sp["beam"], sp["max_iterations"], sp["hash_bit"]) == (world["sp_b"].beam, world["sp_b"].max_iterations, world["sp_b"].hash_bit)
     expect = np.full((N, D), INVALID, dtype=np.uint32)
@@ -160,6 +166,7 @@ def test_subgraph_rows_equal_the_oracle(world):
 
 
 def test_graph_rows_and_determinism(world):
+    D, K, NQ = world["D"], world["K"], world["NQ"]
     g = world["graph"]
     assert g.shape == (N, D)
     assert np.array_equal(g, world["graph_again"]), "two builds from one kNN graph differ"
@@ -179,6 +186,7 @@ def test_graph_rows_and_determinism(world):
 
 @pytest.mark.parametrize("beam", [32, 256])
 def test_search_sample_equals_the_oracle(hip, world, beam):
+    D, K, NQ = world["D"], world["K"], world["NQ"]
     from glide_amd import index as G
     from oracle import oracle as O
     sp = G.make_search_parameter(beam, D, 10)
@@ -198,6 +206,7 @@ def test_search_sample_equals_the_oracle(hip, world, beam):
 
 @pytest.mark.parametrize("beam", [32, 64])
 def test_search_properties(hip, world, beam):
+    D, K, NQ = world["D"], world["K"], world["NQ"]
     from glide_amd import datasets as Ds, index as G
     data, queries = world["data"], world["queries"]
     sp = G.make_search_parameter(beam, D, 10)
@@ -215,8 +224,8 @@ def test_search_properties(hip, world, beam):
     perm = np.random.default_rng(1).permutation(NQ)
     p_ids, p_dists = world["index"].search(sp, hip.DeviceArray.from_numpy(np.ascontiguousarray(queries[perm])))
     assert np.array_equal(p_ids, ids[perm]) and np.array_equal(p_dists, dists[perm])
-    h_ids, _ = world["index"].search(sp, hip.DeviceArray.from_numpy(np.ascontiguousarray(queries[:3333])))
-    assert np.array_equal(h_ids, ids[:3333])
+    h_ids, _ = world["index"].search(sp, hip.DeviceArray.from_numpy(np.ascontiguousarray(queries[:NQ // 3])))
+    assert np.array_equal(h_ids, ids[:NQ // 3])
     # recall against exact neighbours of the first 1000 queries (the oracle's brute force)
     gt = _truth(world)
     r = Ds.recall(ids[:gt.shape[0]], gt, 10)
@@ -233,6 +242,7 @@ def test_recall_is_bounded_by_what_the_entry_point_reaches(hip, world):
     beam must come close to it -- which is what makes the low recall of the mixtures a property of the algorithm on that
     data (components the kNN graph does not connect) and not of this implementation."""
     from glide_amd import datasets as Ds, index as G
+    D, K, NQ = world["D"], world["K"], world["NQ"]
     gt = _truth(world)
     m = gt.shape[0]
     bound, reach_frac, per_query = Ds.reachable_recall_bound(world["graph"], world["centroids"], world["start_points"], world["queries"][:m], gt,
@@ -250,5 +260,7 @@ def test_recall_is_bounded_by_what_the_entry_point_reaches(hip, world):
     assert recalls[512] <= bound and bound - recalls[512] <= 0.05
     if world["kind"] == "lowdim_integer":
         assert bound >= 0.999 and recalls[32] >= 0.96
+    elif world["kind"] == "beta_scaled_960":
+        assert bound >= 0.99 and recalls[512] >= 0.95, "the 960-dim configuration reaches the metric's operating point inside the reference's beam range"
     else:
         assert bound < 0.5, "the mixtures' components are not connected: no beam can reach recall@10 0.95"

@@ -98,6 +98,37 @@ def test_search_degree64_dim960(hip):
         assert np.array_equal(gids, eids) and np.array_equal(gdists, edists)
 
 
+@pytest.mark.parametrize("dim,deg", [(960, 64), (384, 32), (1024, 160)])
+def test_long_rows_small_and_large_batches_agree(hip, dim, deg):
+    """Rows of more than 256 dims are searched by a team of four wavefronts per query while the batch is small and by one
+    wavefront per query once it fills the chip; both forms must give the oracle's ids, distances and counters (integer
+    data: exact sums, frequent ties), for every beam bucket including the two-half merge above 256, and a query must get
+    the same answer whichever batch it arrives in."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(dim + deg)
+    n, big = 2500, 2100                         # 2100 queries: beyond two wavefronts per SIMD for a team of four
+    data = np.rint(rng.random((n, dim)) * 9).astype(np.float32)
+    queries = np.rint(rng.random((big, dim)) * 9).astype(np.float32)
+    graph = rng.integers(0, n, (n, deg)).astype(np.uint32)
+    graph[rng.random(graph.shape) < 0.05] = 0xFFFFFFFF
+    centroids = data[:5].copy()
+    start_points = rng.integers(0, n, 5).astype(np.uint32)
+    for beam in (32, 128, 256, 448):
+        sp = O.search_params(beam, deg)
+        print("dim", dim, "degree", deg, "beam", beam, flush=True)
+        small = run_gpu_search(hip, data, graph, centroids, start_points, queries[:70], 10, sp, counters=True)
+        eids, edists, est = O.search(data, graph, centroids, start_points, queries[:70], 10, **sp)
+        assert np.array_equal(small[0], eids) and np.array_equal(small[1], edists)
+        assert small[2] == [est["iterations"], est["rows_scored"], est["graph_rows"]]
+        large = run_gpu_search(hip, data, graph, centroids, start_points, queries, 10, sp, counters=True)
+        assert np.array_equal(large[0][:70], eids) and np.array_equal(large[1][:70], edists)
+        pick = rng.choice(big, 40, replace=False)
+        eids, edists, _ = O.search(data, graph, centroids, start_points, queries[pick], 10, **sp)
+        assert np.array_equal(large[0][pick], eids) and np.array_equal(large[1][pick], edists)
+        one = run_gpu_search(hip, data, graph, centroids, start_points, queries[pick[:1]], 10, sp)
+        assert np.array_equal(one[0], eids[:1]) and np.array_equal(one[1], edists[:1])
+
+
 @pytest.mark.parametrize("deg", [160, 256])
 def test_search_degree_above_128(hip, deg):
     """Degrees above 128 sort the candidate list as two half-wave networks, beams above 256 merge the same way

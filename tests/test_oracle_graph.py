@@ -393,3 +393,36 @@ def test_hash_reset_every_iteration_returns_no_id_twice():
         # a forgotten node is farther than everything the beam held when it left, so scoring it again changes nothing
         assert np.array_equal(ids, base[0]) and np.array_equal(dists, base[1])
         assert st["rows_scored"] > base[2]["rows_scored"] and st["iterations"] == base[2]["iterations"]
+
+
+def test_nnd_oracle_from_given_start_lists():
+    """The build from caller-supplied start lists (what pairs the GPU and CPU sides of the pipeline comparison) is the
+    same algorithm: same recall as the build from shuffled lists, valid structure, and it does depend on the lists."""
+    from glide_amd.datasets import recall
+    rng = np.random.default_rng(15)
+    data = lowdim_data(4000, 128, seed=9)
+    seg_start, seg_len = np.array([0, 2500], np.uint32), np.array([2500, 1500], np.uint32)
+    for k in (32, 64):
+        width = O.nnd_extended_degree(k)
+        num_sub = width // 32
+
+        def lists(seed):
+            r = np.random.default_rng(seed)
+            out = np.empty((4000, width), np.int32)
+            for s, l in ((0, 2500), (2500, 1500)):
+                for sub in range(num_sub):       # sub-list `sub` holds ids congruent to sub modulo num_sub
+                    pool = np.arange(sub, l, num_sub)
+                    out[s:s + l, sub * 32:(sub + 1) * 32] = r.choice(pool, (l, 32))
+            return out
+
+        a = O.nnd_build_from(data, seg_start, seg_len, k, 8, lists(1)).astype(np.uint32)
+        b = O.nnd_build_from(data, seg_start, seg_len, k, 8, lists(1)).astype(np.uint32)
+        c = O.nnd_build_from(data, seg_start, seg_len, k, 8, lists(2)).astype(np.uint32)
+        ref = O.nnd_build(data, seg_start, seg_len, k, 8).astype(np.uint32)
+        for s, l in ((0, 2500), (2500, 1500)):
+            assert (a[s:s + l] < l).all()
+            gt, _ = O.bruteforce_knn(data[s:s + l], data[s:s + 200], 32, exclude_self=True)
+            ra, rr = recall(a[s:s + 200, :32], gt, 32), recall(ref[s:s + 200, :32], gt, 32)
+            assert abs(ra - rr) <= 0.01 and ra >= 0.9, (k, ra, rr)
+        assert not np.array_equal(a, c)
+        assert (np.sort(a, 1) == np.sort(b, 1)).mean() > 0.99      # the same lists in, the same graph out up to thread timing
