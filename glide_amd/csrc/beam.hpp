@@ -381,11 +381,33 @@ struct Beam {
         return true;
     }
 
+    // True when no candidate of the latest expansion is below the last beam entry.  The beam then stays as it is: the
+    // half-cleaner of the merge replaces an entry only by a strictly smaller candidate, entry `beam - 1 - k` by the k-th
+    // smallest, so if even the smallest candidate is not below the largest entry nothing is replaced, and the candidate
+    // sort in front of it only feeds that test.  Half of all iterations of a wide beam end here (the further a search has
+    // come, the fewer neighbours of its frontier are nearer than the worst entry it holds), for one LDS read per lane.
+    __device__ __forceinline__ bool nothing_enters() {
+        static_assert(MAX_CAND == 64, "one candidate slot per lane");
+        // The beam is ascending, so its last entry is the largest key of the lane that holds it among that lane's entries
+        // below `beam` (written as a maximum: a chain of selects between the registers becomes a run-time index, which
+        // moves the beam out of the registers).  Keys are not negative.
+        const uint32_t last = p.beam - 1;
+        float mine = bk[0];
+#pragma unroll
+        for (int r = 1; r < NB; r++) mine = fmaxf(mine, NB * lane + r <= static_cast<int>(last) ? bk[r] : 0.f);
+        const float tail = read_lane(mine, static_cast<int>(last / NB));
+        const float ck = static_cast<uint32_t>(lane) < p.degree ? lds->cand_dist[lane] : FLT_MAX;
+        return ballot(ck < tail) == 0;
+    }
+
     // reference update_result_buffer: sort the candidates, then fold them into the beam
     __device__ __forceinline__ void absorb(bool first) {
         // No row scored: every candidate distance is FLT_MAX, the sort would not move anything (equal keys are never
         // exchanged) and no candidate can displace a beam entry, so the beam stays as it is.
         if (!first && last_scored == 0) return;
+        if constexpr (MAX_CAND == 64) {
+            if (!first && nothing_enters()) return;
+        }
         if constexpr (MAX_CAND > 128) sort_candidates_two();
         else sort_candidates_one();
         if (first) {
