@@ -34,6 +34,7 @@ NAMED_BEAMS = {"cfg1": (32, 64, 128, 256)}  # the medium configuration names its
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "search_kernels_hbm_traffic.md")
 VALU_PROFILE = os.path.join(ROOT, "profiles", "build_refine_kernels_counters.md")
 NND_PROFILE = os.path.join(ROOT, "profiles", "nnd_kernels_cfg1_rounds_and_counters.md")
+GATHER_PROFILE = os.path.join(ROOT, "profiles", "gather_probe_scattered_rows.md")
 NND_OFFERS_NOTE = ("nnd_offers: distinct offers the merge steps found in the offer tables, all rounds.  nnd_offers_declined_by_threshold: offers a "
                    "join did not send because their distance was not below the threshold their target announced (the distance of its 64th "
                    "best offer of the round before, announced only by nodes whose table was five eighths full).  Nothing depends on the order "
@@ -55,6 +56,22 @@ def measured_traffic(workload, beam):
             return dict(bytes=float(m.group(3)) * 1024 * float(m.group(5)) + float(m.group(4)) * 1024 * float(m.group(6)),
                         source="profiles/" + os.path.basename(TRAFFIC_PROFILE))
     return None
+
+
+def scattered_row_ceiling(row_bytes):
+    """The rate (GB/s) at which this GPU reads rows of `row_bytes` scattered over a table when a kernel does nothing else,
+    from the committed summary of `--gather-calibration` (the probe kernel's best figure over its residencies): what the
+    search kernels' row gathers can reach at all, below the 8 TB/s the HBM stacks are specified at.  The table rows are
+    `| row bytes | best GB/s | fraction of 8 TB/s |`; the row of the nearest length at or above `row_bytes` is used."""
+    try:
+        text = open(GATHER_PROFILE).read()
+    except OSError:
+        return None
+    rows = sorted((int(m.group(1)), float(m.group(2))) for m in re.finditer(r"^\|\s*(\d+)\s*\|\s*([\d.]+)\s*\|\s*[\d.]+\s*\|\s*$", text, re.M))
+    for length, gbs in rows:
+        if length >= row_bytes:
+            return dict(row_bytes=length, GBps=gbs, source="profiles/" + os.path.basename(GATHER_PROFILE))
+    return dict(row_bytes=rows[-1][0], GBps=rows[-1][1], source="profiles/" + os.path.basename(GATHER_PROFILE)) if rows else None
 
 
 def measured_stage(stage, workload):
@@ -369,6 +386,11 @@ def run_workload(args, workload, torch, want_cpu):
                                                1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8),
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )
+    # what scattered rows of this length can be read at on this GPU at all (a probe kernel that only gathers rows)
+    ceiling = scattered_row_ceiling(dim * 4)
+    if ceiling:
+        out["roofline"].update(scattered_row_ceiling_GBps=ceiling["GBps"], scattered_row_ceiling_frac=ceiling["GBps"] / HBM_PEAK_GBS,
+                               frac_of_scattered_row_ceiling=achieved / ceiling["GBps"], scattered_row_ceiling_source=ceiling["source"])
 
     if want_cpu == "full":
         out["cpu_baseline"] = cpu_baseline(data, queries, graph, d_cent.numpy(), index.d_start_points.numpy(), sp, top_k, gt, metric)
@@ -489,6 +511,7 @@ def main():
                                                     ("3840-byte rows (960 dims), 64 lanes a row, 8 rows in flight per wavefront", 3840, 3840, 1, 1 << 20),
                                                     ("3840-byte rows 4096 bytes apart, 32 lanes a row, 8 rows in flight per wavefront", 3840, 4096, 2, 1 << 20),
                                                     ("3840-byte rows 3968 bytes apart, 32 lanes a row, 8 rows in flight per wavefront", 3840, 3968, 2, 1 << 20),
+                                                    ("384-byte rows (96 dims), 8 lanes a row, 16 rows in flight per wavefront", 384, 384, 8, 1 << 20),
                                                     ("4096-byte rows (1024 dims), 32 lanes a row, 8 rows in flight per wavefront", 4096, 4096, 2, 1 << 20),
                                                     ("2048-byte rows (512 dims), 32 lanes a row, 8 rows in flight per wavefront", 2048, 2048, 2, 1 << 20)):
             table = capi.DeviceArray.full(rows * stride // 4, 0x3F800000, np.uint32)
@@ -610,14 +633,17 @@ def headline(args, workload, details, device):
         "stage_fracs": {k: r3(v.get("frac")) for k, v in r["stage_rooflines"].items()},
         "roofline": {"bound": roof["bound"], "achieved": round(roof["achieved"], 1), "peak": roof["peak"], "unit": roof["unit"],
                      "frac": r3(roof["frac"]), "traffic": roof["traffic"], "kernel": roof["kernel"],
-                     "algorithmic_bytes_per_launch": roof["algorithmic_bytes_per_launch"]},
+                     "algorithmic_bytes_per_launch": roof["algorithmic_bytes_per_launch"],
+                     "scattered_row_ceiling_frac": r3(roof.get("scattered_row_ceiling_frac")),
+                     "frac_of_scattered_row_ceiling": r3(roof.get("frac_of_scattered_row_ceiling"))},
     }
     if "cpu_baseline" in r:
         c = r["cpu_baseline"]
         line["cpu_baseline"] = {k: (r3(c[k]) if isinstance(c[k], float) else c[k])
                                 for k in ("value", "unit", "cores", "kind", "sample", "recall_at_10", "nnd_points_per_sec", "bruteforce_qps") if k in c}
     # where the metric's operating point exists in this run: workload -> beam, QPS, recall, roofline fraction
-    line["recall_target_met_on"] = {n: dict(beam=d["beam"], qps=round(d["qps"]), recall_at_10=r3(d["recall_at_10"]), roofline_frac=r3(d["roofline"]["frac"]))
+    line["recall_target_met_on"] = {n: dict(beam=d["beam"], qps=round(d["qps"]), recall_at_10=r3(d["recall_at_10"]), roofline_frac=r3(d["roofline"]["frac"]),
+                                            frac_of_scattered_row_ceiling=r3(d["roofline"].get("frac_of_scattered_row_ceiling")))
                                     for n, d in details.items() if d["recall_target_met"]}
     line["other_workloads"] = {n: dict(beam=d["beam"], qps=round(d["qps"]), recall_at_10=r3(d["recall_at_10"]), bound=r3(d["reachable_recall_bound"]),
                                        roofline_frac=r3(d["roofline"]["frac"]), build_sec=r3(d["build_sec"]))
