@@ -11,7 +11,7 @@ recall@10 of the whole beam sweep (32 ... 512, the reference's range) are measur
 shapes on navigable data and the other single-GPU configurations cfg0, cfg2, cfg3: build stages, graph recall, beam
 sweep, stage rooflines, roofline of the timed search kernel, the CPU restatement's recall and throughput at the same
 beam) and ends with ONE compact line of a few KB: the benchmark record of cfg1 (`headline()` below).  The same details
-go to gpurun_out/bench_full.json.  cfg4 (50M rows staged from pinned host memory) has a run of its own: --workload cfg4.
+go to the file --details-file names.  cfg4 (50M rows staged from pinned host memory) has a run of its own: --workload cfg4.
 
 Everything on the product path goes through libglide_hip.so.  torch is imported only to compute exact ground
 truth on the GPU (a checker); the CPU oracle is used only for the cpu_baseline legs.
@@ -138,6 +138,8 @@ def parse():
                     help="only run the scattered-atomics kernel (yardstick for the NN-descent offers and slot reservations) and exit")
     ap.add_argument("--gather-calibration", action="store_true",
                     help="only run the scattered-row read kernel (yardstick for the search kernels' row gathers) and exit")
+    ap.add_argument("--details-file", default=os.path.join("gpurun_out", "bench_full.json"),
+                    help="where the per-workload details are written as one JSON file (relative to the repository root)")
     ap.add_argument("--queries", type=int, default=0, help="use only the first N queries of the workload (small-batch measurements)")
     ap.add_argument("--partition-only", type=int, default=0, metavar="C",
                     help="only time partition assignment of 1M x 128 rows against C centroids (fp32 matrix-core tile) and exit")
@@ -585,12 +587,13 @@ def main():
             details[name]["wall_sec"] = time.time() - t0
             emit_detail(name, details[name])
     try:    # the whole record in one file, for whoever wants more than the stdout lines
-        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-        with open(os.path.join(ROOT, "gpurun_out", "bench_full.json"), "w") as f:
+        path = os.path.join(ROOT, args.details_file)
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
             json.dump(details, f, default=float, indent=1)
     except OSError:
         pass
-    print(json.dumps(headline(args, args.workload, details, info["name"]), default=float), flush=True)
+    print(json.dumps(headline(args, args.workload, details, info["name"], args.details_file), default=float), flush=True)
 
 
 DETAIL_KEYS = ("workload", "build_sec", "build_stages", "graph_recall_at_32", "graph_recall_at_32_global", "empty_slots_fraction", "beam",
@@ -603,7 +606,7 @@ def emit_detail(name, res):
     print(json.dumps({"bench_detail": name, **{k: res[k] for k in DETAIL_KEYS if k in res}}, default=float), flush=True)
 
 
-def headline(args, workload, details, device):
+def headline(args, workload, details, device, details_file="the details file"):
     """The record's last stdout line: the fields of the benchmark contract for the headline workload, short enough (a few KB)
     that a consumer keeping only the tail of stdout still holds all of it.  `value` is the throughput of the timed steps;
     `metric` says what that is: the metric's operating point (the smallest beam with recall@10 >= 0.95) where the sweep
@@ -648,7 +651,7 @@ def headline(args, workload, details, device):
     line["other_workloads"] = {n: dict(beam=d["beam"], qps=round(d["qps"]), recall_at_10=r3(d["recall_at_10"]), bound=r3(d["reachable_recall_bound"]),
                                        roofline_frac=r3(d["roofline"]["frac"]), build_sec=r3(d["build_sec"]))
                                for n, d in details.items() if n != workload}
-    line["details"] = "one 'bench_detail' JSON line per workload earlier on stdout; gpurun_out/bench_full.json"
+    line["details"] = "one 'bench_detail' JSON line per workload earlier on stdout; " + details_file
     return line
 
 
