@@ -135,12 +135,12 @@ __device__ __forceinline__ uint32_t hash_insert(uint32_t* table, uint32_t bitlen
 // Narrow rows use narrow groups: the cross-lane sum then needs log2(LPR) steps instead of 5 and one instruction
 // serves 64/LPR rows.  DIMV selects the shape by row length (dim <= 128*DIMV):
 //   DIMV 1: 8 lanes x 4 loads (8 rows per wavefront)    DIMV 2: 16 lanes x 4 loads (4 rows)
-//   DIMV 4: 32 lanes x 4 loads (2 rows)                 DIMV 8: 32 lanes x 8 loads (2 rows)
+//   DIMV 4: 32 lanes x 4 loads (2 rows)                 DIMV 8 / 16: 32 lanes x 8 / 16 loads (2 rows)
 template <int DIMV>
 struct RowShape {
-    static_assert(DIMV == 1 || DIMV == 2 || DIMV == 4 || DIMV == 8, "row shape");
+    static_assert(DIMV == 1 || DIMV == 2 || DIMV == 4 || DIMV == 8 || DIMV == 16, "row shape");
     static constexpr int LPR = DIMV == 1 ? 8 : (DIMV == 2 ? 16 : 32);
-    static constexpr int NV = DIMV == 8 ? 8 : 4;
+    static constexpr int NV = DIMV == 16 ? 16 : (DIMV == 8 ? 8 : 4);
     static constexpr int ROWS = 64 / LPR;
     static __device__ __forceinline__ int lane_in_row(int lane) { return lane & (LPR - 1); }
     static __device__ __forceinline__ int row_of_lane(int lane) { return lane / LPR; }

@@ -294,7 +294,8 @@ build_fn pick_build_dim(uint32_t dim) {
     if (dim <= 128) return build_kernel<MAX_CAND, MAX_BEAM, 1>;
     if (dim <= 256) return build_kernel<MAX_CAND, MAX_BEAM, 2>;
     if (dim <= 512) return build_kernel<MAX_CAND, MAX_BEAM, 4>;
-    return build_kernel<MAX_CAND, MAX_BEAM, 8>;
+    if (dim <= 1024) return build_kernel<MAX_CAND, MAX_BEAM, 8>;
+    return build_kernel<MAX_CAND, MAX_BEAM, 16>;
 }
 template <int MAX_CAND>
 build_fn pick_build_beam(uint32_t beam, uint32_t dim) {
@@ -308,7 +309,8 @@ refine_fn pick_refine_dim(uint32_t dim) {
     if (dim <= 128) return refine_kernel<MAX_CAND, MAX_BEAM, 1>;
     if (dim <= 256) return refine_kernel<MAX_CAND, MAX_BEAM, 2>;
     if (dim <= 512) return refine_kernel<MAX_CAND, MAX_BEAM, 4>;
-    return refine_kernel<MAX_CAND, MAX_BEAM, 8>;
+    if (dim <= 1024) return refine_kernel<MAX_CAND, MAX_BEAM, 8>;
+    return refine_kernel<MAX_CAND, MAX_BEAM, 16>;
 }
 template <int MAX_CAND>
 refine_fn pick_refine_beam(uint32_t beam, uint32_t dim) {
@@ -334,7 +336,7 @@ size_t prune_lds_bytes_refine(uint32_t beam, uint32_t degree) {
 int check_beam_sizes(uint32_t degree, uint32_t graph_degree, uint32_t beam, uint32_t dim, uint32_t hash_bit, int metric) {
     if (degree == 0 || graph_degree == 0 || beam == 0 || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
-    if (degree > kMaxDegree || graph_degree > kMaxDegree || beam > 512 || dim % 4 != 0 || dim > 1024 || hash_bit < 1 || hash_bit > 13)
+    if (degree > kMaxDegree || graph_degree > kMaxDegree || beam > 512 || dim % 4 != 0 || dim > 2048 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     return GLIDE_OK;
 }
