@@ -70,3 +70,20 @@ def test_reachable_recall_bound_on_a_hand_built_graph():
     # query 0: {1} of {0, 1} -> 0.5; query 1: 4 reachable (edge back), 3 on the other chain -> 0.5; query 2: both -> 1.0
     assert abs(bound - (0.5 + 0.5 + 1.0) / 3) < 1e-12
     assert abs(frac - (3 / 8 + 4 / 8) / 2) < 1e-12
+
+
+def test_committed_profile_tables_are_readable():
+    """bench.py takes measured traffic, stage counters and the scattered-row ceiling from the committed profile summaries;
+    a change of their table format must not silently turn those fields into nulls."""
+    for workload, beam in (("cfg1", 256), ("cfg1-navigable", 32), ("cfg3", 448)):
+        t = bench.measured_traffic(workload, beam)
+        assert t and t["bytes"] > 1e9, (workload, beam)
+    for workload in ("cfg1", "cfg1-navigable", "cfg0", "cfg2", "cfg3"):
+        for stage in ("subgraph+boundary", "refine"):
+            m = bench.measured_stage(stage, workload)
+            assert m and m[0] > 1e9 and m[2] > 100 and m[3] > 1.5, (stage, workload)
+    assert bench.measured_knn("cfg1") and bench.measured_knn_bytes("cfg1") > 1e11
+    for row_bytes, low, high in ((384, 0.8, 0.9), (512, 0.8, 0.9), (3840, 0.7, 0.82)):
+        c = bench.scattered_row_ceiling(row_bytes)
+        assert c and low < c["GBps"] / bench.HBM_PEAK_GBS < high, row_bytes
+    assert bench.scattered_row_ceiling(8192)["row_bytes"] == 4096      # beyond the table: its longest row
