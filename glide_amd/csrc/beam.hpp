@@ -32,11 +32,11 @@ struct BeamLds {  // per-wave LDS (the hash table follows, 1 << hash_bit words)
 };
 
 // Host-side sizes of the dynamic LDS regions: the candidate lists for a degree bucket, and the staging area that the
-// two-half beam merge (beams above 256) keeps behind the hash table: 512 distances, 512 ids, two turning points.
+// beam merges of beams above 256 keep behind the hash table: 512 + 4 distances, as many ids, the turning points.
 inline size_t beam_lds_bytes(uint32_t degree) {
     return degree <= 64 ? sizeof(BeamLds<64>) : degree <= 128 ? sizeof(BeamLds<128>) : sizeof(BeamLds<256>);
 }
-inline size_t beam_stage_bytes(uint32_t beam) { return beam > 256 ? (2 * 512 + 4) * sizeof(uint32_t) : 0; }
+inline size_t beam_stage_bytes(uint32_t beam) { return beam > 256 ? (2 * (512 + 4) + 4) * sizeof(uint32_t) : 0; }
 
 __device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
 // The same point in a wavefront that shares its workgroup with others (TEAM): a workgroup barrier would wait for them.
@@ -126,6 +126,7 @@ struct Beam {
     BeamCounters cnt;
     int lane;
     uint32_t last_scored;   // rows scored by the latest expansion (wave-uniform)
+    uint32_t ranked_pause;  // beams above 256: merges left before the ranked insertion is tried again (wave-uniform)
 
     __device__ __forceinline__ void init(BeamLds<MAX_CAND>* lds_, uint32_t* hash_, const BeamParams& p_, const float* query) {
         lds = lds_;
@@ -133,8 +134,8 @@ struct Beam {
         p = p_;
         lane = lane_id();
         stage_dist = reinterpret_cast<float*>(hash_ + (size_t{1} << p_.hash_bit));
-        stage_id = reinterpret_cast<uint32_t*>(stage_dist + MAX_BEAM);
-        stage_ws = stage_id + MAX_BEAM;
+        stage_id = reinterpret_cast<uint32_t*>(stage_dist + MAX_BEAM + 4);
+        stage_ws = stage_id + MAX_BEAM + 4;
         load_row<DIMV>(q, query, p.dim, RowShape<DIMV>::lane_in_row(lane));
         hash_clear(hash, p.hash_bit, lane);
         wave_sync();
@@ -381,12 +382,13 @@ struct Beam {
         return true;
     }
 
-    // True when no candidate of the latest expansion is below the last beam entry.  The beam then stays as it is: the
-    // half-cleaner of the merge replaces an entry only by a strictly smaller candidate, entry `beam - 1 - k` by the k-th
-    // smallest, so if even the smallest candidate is not below the largest entry nothing is replaced, and the candidate
-    // sort in front of it only feeds that test.  Half of all iterations of a wide beam end here (the further a search has
-    // come, the fewer neighbours of its frontier are nearer than the worst entry it holds), for one LDS read per lane.
-    __device__ __forceinline__ bool nothing_enters() {
+    // The candidates of the latest expansion that are below the last beam entry, as a lane mask (one candidate slot per
+    // lane).  None: the beam stays as it is -- the half-cleaner of the merge replaces an entry only by a strictly smaller
+    // candidate, entry `beam - 1 - k` by the k-th smallest, so if even the smallest candidate is not below the largest
+    // entry nothing is replaced, and the candidate sort in front of it only feeds that test.  Half of all iterations of
+    // a wide beam end here (the further a search has come, the fewer neighbours of its frontier are nearer than the worst
+    // entry it holds), for one LDS read per lane.
+    __device__ __forceinline__ uint64_t entering(float& ck) {
         static_assert(MAX_CAND == 64, "one candidate slot per lane");
         // The beam is ascending, so its last entry is the largest key of the lane that holds it among that lane's entries
         // below `beam` (written as a maximum: a chain of selects between the registers becomes a run-time index, which
@@ -396,8 +398,113 @@ struct Beam {
 #pragma unroll
         for (int r = 1; r < NB; r++) mine = fmaxf(mine, NB * lane + r <= static_cast<int>(last) ? bk[r] : 0.f);
         const float tail = read_lane(mine, static_cast<int>(last / NB));
-        const float ck = static_cast<uint32_t>(lane) < p.degree ? lds->cand_dist[lane] : FLT_MAX;
-        return ballot(ck < tail) == 0;
+        ck = static_cast<uint32_t>(lane) < p.degree ? lds->cand_dist[lane] : FLT_MAX;
+        return ballot(ck < tail);
+    }
+
+    // Does the beam hold two equal keys (pads aside)?  Asked for beams above 256, where it decides whether the ranked
+    // insertion below is tried.  An entry without a distance that still names a point (the build kernels leave the point
+    // itself unscored) counts as a tie with the pads around it.
+    __device__ __forceinline__ bool beam_has_ties() const {
+        const float up = shfl_f32(bk[0], (lane + 1) & 63);   // first key of the next lane
+        bool t = false;
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t e = NB * lane + r;
+            const float next = r + 1 < NB ? bk[r + 1 < NB ? r + 1 : r] : up;
+            t |= e + 1 < p.beam && bk[r] == next && bk[r] < FLT_MAX;
+            t |= e < p.beam && !(bk[r] < FLT_MAX) && bv[r] != kInvalid;
+        }
+        return ballot(t) != 0;
+    }
+
+    // x + 1 in the lanes whose bit is set in `mask`: the carry-in of an add, so one instruction per counter
+    static __device__ __forceinline__ uint32_t add_by_mask(uint32_t x, uint64_t mask) {
+        uint32_t out;
+        uint64_t carry_out;
+        asm("v_addc_co_u32_e64 %0, %1, %2, 0, %3" : "=v"(out), "=s"(carry_out) : "v"(x), "s"(mask));
+        return out;
+    }
+
+    // Beams above 256: candidate sort + two-half merge in one step when a few candidates enter a beam and every key
+    // involved is distinct.  The reference's networks then simply produce "the smallest `beam` of beam and candidates,
+    // ascending", and that can be had without sorting anything: a beam entry moves down by the number of entering
+    // candidates below it, a candidate goes to (beam entries not above it) + (entering candidates before it).  One pass over
+    // the entering candidates (a broadcast and a compare per beam register each) gives all of these counts; the entries
+    // are stored to their places in LDS and read back in beam order.  Equal keys are where the networks' result is their
+    // own business (they never exchange equal keys, and a merge network is not stable): entries ahead of the first
+    // candidate's place never move in either scheme, so ties there do not matter; from there to the first entry that
+    // drops out every two neighbours must differ, or the step reports failure and the caller runs the networks on the
+    // untouched beam.  `em`: lanes whose candidate (`ck`) enters.  Returns true when the beam is up to date.
+    static constexpr uint32_t kRankedLimit = 24;   // more entering candidates than this: the networks are cheaper
+    __device__ __forceinline__ bool insert_ranked(uint64_t em, float ck) {
+        if (static_cast<uint32_t>(__popcll(em)) > kRankedLimit) return false;
+        const bool enter = (em >> lane) & 1;
+        const uint32_t cv = lds->cand_id[lane];
+        uint32_t shift[NB];
+#pragma unroll
+        for (int r = 0; r < NB; r++) shift[r] = 0;
+        uint32_t crank = 0, below = 0, first_place = MAX_BEAM;
+        for (uint64_t rest = em; rest != 0; rest &= rest - 1) {
+            const int j = __builtin_ctzll(rest);
+            const float cj = read_lane(ck, j);
+            uint32_t greater = 0;                               // beam entries above candidate j (wave-uniform)
+#pragma unroll
+            for (int r = 0; r < NB; r++) {
+                const uint64_t g = ballot(cj < bk[r]);
+                shift[r] = add_by_mask(shift[r], g);
+                greater += static_cast<uint32_t>(__popcll(g));
+            }
+            // candidates in (key, lane) order: j goes before this lane's candidate if its key is smaller, or equal from a lower lane
+            const uint64_t lt = ballot(cj < ck), le = ballot(cj <= ck);
+            const uint64_t lanes_above = j == 63 ? 0ull : (~0ull << (j + 1));
+            crank = add_by_mask(crank, (le & lanes_above) | (lt & ~lanes_above));
+            const uint32_t place = MAX_BEAM - greater;          // beam entries not above it (pads count as above)
+            below = lane == j ? place : below;
+            first_place = place < first_place ? place : first_place;
+        }
+        // everything to its place; places 0 .. beam are each taken exactly once (place `beam` by the first entry to drop out)
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t at = NB * lane + r + shift[r];
+            if (at <= p.beam) {
+                stage_dist[at] = bk[r];
+                stage_id[at] = bv[r];
+            }
+        }
+        if (enter) {
+            const uint32_t at = below + crank;
+            if (at <= p.beam) {
+                stage_dist[at] = ck;
+                stage_id[at] = cv;
+            }
+        }
+        wave_sync();
+        float nk[NB + 1];
+        uint32_t nv[NB + 1];
+#pragma unroll
+        for (int r = 0; r <= NB; r++) {
+            const uint32_t e = NB * lane + r;
+            nk[r] = e <= p.beam ? stage_dist[e] : FLT_MAX;
+            nv[r] = e <= p.beam ? stage_id[e] : kInvalid;
+        }
+        bool tie = false;
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t e = NB * lane + r;
+            tie |= e + 1 >= first_place && e + 1 <= p.beam && nk[r] == nk[r + 1] && !(nv[r] == kInvalid && nv[r + 1] == kInvalid);
+        }
+        const bool clean = ballot(tie) == 0;
+        if (clean) {
+#pragma unroll
+            for (int r = 0; r < NB; r++) {
+                const uint32_t e = NB * lane + r;
+                bk[r] = e < p.beam ? nk[r] : FLT_MAX;
+                bv[r] = e < p.beam ? nv[r] : kInvalid;
+            }
+        }
+        wave_sync();   // the staging area is free again
+        return clean;
     }
 
     // reference update_result_buffer: sort the candidates, then fold them into the beam
@@ -406,7 +513,23 @@ struct Beam {
         // exchanged) and no candidate can displace a beam entry, so the beam stays as it is.
         if (!first && last_scored == 0) return;
         if constexpr (MAX_CAND == 64) {
-            if (!first && nothing_enters()) return;
+            if (!first) {
+                float ck;
+                const uint64_t em = entering(ck);
+                if (em == 0) return;
+                if constexpr (MAX_BEAM > 256) {
+                    // Only worth trying on a beam without equal keys (on integer-valued rows a beam of 512 rarely is): a
+                    // failed attempt is time lost on a path that is bound by the latency of its own steps.  After a beam
+                    // with equal keys, or an attempt that failed on a candidate's key, the next 16 merges go straight to
+                    // the networks.
+                    if (ranked_pause != 0) {
+                        ranked_pause--;
+                    } else {
+                        if (!beam_has_ties() && insert_ranked(em, ck)) return;
+                        ranked_pause = 16;
+                    }
+                }
+            }
         }
         if constexpr (MAX_CAND > 128) sort_candidates_two();
         else sort_candidates_one();
@@ -418,6 +541,7 @@ struct Beam {
                 bk[r] = take ? lds->cand_dist[e] : FLT_MAX;
                 bv[r] = take ? lds->cand_id[e] : kInvalid;
             }
+            if constexpr (MAX_BEAM > 256) ranked_pause = 0;
         } else if constexpr (MAX_BEAM > 256) {
             merge_beam_two();
         } else {
