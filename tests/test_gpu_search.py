@@ -129,6 +129,37 @@ def test_long_rows_small_and_large_batches_agree(hip, dim, deg):
         assert np.array_equal(one[0], eids[:1]) and np.array_equal(one[1], edists[:1])
 
 
+@pytest.mark.parametrize("deg", [32, 64])
+def test_wide_beams_on_distinct_keys(hip, deg):
+    """Beams above 256 insert a few entering candidates by rank instead of running candidate sort and two-half merge when
+    every key involved is distinct.  Points on a line and queries beyond its ends make all distances of a search distinct
+    (and exact), so that path does the merging here; ids, distances and counters must be the oracle's.  A second data
+    set repeats every position once: beams with equal keys, where the networks must take over."""
+    from oracle import oracle as O
+    rng = np.random.default_rng(deg)
+    n = 3000
+    for repeats in (1, 2):
+        data = np.zeros((n, 4), np.float32)
+        data[:, 0] = rng.permutation(n) // repeats
+        queries = np.zeros((120, 4), np.float32)
+        queries[:60, 0] = n + 0.5 + np.arange(60)
+        queries[60:, 0] = -0.5 - np.arange(60)
+        graph = rng.integers(0, n, (n, deg)).astype(np.uint32)
+        graph[rng.random(graph.shape) < 0.1] = 0xFFFFFFFF
+        centroids = data[:3].copy()
+        start_points = rng.integers(0, n, 3).astype(np.uint32)
+        for beam in (288, 448, 512):
+            sp = O.search_params(beam, deg)
+            args = (data, graph, centroids, start_points, queries, 10)
+            eids, edists, est = O.search(*args, **sp)
+            print("degree", deg, "repeats", repeats, "beam", beam, flush=True)
+            gids, gdists, gcnt = run_gpu_search(hip, *args, sp, counters=True)
+            assert np.array_equal(gids, eids) and np.array_equal(gdists, edists)
+            assert gcnt == [est["iterations"], est["rows_scored"], est["graph_rows"]]
+            if repeats == 1:
+                assert np.unique(edists[0]).size == 10
+
+
 @pytest.mark.parametrize("deg", [160, 256])
 def test_search_degree_above_128(hip, deg):
     """Degrees above 128 sort the candidate list as two half-wave networks, beams above 256 merge the same way
