@@ -191,6 +191,7 @@ def run_workload(args, workload, torch, want_cpu):
     if args.nnd_iterations:
         nnd_iters = args.nnd_iterations
     top_k = 10
+    info_cus = capi.device_info()["compute_units"]
     t0 = time.time()
     data, queries = make_data(workload, num, nq)
     if args.queries:
@@ -382,10 +383,11 @@ def run_workload(args, workload, torch, want_cpu):
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=(measured_traffic(workload, chosen["beam"]) or {}).get("bytes"),
                       traffic_source=(measured_traffic(workload, chosen["beam"]) or {}).get("source"),
-                      kernel="%s<%d,%d,%d>" % ("search_kernel_dense" if 128 < chosen["beam"] <= 256 and degree <= 128 and dim <= 512 else "search_kernel",
+                      kernel="%s<%d,%d,%d>" % ("search_team_kernel" if dim > 256 and nq * 4 <= 2 * 4 * info_cus else
+                                               "search_kernel_dense" if 128 < chosen["beam"] <= 256 and degree <= 128 and dim <= 512 else "search_kernel",
                                                64 if degree <= 64 else 128 if degree <= 128 else 256,
                                                64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256 if chosen["beam"] <= 256 else 512,
-                                               1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8),
+                                               1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8 if dim <= 1024 else 16),
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )
     # what scattered rows of this length can be read at on this GPU at all (a probe kernel that only gathers rows)
