@@ -400,6 +400,11 @@ def widen_u8(src, count, dst, stream=None):
     check(lib().glide_hip_widen_u8(_ptr(src), C.c_size_t(count), _ptr(dst), vp(stream)), "glide_hip_widen_u8")
 
 
+def copy_rows(src, num, src_dim, dst, dst_dim, stream=None):
+    check(lib().glide_hip_copy_rows(_ptr(src), C.c_uint64(num), C.c_uint32(src_dim), _ptr(dst), C.c_uint32(dst_dim), vp(stream)),
+          "glide_hip_copy_rows")
+
+
 def build_segment(segment_data, num, dim, knn_graph, knn_degree, start_point, graph_degree, beam, max_iterations,
                   min_iterations, hash_bit, hash_reset_interval, relaxant, metric, graph, counters=None, stream=None):
     check(lib().glide_hip_build_segment(_ptr(segment_data), u32(num), u32(dim), _ptr(knn_graph), u32(knn_degree),

@@ -17,6 +17,17 @@ __global__ __launch_bounds__(256) void widen_u8_kernel(const unsigned char* src,
     if (blockIdx.x == 0 && threadIdx.x < count % 4) dst[quads * 4 + threadIdx.x] = static_cast<float>(src[quads * 4 + threadIdx.x]);
 }
 
+// Rows of src_dim values into rows of dst_dim values: the first min(src_dim, dst_dim) values of each row, zeros behind
+// them.  One thread per destination value, so the stores are coalesced whatever the two row lengths are.
+__global__ __launch_bounds__(256) void copy_rows_kernel(const float* src, size_t num, uint32_t src_dim, float* dst, uint32_t dst_dim) {
+    const size_t total = num * dst_dim;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += static_cast<size_t>(gridDim.x) * 256) {
+        const size_t r = i / dst_dim;
+        const uint32_t c = static_cast<uint32_t>(i - r * dst_dim);
+        dst[i] = c < src_dim ? src[r * src_dim + c] : 0.f;
+    }
+}
+
 __global__ __launch_bounds__(64) void distance_batch_kernel(const float* a, const float* b, uint32_t n, uint32_t dim,
                                                             int metric, float* out) {
     const int lane = lane_id();
@@ -111,6 +122,15 @@ int glide_hip_widen_u8(const unsigned char* src, size_t count, float* dst, void*
     const size_t quads = (count + 3) / 4;
     const size_t blocks = (quads + 255) / 256;
     hipLaunchKernelGGL(widen_u8_kernel, dim3(static_cast<uint32_t>(blocks < 16384 ? blocks : 16384)), dim3(256), 0, as_stream(stream), src, count, dst);
+    return launch_status();
+}
+
+int glide_hip_copy_rows(const float* src, uint64_t num, uint32_t src_dim, float* dst, uint32_t dst_dim, void* stream) {
+    if (!src || !dst || src_dim == 0 || dst_dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
+    if (num == 0) return GLIDE_OK;
+    const size_t blocks = (static_cast<size_t>(num) * dst_dim + 255) / 256;
+    hipLaunchKernelGGL(copy_rows_kernel, dim3(static_cast<uint32_t>(blocks < 65536 ? blocks : 65536)), dim3(256), 0, as_stream(stream), src,
+                       static_cast<size_t>(num), src_dim, dst, dst_dim);
     return launch_status();
 }
 

@@ -35,14 +35,14 @@ public:
     // glide_large_impl.cuh:14-28: an index to be built
     GLIDE_large(device_resources& handle, uint32_t graph_degree, Metric metric, std::string& reorder_file, std::string& map_file,
                 std::string& centroid_file, std::string& segment_file)
-        : handle(handle), metric(metric), h_data(load_matrix_pinned<Data_t>(reorder_file)), h_map(load_vector_data(map_file)),
-          h_centroids(load_matrix_data<float, uint32_t>(centroid_file)), h_segment_start(load_segment_start(segment_file)),
+        : handle(handle), metric(metric), h_data(load_points_pinned<Data_t>(reorder_file)), h_map(load_vector_data(map_file)),
+          h_centroids(load_point_data<float, uint32_t>(centroid_file, 16 / sizeof(Data_t))), h_segment_start(load_segment_start(segment_file)),
           h_segment_length(load_segment_length(segment_file)), h_start_point(h_segment_start.size()), h_graph(point_num(), graph_degree) {}
     // glide_large_impl.cuh:29-43: a finished index
     GLIDE_large(device_resources& handle, Metric metric, std::string& reorder_file, std::string& map_file, std::string& centroid_file,
                 std::string& segment_file, std::string& start_point_file, std::string& graph_file)
-        : handle(handle), metric(metric), h_data(load_matrix_pinned<Data_t>(reorder_file)), h_map(load_vector_data(map_file)),
-          h_centroids(load_matrix_data<float, uint32_t>(centroid_file)), h_segment_start(load_segment_start(segment_file)),
+        : handle(handle), metric(metric), h_data(load_points_pinned<Data_t>(reorder_file)), h_map(load_vector_data(map_file)),
+          h_centroids(load_point_data<float, uint32_t>(centroid_file, 16 / sizeof(Data_t))), h_segment_start(load_segment_start(segment_file)),
           h_segment_length(load_segment_length(segment_file)), h_start_point(load_vector_data(start_point_file)),
           h_graph(load_matrix_pinned<uint32_t>(graph_file)) {}
 

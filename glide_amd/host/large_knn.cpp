@@ -12,7 +12,7 @@ using namespace glide;
 template <typename Data_t>
 static void run(device_resources& handle, const std::string& preprocess_file, const std::string& knn_file, std::string& result_file,
                 uint32_t knn_degree) {
-    auto h_reorder = load_matrix_pinned<Data_t>(preprocess_file + ".reorder");
+    auto h_reorder = load_points_pinned<Data_t>(preprocess_file + ".reorder");
     auto h_segment_start = load_segment_start(preprocess_file + ".segment");
     auto h_segment_length = load_segment_length(preprocess_file + ".segment");
     const uint32_t iterations = std::getenv("GLIDE_NND_ITERATIONS") ? std::atoi(std::getenv("GLIDE_NND_ITERATIONS")) : 20;

@@ -16,7 +16,8 @@ using namespace glide;
 template <typename Data_t>
 static void run(device_resources& handle, PartitionParameter& param, const std::string& data_file, const std::string& preprocess_file,
                 std::string& result_file, uint32_t batch_num) {
-    auto h_data = load_matrix_pinned<Data_t>(data_file);
+    uint32_t file_dim = 0;   // rows are held padded to 16 bytes (load.hpp); the files written below keep the data file's length
+    auto h_data = load_points_pinned<Data_t>(data_file, &file_dim);
     const size_t num = h_data.extent(0), dim = h_data.extent(1);
     pinned_matrix<Data_t> h_reorder(num, dim);
     host_vector<uint32_t> h_map(num), h_segment_start(param.centroid_num), h_segment_length(param.centroid_num);
@@ -25,24 +26,25 @@ static void run(device_resources& handle, PartitionParameter& param, const std::
                                 batch_num, result_file);
     host_matrix<float> h_centroids(param.centroid_num, dim);
     copy_to_host(h_centroids.data_handle(), d_centroids.data_handle(), h_centroids.size());
-    save_matrix_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view());
+    save_point_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view(), file_dim);
     save_segment(preprocess_file + ".segment", std::as_const(h_segment_start).view(), std::as_const(h_segment_length).view());
     save_vector_data(preprocess_file + ".map", std::as_const(h_map).view());
-    save_matrix_pinned(preprocess_file + ".reorder", h_reorder);
+    save_points_pinned(preprocess_file + ".reorder", h_reorder, file_dim);
 }
 
 template <typename Data_t>
 static void run_merge(device_resources& handle, PartitionParameter& param, const std::string& data_file, const std::string& preprocess_file,
                       std::string& result_file, uint32_t batch_num) {
-    auto h_data = load_matrix_pinned<Data_t>(data_file);
+    uint32_t file_dim = 0;   // rows are held padded to 16 bytes (load.hpp); the files written below keep the data file's length
+    auto h_data = load_points_pinned<Data_t>(data_file, &file_dim);
     device_matrix<float> d_centroids(param.centroid_num, h_data.extent(1));
     auto part = preprocess_for_large_merge<Data_t>(handle, param, h_data, d_centroids.view(), batch_num, result_file);
     host_matrix<float> h_centroids(param.centroid_num, h_data.extent(1));
     copy_to_host(h_centroids.data_handle(), d_centroids.data_handle(), h_centroids.size());
-    save_matrix_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view());
+    save_point_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view(), file_dim);
     save_segment(preprocess_file + ".segment", std::as_const(part.h_segment_start).view(), std::as_const(part.h_segment_length).view());
     save_vector_data(preprocess_file + ".map", std::as_const(part.h_map).view());
-    save_matrix_pinned(preprocess_file + ".reorder", part.h_reorder_data);
+    save_points_pinned(preprocess_file + ".reorder", part.h_reorder_data, file_dim);
 }
 
 int main(int argc, char** argv) {

@@ -51,7 +51,7 @@ int main(int argc, char** argv) {
         adjust_search_params(param.min_iterations, param.max_iterations, param.beam);
         param.hash_bit = calculate_hash_bitlen(param.beam, index.graph_degree(), param.hash_max_fill_rate, param.hashmap_min_bitlen);
         param.hash_reset_interval = calculate_hash_reset_interval(param.beam, index.graph_degree(), param.hash_max_fill_rate, param.hash_bit);
-        auto h_query = load_matrix_data<Data_t, uint32_t>(query_file);
+        auto h_query = load_point_data<Data_t, uint32_t>(query_file);
         device_matrix<Data_t> d_query(h_query.extent(0), h_query.extent(1));
         copy_to_device(d_query.data_handle(), h_query.data_handle(), h_query.size());
         index.search(param, min_segment_num, boundary_factor, d_query.view(), result_ids.view(), result_dists.view(), result_file);

@@ -59,6 +59,30 @@ pinned_matrix<T> load_matrix_pinned(const std::string& path) {
     return m;
 }
 
+// A file of points into pinned memory, rows padded by zeros to a multiple of 16 bytes (load.hpp: load_point_data).
+template <typename T>
+pinned_matrix<T> load_points_pinned(const std::string& path, uint32_t* file_dim = nullptr) {
+    std::ifstream file(path, std::ios::binary);
+    if (!file) std::cerr << "Error opening file: " << path << std::endl;
+    uint32_t num = 0, dim = 0;
+    file.read(reinterpret_cast<char*>(&num), sizeof(uint32_t));
+    file.read(reinterpret_cast<char*>(&dim), sizeof(uint32_t));
+    if (file_dim) *file_dim = dim;
+    constexpr uint32_t multiple = 16 / sizeof(T);
+    const uint32_t held = (dim + multiple - 1) / multiple * multiple;
+    if (held == dim) return load_matrix_pinned<T>(path);
+    pinned_matrix<T> m(num, held);
+    for (size_t r = 0; r < num; r++) {
+        file.read(reinterpret_cast<char*>(m.row(r)), static_cast<std::streamsize>(dim * sizeof(T)));
+        std::memset(m.row(r) + dim, 0, (held - dim) * sizeof(T));
+    }
+    return m;
+}
+
+// The first `file_dim` values of every row.
+template <typename T>
+void save_points_pinned(const std::string& path, const pinned_matrix<T>& m, uint32_t file_dim);
+
 template <typename T>
 void save_matrix_pinned(const std::string& path, const pinned_matrix<T>& m) {
     std::ofstream file(path, std::ios::binary);
@@ -74,6 +98,16 @@ void save_matrix_pinned(const std::string& path, const pinned_matrix<T>& m) {
         src += n;
         left -= n;
     }
+}
+
+template <typename T>
+void save_points_pinned(const std::string& path, const pinned_matrix<T>& m, uint32_t file_dim) {
+    if (file_dim == m.extent(1)) return save_matrix_pinned(path, m);
+    std::ofstream file(path, std::ios::binary);
+    const uint32_t num = m.extent(0);
+    file.write(reinterpret_cast<const char*>(&num), sizeof(uint32_t));
+    file.write(reinterpret_cast<const char*>(&file_dim), sizeof(uint32_t));
+    for (size_t r = 0; r < m.extent(0); r++) file.write(reinterpret_cast<const char*>(m.row(r)), static_cast<std::streamsize>(file_dim * sizeof(T)));
 }
 
 // Size in bytes of one element of an fbin file, from its length: header (num, dim) + num * dim elements.  The reference's

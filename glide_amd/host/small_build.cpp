@@ -39,12 +39,12 @@ int main(int argc, char** argv) {
     search_param_refine.beam = std::stoi(argv[11]);
     if (search_param_refine.beam != 0) size_param(search_param_refine, search_param_refine.beam);
 
-    auto h_data = load_matrix_data<float, uint32_t>(data_file);
-    auto h_centroids = load_matrix_data<float, uint32_t>(preprocess_file + ".centroid");
+    auto h_data = load_point_data<float, uint32_t>(data_file);
+    auto h_centroids = load_point_data<float, uint32_t>(preprocess_file + ".centroid");
     auto h_segment_start = load_segment_start(preprocess_file + ".segment");
     auto h_segment_length = load_segment_length(preprocess_file + ".segment");
     auto h_map = load_vector_data(preprocess_file + ".map");
-    auto h_reorder_data = load_matrix_data<float, uint32_t>(preprocess_file + ".reorder");
+    auto h_reorder_data = load_point_data<float, uint32_t>(preprocess_file + ".reorder");
     auto h_knn_graph = load_matrix_data<uint32_t, uint32_t>(knn_file);
 
     std::optional<device_matrix<float, uint32_t>> d_reorder_data;

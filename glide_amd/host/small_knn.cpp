@@ -19,7 +19,7 @@ int main(int argc, char** argv) {
     std::string preprocess_file(argv[1]), knn_file(argv[2]), result_file(argv[3]);
     const uint32_t knn_degree = std::stoi(argv[4]);
 
-    auto h_reorder = load_matrix_data<float, uint32_t>(preprocess_file + ".reorder");
+    auto h_reorder = load_point_data<float, uint32_t>(preprocess_file + ".reorder");
     auto h_segment_start = load_segment_start(preprocess_file + ".segment");
     auto h_segment_length = load_segment_length(preprocess_file + ".segment");
     std::optional<device_matrix<float>> d_data;

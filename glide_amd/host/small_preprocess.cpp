@@ -32,7 +32,8 @@ int main(int argc, char** argv) {
         result_out << "pre_time,knn_time,degree,index_time,beam,search_time,QPS,recall" << std::endl;
     }
 
-    auto h_data = load_matrix_data<float, uint32_t>(data_file);
+    uint32_t file_dim = 0;   // rows are held padded to a multiple of four values (load.hpp); the files written below keep the data file's length
+    auto h_data = load_point_data<float, uint32_t>(data_file, 4, &file_dim);
     const uint32_t num = h_data.extent(0), dim = h_data.extent(1);
     device_matrix<float, uint32_t> d_data(num, dim);
     copy_to_device(d_data.data_handle(), h_data.data_handle(), h_data.size());
@@ -51,9 +52,9 @@ int main(int argc, char** argv) {
     host_vector<uint32_t> h_map(d_map->size());
     copy_to_host(h_map.data_handle(), d_map->data_handle(), h_map.size());
 
-    save_matrix_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view());
+    save_point_data<float, uint32_t>(preprocess_file + ".centroid", std::as_const(h_centroids).view(), file_dim);
     save_segment(preprocess_file + ".segment", std::as_const(h_segment_start).view(), std::as_const(h_segment_length).view());
     save_vector_data(preprocess_file + ".map", std::as_const(h_map).view());
-    save_matrix_data<float, uint32_t>(preprocess_file + ".reorder", std::as_const(h_reorder).view());
+    save_point_data<float, uint32_t>(preprocess_file + ".reorder", std::as_const(h_reorder).view(), file_dim);
     return 0;
 }

@@ -33,10 +33,10 @@ int main(int argc, char** argv) {
         result_file(argv[6]), metric_name(argv[7]);
     Metric metric = metric_name == "Cosine" ? Metric::Cosine : Metric::Euclidean;
 
-    auto h_data = load_matrix_data<float, uint32_t>(data_file);
-    auto h_query = load_matrix_data<float, uint32_t>(query_file);
+    auto h_data = load_point_data<float, uint32_t>(data_file);
+    auto h_query = load_point_data<float, uint32_t>(query_file);
     auto h_truth = load_matrix_data<uint32_t, uint32_t>(truth_file);
-    auto h_centroids = load_matrix_data<float, uint32_t>(preprocess_file + ".centroid");
+    auto h_centroids = load_point_data<float, uint32_t>(preprocess_file + ".centroid");
     auto h_graph = load_matrix_data<uint32_t, uint32_t>(graph_base_file + ".graph");
     auto h_start_points = load_vector_data(graph_base_file + ".sp");
 

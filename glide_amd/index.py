@@ -138,12 +138,48 @@ class _Timer:
         self.seconds = self.start.elapsed_ms(self.stop) / 1000.0
 
 
+def pad_rows(rows, multiple=4):
+    """Points as the entry points want them: fp32 rows on the device whose length is a multiple of four values.  The
+    reference's kernels loop over single values and take any dim (distance.cuh:9-27); here rows are read in 16-byte
+    pieces, so points of another length get zeros behind them once, which changes no squared distance, inner product
+    or norm.  numpy (num, dim) or DeviceArray in, DeviceArray (num, padded dim) out -- the same DeviceArray when its
+    rows already fit, else a padded copy made on the device."""
+    d = rows if isinstance(rows, capi.DeviceArray) else capi.DeviceArray.from_numpy(rows, np.float32)
+    num, dim = d.shape
+    held = (dim + multiple - 1) // multiple * multiple
+    if held == dim:
+        return d
+    out = capi.DeviceArray((num, held), np.float32)
+    capi.copy_rows(d, num, dim, out, held)
+    capi.synchronize()
+    if d is not rows:
+        d.free()
+    return out
+
+
+def cut_rows(d_rows, dim):
+    """The first `dim` values of every row of a DeviceArray of points, as numpy: centroids or reordered rows of padded
+    points in the length the caller's data has."""
+    num, held = d_rows.shape
+    if held == dim:
+        return d_rows.numpy()
+    out = capi.DeviceArray((num, dim), np.float32)
+    capi.copy_rows(d_rows, num, held, out, dim)
+    capi.synchronize()
+    h = out.numpy()
+    out.free()
+    return h
+
+
 def preprocess(param, d_data, result=None):
-    """partition.cuh:159-193.  d_data: DeviceArray (num, dim) float32.
+    """partition.cuh:159-193.  d_data: DeviceArray (num, dim) float32; rows of a length that is no multiple of four are
+    padded (pad_rows), and the reordered rows and centroids returned then have the padded length (cut_rows gives them
+    back in the data's own).
 
     Returns (d_reorder_data, d_map, h_segment_start, h_segment_length, d_centroids).  h_segment_* have
     centroid_num + 1 entries, the last being the boundary segment (start = num).
     """
+    d_data = pad_rows(d_data)
     num, dim = d_data.shape
     c = param.centroid_num
     times = {}
@@ -216,11 +252,14 @@ class GLIDE:
     """glide.cuh:14-125 for Data_t = float, Index_t = uint32_t."""
 
     def __init__(self, graph_degree, data, centroids, metric):
-        """data: numpy (num, dim) float32 or DeviceArray; centroids likewise (glide_impl.cuh:15-30)."""
+        """data: numpy (num, dim) float32 or DeviceArray; centroids likewise (glide_impl.cuh:15-30).  Rows of a length
+        that is no multiple of four are held padded (pad_rows); dim() is then the padded length."""
         _check_sizes(0, graph_degree)
         self.metric = metric
-        self.d_data = data if isinstance(data, capi.DeviceArray) else capi.DeviceArray.from_numpy(data, np.float32)
-        self.d_centroids = centroids if isinstance(centroids, capi.DeviceArray) else capi.DeviceArray.from_numpy(centroids, np.float32)
+        self.d_data = pad_rows(data)
+        self.d_centroids = pad_rows(centroids)
+        if self.d_centroids.shape[1] != self.d_data.shape[1]:
+            raise ValueError("centroids of %d values for points of %d" % (self.d_centroids.shape[1], self.d_data.shape[1]))
         self._graph_degree = int(graph_degree)
         self.d_graph = capi.DeviceArray((self.num(), self._graph_degree), np.uint32)
         self.d_start_points = None
@@ -319,9 +358,13 @@ class GLIDE:
             result["build_stages"] = times
 
     def search(self, param, d_query, result=None, counters=None, stream=None, out=None):
-        """glide_impl.cuh:370-454.  d_query: DeviceArray (query_num, dim).  Returns (ids, dists) as numpy arrays
-        unless `out` = (d_ids, d_dists) is given, in which case nothing is copied back."""
+        """glide_impl.cuh:370-454.  d_query: DeviceArray (query_num, dim), in the data's own row length or padded as
+        the data is held.  Returns (ids, dists) as numpy arrays unless `out` = (d_ids, d_dists) is given, in which case
+        nothing is copied back."""
         _check_sizes(param.beam, self._graph_degree)
+        d_query = pad_rows(d_query)
+        if d_query.shape[1] != self.dim():
+            raise ValueError("queries of %d values for points of %d" % (d_query.shape[1], self.dim()))
         nq = d_query.shape[0]
         d_ids, d_dists = out if out is not None else (capi.DeviceArray((nq, param.top_k), np.uint32), capi.DeviceArray((nq, param.top_k), np.float32))
         with _Timer() as t:

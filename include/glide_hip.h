@@ -414,6 +414,13 @@ int glide_hip_stream_wait_event(void *stream, void *event);
  * graph_kernel.cuh:675-821); here a staged partition is widened once after its upload and every kernel reads fp32. */
 int glide_hip_widen_u8(const unsigned char *src, size_t count, float *dst, void *stream);
 
+/* Rows of src_dim values -> rows of dst_dim values: the first min(src_dim, dst_dim) values of every row, zeros behind
+ * them (both 4-byte aligned, no overlap).  Every other entry point reads rows in 16-byte pieces and wants dim % 4 == 0;
+ * the reference's kernels loop over single values and take any dim (distance.cuh:9-27).  Points of another length are
+ * padded once with this call (dst_dim = dim rounded up to a multiple of 4; a zero coordinate changes no squared
+ * distance, inner product or norm) and centroids or reordered rows are cut back with it where a caller wants them. */
+int glide_hip_copy_rows(const float *src, uint64_t num, uint32_t src_dim, float *dst, uint32_t dst_dim, void *stream);
+
 /* ---- test hooks for the device primitives (subsystems 5, 6 and the hash set) ------------------------------ */
 /* compute_similarity_warp (distance.cuh:9-27): out[i] = dist(a[i], b[i]) for n row pairs */
 int glide_hip_distance_batch(const float *a, const float *b, uint32_t n, uint32_t dim, int metric, float *out,
