@@ -383,7 +383,7 @@ def run_workload(args, workload, torch, want_cpu):
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=(measured_traffic(workload, chosen["beam"]) or {}).get("bytes"),
                       traffic_source=(measured_traffic(workload, chosen["beam"]) or {}).get("source"),
-                      kernel="%s<%d,%d,%d>" % ("search_team_kernel" if dim > 256 and nq * 4 <= 2 * 4 * info_cus else
+                      kernel=("%s<%d,%d,%d,true>" if chosen["beam"] == 512 else "%s<%d,%d,%d>") % ("search_team_kernel" if dim > 256 and nq * 4 <= 2 * 4 * info_cus else
                                                "search_kernel_dense" if 128 < chosen["beam"] <= 256 and degree <= 128 and dim <= 512 else "search_kernel",
                                                64 if degree <= 64 else 128 if degree <= 128 else 256,
                                                64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256 if chosen["beam"] <= 256 else 512,

@@ -36,7 +36,8 @@ struct BeamLds {  // per-wave LDS (the hash table follows, 1 << hash_bit words)
 inline size_t beam_lds_bytes(uint32_t degree) {
     return degree <= 64 ? sizeof(BeamLds<64>) : degree <= 128 ? sizeof(BeamLds<128>) : sizeof(BeamLds<256>);
 }
-inline size_t beam_stage_bytes(uint32_t beam) { return beam > 256 ? (2 * (512 + 4) + 4) * sizeof(uint32_t) : 0; }
+// A kernel that merges the whole of the widest beam in its registers (Beam<..., WHOLE>) stages nothing.
+inline size_t beam_stage_bytes(uint32_t beam, bool whole = false) { return beam > 256 && !whole ? (2 * (512 + 4) + 4) * sizeof(uint32_t) : 0; }
 
 __device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
 // The same point in a wavefront that shares its workgroup with others (TEAM): a workgroup barrier would wait for them.
@@ -107,8 +108,11 @@ __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float
 }
 
 // TEAM: the beam's wavefront is one of several in its workgroup (the others only score rows, see search_team_kernel).
-template <int MAX_CAND, int MAX_BEAM, int DIMV, bool TEAM = false>
+// WHOLE: the host promises beam == MAX_BEAM (asked for beams above 256 only, i.e. beam 512): the beam merge then stays in
+// the registers (merge_beam_full), and a kernel without the staged two-half merge needs 126 registers instead of 161.
+template <int MAX_CAND, int MAX_BEAM, int DIMV, bool TEAM = false, bool WHOLE = false>
 struct Beam {
+    static_assert(!WHOLE || MAX_BEAM > 256, "beams up to 256 merge in the registers anyway");
     static __device__ __forceinline__ void wave_sync() { wave_sync_in<TEAM>(); }
     static constexpr int NB = MAX_BEAM / 64;
     static constexpr int NC = MAX_CAND / 64;
@@ -382,6 +386,47 @@ struct Beam {
         return true;
     }
 
+    // v of the lane 32 places away: one swap of the 32-lane halves of a register pair and a select
+    template <class T>
+    static __device__ __forceinline__ T other_half(T v, bool upper) {
+        const int x = __builtin_bit_cast(int, v);
+        const auto s = __builtin_amdgcn_permlane32_swap(x, x, false, false);   // s[0]: upper lanes hold the lower half's, s[1]: the reverse
+        return __builtin_bit_cast(T, upper ? s[0] : s[1]);
+    }
+
+    // The same merge for a beam of exactly MAX_BEAM entries, in the registers.  Element NB * lane + r puts the two halves
+    // of the beam into the two 32-lane halves of the wavefront, each in the order its merge network wants, so the
+    // compare-exchange between the halves is a swap of register halves; and with half == PER the layout
+    // [untouched prefix | padding | touched rest] of a half is the half as it stands, whatever the turning points are,
+    // so they are not tracked.  No copy of the beam through LDS, no LDS atomics, no waits between the steps.
+    __device__ __forceinline__ void merge_beam_full() {
+        bool replaced = false;
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const uint32_t k = MAX_BEAM - 1 - (NB * lane + r);
+            if (k < p.degree) {
+                const float c = lds->cand_dist[k];
+                if (bk[r] > c) {
+                    bk[r] = c;
+                    bv[r] = lds->cand_id[k];
+                    replaced = true;
+                }
+            }
+        }
+        if (ballot(replaced) == 0) return;
+        const bool upper = lane >= 32;
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const float ok = other_half(bk[r], upper);
+            const uint32_t ov = other_half(bv[r], upper);
+            const bool take = upper ? ok > bk[r] : bk[r] > ok;   // entry j of the first half and entry j of the second change places when the first is larger
+            bk[r] = take ? ok : bk[r];
+            bv[r] = take ? ov : bv[r];
+            __builtin_amdgcn_sched_barrier(0);   // one register at a time: interleaved, the eight exchanges cost the kernel a wavefront per SIMD in registers
+        }
+        WaveNet<MAX_BEAM / 2, 32>::merge(bk, bv, lane);
+    }
+
     // The candidates of the latest expansion that are below the last beam entry, as a lane mask (one candidate slot per
     // lane).  None: the beam stays as it is -- the half-cleaner of the merge replaces an entry only by a strictly smaller
     // candidate, entry `beam - 1 - k` by the k-th smallest, so if even the smallest candidate is not below the largest
@@ -517,7 +562,9 @@ struct Beam {
                 float ck;
                 const uint64_t em = entering(ck);
                 if (em == 0) return;
-                if constexpr (MAX_BEAM > 256) {
+                if constexpr (MAX_BEAM > 256 && !WHOLE) {
+                    // (A WHOLE kernel does without: its merge is cheap, and without the staging area four of its wavefronts
+                    // fit a SIMD's share of the LDS instead of three, which is worth more than the shortcut was.)
                     // Only worth trying on a beam without equal keys (on integer-valued rows a beam of 512 rarely is): a
                     // failed attempt is time lost on a path that is bound by the latency of its own steps.  After a beam
                     // with equal keys, or an attempt that failed on a candidate's key, the next 16 merges go straight to
@@ -543,7 +590,8 @@ struct Beam {
             }
             if constexpr (MAX_BEAM > 256) ranked_pause = 0;
         } else if constexpr (MAX_BEAM > 256) {
-            merge_beam_two();
+            if constexpr (WHOLE) merge_beam_full();
+            else merge_beam_two();
         } else {
             bool replaced = false;
 #pragma unroll

@@ -29,7 +29,7 @@ __device__ __forceinline__ uint32_t pick_centroid(uint32_t max_centroid, const R
     }
 }
 
-template <int MAX_CAND, int MAX_BEAM, int DIMV>
+template <int MAX_CAND, int MAX_BEAM, int DIMV, bool WHOLE = false>
 __device__ __forceinline__ void search_body(const SearchArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     auto* lds = reinterpret_cast<BeamLds<MAX_CAND>*>(smem);
@@ -37,7 +37,7 @@ __device__ __forceinline__ void search_body(const SearchArgs a) {
     uint32_t* hash = reinterpret_cast<uint32_t*>(cent + round_up32(a.centroid_num));
     // a wavefront takes queries blockIdx.x, blockIdx.x + gridDim.x, ... (the host sizes the grid)
     for (uint32_t qid = blockIdx.x; qid < a.query_num; qid += gridDim.x) {
-        Beam<MAX_CAND, MAX_BEAM, DIMV> b;
+        Beam<MAX_CAND, MAX_BEAM, DIMV, false, WHOLE> b;
         b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
         const uint32_t c0 = pick_centroid<DIMV>(a.max_centroid, b.q, a.centroids, a.centroid_num, a.p.dim, a.p.metric, cent, b.lane);
         const uint32_t entry = a.start_points[c0];
@@ -58,9 +58,9 @@ __device__ __forceinline__ void search_body(const SearchArgs a) {
     }
 }
 
-template <int MAX_CAND, int MAX_BEAM, int DIMV>
+template <int MAX_CAND, int MAX_BEAM, int DIMV, bool WHOLE = false>
 __global__ __launch_bounds__(64) void search_kernel(SearchArgs a) {
-    search_body<MAX_CAND, MAX_BEAM, DIMV>(a);
+    search_body<MAX_CAND, MAX_BEAM, DIMV, WHOLE>(a);
 }
 // The beam-256 kernels are bound by the vector ALU (sorting networks) and need 103 registers, one wavefront per SIMD
 // short of the next occupancy step: held to five wavefronts per SIMD (96 registers, five of them spilled) they run
@@ -88,7 +88,7 @@ struct TeamShape {
     static constexpr size_t query_bytes = sizeof(float4) * RowShape<DIMV>::NV * RowShape<DIMV>::LPR;
 };
 
-template <int MAX_CAND, int MAX_BEAM, int DIMV>
+template <int MAX_CAND, int MAX_BEAM, int DIMV, bool WHOLE = false>
 __global__ __launch_bounds__(64 * kTeam) void search_team_kernel(SearchArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     using Shape = RowShape<DIMV>;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(64 * kTeam) void search_team_kernel(SearchArgs a) {
     const uint32_t wave = threadIdx.x >> 6;
     const int lane = lane_id();
     for (uint32_t qid = blockIdx.x; qid < a.query_num; qid += gridDim.x) {
-        Beam<MAX_CAND, MAX_BEAM, DIMV, true> b;
+        Beam<MAX_CAND, MAX_BEAM, DIMV, true, WHOLE> b;
         uint32_t iter = 0;
         bool terminate = false;
         if (wave == 0) {
@@ -387,7 +387,7 @@ __device__ __forceinline__ void merge_result(const float* beam_dist, const uint3
 }
 
 // search_on_sub_kernel (search_kernel.cuh:653-765)
-template <int MAX_CAND, int MAX_BEAM, int DIMV>
+template <int MAX_CAND, int MAX_BEAM, int DIMV, bool WHOLE = false>
 __global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     auto* lds = reinterpret_cast<BeamLds<MAX_CAND>*>(smem);
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
         if (!is_search) return;
     }
 
-    Beam<MAX_CAND, MAX_BEAM, DIMV> b;
+    Beam<MAX_CAND, MAX_BEAM, DIMV, false, WHOLE> b;
     b.init(lds, hash, a.p, a.queries + static_cast<size_t>(qid) * a.p.dim);
     b.expand(start_point, graph, data, kInvalid, kInvalid);   // get_init with point_id = 0xffffffff
     b.run(graph, data, kInvalid);
@@ -470,46 +470,48 @@ __global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
 using search_fn = void (*)(SearchArgs);
 using sub_fn = void (*)(SubArgs);
 
-template <int MAX_CAND, int MAX_BEAM>
+template <int MAX_CAND, int MAX_BEAM, bool WHOLE = false>
 sub_fn pick_sub_dim(uint32_t dim) {
-    if (dim <= 128) return search_sub_kernel<MAX_CAND, MAX_BEAM, 1>;
-    if (dim <= 256) return search_sub_kernel<MAX_CAND, MAX_BEAM, 2>;
-    if (dim <= 512) return search_sub_kernel<MAX_CAND, MAX_BEAM, 4>;
-    if (dim <= 1024) return search_sub_kernel<MAX_CAND, MAX_BEAM, 8>;
-    return search_sub_kernel<MAX_CAND, MAX_BEAM, 16>;
+    if (dim <= 128) return search_sub_kernel<MAX_CAND, MAX_BEAM, 1, WHOLE>;
+    if (dim <= 256) return search_sub_kernel<MAX_CAND, MAX_BEAM, 2, WHOLE>;
+    if (dim <= 512) return search_sub_kernel<MAX_CAND, MAX_BEAM, 4, WHOLE>;
+    if (dim <= 1024) return search_sub_kernel<MAX_CAND, MAX_BEAM, 8, WHOLE>;
+    return search_sub_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
 }
 template <int MAX_CAND>
 sub_fn pick_sub_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_sub_dim<MAX_CAND, 64>(dim);
     if (beam <= 128) return pick_sub_dim<MAX_CAND, 128>(dim);
     if (beam <= 256) return pick_sub_dim<MAX_CAND, 256>(dim);
+    if (beam == 512) return pick_sub_dim<MAX_CAND, 512, true>(dim);   // the whole of the widest beam: merged in the registers
     return pick_sub_dim<MAX_CAND, 512>(dim);
 }
 
-template <int MAX_CAND, int MAX_BEAM>
+template <int MAX_CAND, int MAX_BEAM, bool WHOLE = false>
 search_fn pick_dim(uint32_t dim) {
     if constexpr (MAX_BEAM == 256 && MAX_CAND <= 128) {
         if (dim <= 128) return search_kernel_dense<MAX_CAND, MAX_BEAM, 1>;
         if (dim <= 256) return search_kernel_dense<MAX_CAND, MAX_BEAM, 2>;
         if (dim <= 512) return search_kernel_dense<MAX_CAND, MAX_BEAM, 4>;
     }
-    if (dim <= 128) return search_kernel<MAX_CAND, MAX_BEAM, 1>;
-    if (dim <= 256) return search_kernel<MAX_CAND, MAX_BEAM, 2>;
-    if (dim <= 512) return search_kernel<MAX_CAND, MAX_BEAM, 4>;
-    if (dim <= 1024) return search_kernel<MAX_CAND, MAX_BEAM, 8>;
-    return search_kernel<MAX_CAND, MAX_BEAM, 16>;
+    if (dim <= 128) return search_kernel<MAX_CAND, MAX_BEAM, 1, WHOLE>;
+    if (dim <= 256) return search_kernel<MAX_CAND, MAX_BEAM, 2, WHOLE>;
+    if (dim <= 512) return search_kernel<MAX_CAND, MAX_BEAM, 4, WHOLE>;
+    if (dim <= 1024) return search_kernel<MAX_CAND, MAX_BEAM, 8, WHOLE>;
+    return search_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
 }
-template <int MAX_CAND, int MAX_BEAM>
+template <int MAX_CAND, int MAX_BEAM, bool WHOLE = false>
 search_fn pick_team_dim(uint32_t dim) {
-    if (dim <= 512) return search_team_kernel<MAX_CAND, MAX_BEAM, 4>;
-    if (dim <= 1024) return search_team_kernel<MAX_CAND, MAX_BEAM, 8>;
-    return search_team_kernel<MAX_CAND, MAX_BEAM, 16>;
+    if (dim <= 512) return search_team_kernel<MAX_CAND, MAX_BEAM, 4, WHOLE>;
+    if (dim <= 1024) return search_team_kernel<MAX_CAND, MAX_BEAM, 8, WHOLE>;
+    return search_team_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
 }
 template <int MAX_CAND>
 search_fn pick_team_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_team_dim<MAX_CAND, 64>(dim);
     if (beam <= 128) return pick_team_dim<MAX_CAND, 128>(dim);
     if (beam <= 256) return pick_team_dim<MAX_CAND, 256>(dim);
+    if (beam == 512) return pick_team_dim<MAX_CAND, 512, true>(dim);
     return pick_team_dim<MAX_CAND, 512>(dim);
 }
 template <int MAX_CAND>
@@ -517,6 +519,7 @@ search_fn pick_beam(uint32_t beam, uint32_t dim) {
     if (beam <= 64) return pick_dim<MAX_CAND, 64>(dim);
     if (beam <= 128) return pick_dim<MAX_CAND, 128>(dim);
     if (beam <= 256) return pick_dim<MAX_CAND, 256>(dim);
+    if (beam == 512) return pick_dim<MAX_CAND, 512, true>(dim);
     return pick_dim<MAX_CAND, 512>(dim);
 }
 
@@ -594,7 +597,7 @@ int launch_search(const float* data, uint32_t num, uint32_t dim, const uint32_t*
     if (team) fn = graph_degree <= 64 ? pick_team_beam<64>(beam, dim) : graph_degree <= 128 ? pick_team_beam<128>(beam, dim) : pick_team_beam<256>(beam, dim);
     else fn = graph_degree <= 64 ? pick_beam<64>(beam, dim) : graph_degree <= 128 ? pick_beam<128>(beam, dim) : pick_beam<256>(beam, dim);
     const size_t lds_bytes = beam_lds_bytes(graph_degree) + round_up32(centroid_num) * sizeof(float) +
-                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam) +
+                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam, beam == 512) +
                              (team ? (dim <= 512 ? TeamShape<4>::query_bytes : dim <= 1024 ? TeamShape<8>::query_bytes : TeamShape<16>::query_bytes) + 16 : 0);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     if (team) hipLaunchKernelGGL(fn, dim3(query_num), dim3(64 * kTeam), lds_bytes, as_stream(stream), a);
@@ -676,7 +679,7 @@ int launch_search_sub(const float* segment_data, uint32_t dim, const uint32_t* s
     a.max_topk = top_k <= 32 ? 32 : (top_k <= 64 ? 64 : 128);
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
     sub_fn fn = graph_degree <= 64 ? pick_sub_beam<64>(beam, dim) : graph_degree <= 128 ? pick_sub_beam<128>(beam, dim) : pick_sub_beam<256>(beam, dim);
-    const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam, beam == 512);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(query_list ? list_len : query_num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
@@ -811,7 +814,7 @@ extern "C" int glide_hip_search_partitions(const float* data, uint32_t dim, cons
         a.list_len = pairs;
         a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
         sub_fn fn = graph_degree <= 64 ? pick_sub_beam<64>(beam, dim) : graph_degree <= 128 ? pick_sub_beam<128>(beam, dim) : pick_sub_beam<256>(beam, dim);
-        const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+        const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam, beam == 512);
         GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
         hipLaunchKernelGGL(fn, dim3(pairs), dim3(64), lds_bytes, s, a);
     }
