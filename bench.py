@@ -105,6 +105,19 @@ def measured_knn(workload):
     return None
 
 
+def search_kernel_name(dim, degree, beam, queries, compute_units):
+    """The kernel glide_hip_search launches for this shape, as a profiler names it (search.hip: launch_search)."""
+    shape = "%d,%d,%d" % (64 if degree <= 64 else 128 if degree <= 128 else 256,
+                          64 if beam <= 64 else 128 if beam <= 128 else 256 if beam <= 256 else 512,
+                          1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8 if dim <= 1024 else 16)
+    whole = "true" if beam == 512 else "false"      # the whole of the widest beam: merged in the registers
+    if dim > 256 and queries * 4 <= 2 * 4 * compute_units:
+        return "search_team_kernel<%s,%s>" % (shape, whole)
+    if 128 < beam <= 256 and degree <= 128 and dim <= 512:
+        return "search_kernel_dense<%s>" % shape
+    return "search_kernel<%s,%s>" % (shape, whole)
+
+
 def measured_knn_bytes(workload):
     """HBM bytes (read + written) of all launches of the NN-descent stage of one workload, from the committed counter
     summary: FETCH_SIZE and WRITE_SIZE summed over the stage's launches, each scaled by the copy kernel's reading.  The
@@ -383,11 +396,7 @@ def run_workload(args, workload, torch, want_cpu):
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=(measured_traffic(workload, chosen["beam"]) or {}).get("bytes"),
                       traffic_source=(measured_traffic(workload, chosen["beam"]) or {}).get("source"),
-                      kernel=("%s<%d,%d,%d,true>" if chosen["beam"] == 512 else "%s<%d,%d,%d>") % ("search_team_kernel" if dim > 256 and nq * 4 <= 2 * 4 * info_cus else
-                                               "search_kernel_dense" if 128 < chosen["beam"] <= 256 and degree <= 128 and dim <= 512 else "search_kernel",
-                                               64 if degree <= 64 else 128 if degree <= 128 else 256,
-                                               64 if chosen["beam"] <= 64 else 128 if chosen["beam"] <= 128 else 256 if chosen["beam"] <= 256 else 512,
-                                               1 if dim <= 128 else 2 if dim <= 256 else 4 if dim <= 512 else 8 if dim <= 1024 else 16),
+                      kernel=search_kernel_name(dim, degree, chosen["beam"], nq, info_cus),
                       algorithmic_bytes_per_launch=chosen["algorithmic_bytes"]),
     )
     # what scattered rows of this length can be read at on this GPU at all (a probe kernel that only gathers rows)
