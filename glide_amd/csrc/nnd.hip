@@ -1025,14 +1025,15 @@ struct MergeArgs {
     uint32_t num, width, num_sub, bloom_sets;
 };
 
-constexpr uint32_t kKnownBits = 9;   // 512-slot id set per wavefront: lists of up to 192 entries + 32 offers
-template <uint32_t SLOTS>
+// KNOWN_BITS: id set per wavefront (512 slots for lists of up to 192 entries + 32 offers, 1024 for the wider lists of
+// degrees above 128); FILTER_WORDS: the node's Bloom filter (16 words per set of 32 entries of the internal degree).
+template <uint32_t SLOTS, uint32_t KNOWN_BITS, uint32_t FILTER_WORDS>
 struct MergeLds {
     unsigned long long keys[4][SLOTS];   // the node's offers, gaps closed
     unsigned long long best[4][kOfferThrRank];  // the best 32 of them (64 where a threshold is due)
     unsigned long long enter[4][kSamples];      // those that enter the list, as keys of the second sort
-    uint32_t known[4][1u << kKnownBits];
-    uint32_t filter[4][128];
+    uint32_t known[4][1u << KNOWN_BITS];
+    uint32_t filter[4][FILTER_WORDS];
     uint32_t flags[4][kSamples];
 };
 
@@ -1097,7 +1098,9 @@ __device__ __forceinline__ uint32_t best_offers_sized(const unsigned long long* 
 // M2 = size of the second network >= width + 32.
 template <int M2, uint32_t SLOTS>
 __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
-    __shared__ MergeLds<SLOTS> L;
+    constexpr uint32_t kKnownBits = M2 > 256 ? 10 : 9;
+    constexpr int kFilterPasses = M2 > 256 ? 4 : 2;   // Bloom filter words per lane: 128 words up to degree 128, 256 beyond
+    __shared__ MergeLds<SLOTS, kKnownBits, 64 * kFilterPasses> L;
     constexpr int NR = M2 / 64;
     constexpr int PASSES = SLOTS / 256;
     const int lane = lane_id();
@@ -1105,7 +1108,8 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
     const uint32_t node = blockIdx.x * 4 + wave;
     if (node >= a.num) return;
     const uint32_t width = a.width, num_sub = a.num_sub;
-    const uint32_t bloom_words = a.bloom_sets * 16;   // at most 128
+    const uint32_t bloom_words = a.bloom_sets * 16;   // at most 64 * kFilterPasses
+    if (bloom_words > 64u * kFilterPasses || width + kSamples > static_cast<uint32_t>(M2)) return;   // not a launch nnd_merge makes: the filter or the list would not fit this form's LDS
 
     // ---- everything the node needs from memory is asked for at once: the kernel is bound by the latency of its
     // dependent memory round trips (this one, the thresholds of the sampled nodes, the slots of their reverse lists),
@@ -1125,9 +1129,9 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
         l_id[r] = e < width ? a.list_ids[static_cast<size_t>(node) * width + e] : kInvalid;
         l_dist[r] = e < width ? a.list_dists[static_cast<size_t>(node) * width + e] : FLT_MAX;
     }
-    uint32_t bloom_in[2];
+    uint32_t bloom_in[kFilterPasses];
 #pragma unroll
-    for (int j = 0; j < 2; j++) bloom_in[j] = lane + 64u * j < bloom_words ? a.bloom[static_cast<size_t>(node) * bloom_words + lane + 64 * j] : 0u;
+    for (int j = 0; j < kFilterPasses; j++) bloom_in[j] = lane + 64u * j < bloom_words ? a.bloom[static_cast<size_t>(node) * bloom_words + lane + 64 * j] : 0u;
     const uint32_t in_force = __float_as_uint(a.norms[node].y);
     uint32_t seg_start, seg_len, state;
     const uint32_t seg = locate_uniform(a.segs, node, seg_start, seg_len, &state);
@@ -1141,7 +1145,7 @@ __global__ __launch_bounds__(256) void nnd_merge_kernel(MergeArgs a) {
     uint32_t* flags = L.flags[wave];
     for (uint32_t i = lane; i < (1u << kKnownBits); i += 64) known[i] = kInvalid;
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < kFilterPasses; j++)
         if (lane + 64u * j < bloom_words) filter[lane + 64 * j] = bloom_in[j];
     __builtin_amdgcn_wave_barrier();
 
@@ -1474,7 +1478,7 @@ using namespace glide;
 namespace {
 uint32_t nnd_width(uint32_t degree) { return round_up32(static_cast<uint32_t>(degree * (degree <= 32 ? 1.0 : 1.3))); }  // nn_descent.cuh:1427-1428
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
-constexpr uint32_t kMaxWidth = 192;   // six sub-lists: degrees up to 128 (width + 32 offers fit one 256-key network)
+constexpr uint32_t kMaxWidth = 480;   // width + 32 offers fit one 512-key network; degree 256, the widest the build searches take, needs 352
 
 struct NndLayout {
     size_t half_rows, norms, list_ids, list_dists, fwd_new, fwd_old, rev_new, rev_old, rev_tables, rev_thr, counts, members, member_counts, offers, bloom, stats,
@@ -1537,7 +1541,7 @@ struct NndCtx {
 };
 
 bool nnd_degree_supported(uint32_t knn_degree) {
-    return knn_degree <= 128 && nnd_width(knn_degree) <= kMaxWidth && nnd_width(static_cast<uint32_t>(1.5 * knn_degree)) / 32 <= 8;   // Bloom filter within 128 words
+    return knn_degree <= 256 && nnd_width(knn_degree) <= kMaxWidth && nnd_width(static_cast<uint32_t>(1.5 * knn_degree)) / 32 <= 16;   // Bloom filter within 256 words
 }
 
 int nnd_context(NndCtx& c, uint32_t reorder_num, uint32_t dim, const uint32_t* segment_starts, const uint32_t* segment_lengths,
@@ -1627,13 +1631,19 @@ int nnd_merge(const NndCtx& c, bool with_stats, bool scatter_reverse = false) {
     MergeArgs ma{c.list_ids, c.list_dists, c.offers, c.bloom, c.fwd_new, c.fwd_old, c.counts, with_stats ? c.stats : nullptr, c.segs,
                  scatter_reverse ? c.rev_new : nullptr, scatter_reverse ? c.rev_old : nullptr, scatter_reverse ? c.rev_tables : nullptr, c.rev_thr, c.norms,
                  c.n, c.l.width, c.l.width / kSamples, c.l.bloom_sets};
+    // The kernel is chosen by the keys of its second sort (list + 32 offers) and by the node's Bloom filter, which the
+    // forms up to 256 keys hold in 128 words of LDS: degrees 129 .. 170 have lists of 224 entries but filters of 160 words.
     const uint32_t m = c.l.width + kSamples;
-    if (m <= 64)
+    const bool small_filter = c.l.bloom_sets * 16 <= 128;
+    if (c.l.bloom_sets * 16 > 256 || m > 512) return GLIDE_ERR_UNSUPPORTED;   // nnd_degree_supported keeps such degrees out
+    if (m <= 64 && small_filter)
         hipLaunchKernelGGL((nnd_merge_kernel<64, kOfferSlotsNarrow>), dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
-    else if (m <= 128)
+    else if (m <= 128 && small_filter)
         hipLaunchKernelGGL((nnd_merge_kernel<128, kOfferSlotsWide>), dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
-    else
+    else if (m <= 256 && small_filter)
         hipLaunchKernelGGL((nnd_merge_kernel<256, kOfferSlotsWide>), dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
+    else
+        hipLaunchKernelGGL((nnd_merge_kernel<512, kOfferSlotsWide>), dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, ma);
     return launch_status();
 }
 
@@ -1649,8 +1659,10 @@ int nnd_finalize(const NndCtx& c, uint32_t knn_degree, uint32_t* knn_graph, unsi
         hipLaunchKernelGGL(nnd_finalize_kernel<64>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, knn_degree, c.segs, knn_graph);
     else if (c.l.width <= 128)
         hipLaunchKernelGGL(nnd_finalize_kernel<128>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, knn_degree, c.segs, knn_graph);
-    else
+    else if (c.l.width <= 256)
         hipLaunchKernelGGL(nnd_finalize_kernel<256>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, knn_degree, c.segs, knn_graph);
+    else
+        hipLaunchKernelGGL(nnd_finalize_kernel<512>, dim3(ceil_div(c.n, 4)), dim3(256), 0, c.s, c.list_ids, c.list_dists, c.n, c.l.width, knn_degree, c.segs, knn_graph);
     if (stats_out) hipLaunchKernelGGL(nnd_stats_reduce_kernel, dim3(1), dim3(1024), 0, c.s, c.stats, stats_out);
     return launch_status();
 }

@@ -154,7 +154,8 @@ int glide_hip_kmeans_fit(const float *sample, uint32_t sample_num, uint32_t dim,
  * rests.  At most 2048 partitions.
  * stats_out (nullable, 2 device u64): distinct offers the merge steps found in the offer tables; offers that stayed
  * away because their target had announced a distance threshold (see `offers` and `norms` below).
- * Limits: knn_degree <= 128 (list width round_up32(1.3 * knn_degree) <= 192 = six sub-lists, Bloom filter <= 4096 bits),
+ * Limits: knn_degree <= 256, the widest degree the build searches that read the kNN graph take (list width
+ * round_up32(1.3 * knn_degree) <= 352 = eleven sub-lists, Bloom filter <= 8192 bits),
  * dim % 4 == 0, reorder_num < 2^26 and reorder_num * list width < 2^32 per call (the large path calls it partition by
  * partition).  Two builds with the same inputs and seed give the same graph: nothing depends on the order in which
  * atomic operations arrive. */

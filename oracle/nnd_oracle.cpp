@@ -414,7 +414,7 @@ extern "C" int go_nnd_build_ex(const float *reorder_data, uint32_t reorder_num, 
 #ifdef _OPENMP
     if (threads > 0) omp_set_num_threads(threads);
 #endif
-    if (knn_degree == 0 || knn_degree > 128) return -1;
+    if (knn_degree == 0 || knn_degree > 256) return -1;
     // preprocess_data_kernel nn_descent.cuh:445-488: rows stored as halfs, squared norms taken from the fp32 input
     std::vector<float> half(static_cast<size_t>(reorder_num) * dim), norms(reorder_num);
 #pragma omp parallel for schedule(static)
@@ -447,7 +447,7 @@ extern "C" int go_nnd_build_from(const float *reorder_data, uint32_t reorder_num
 #ifdef _OPENMP
     if (threads > 0) omp_set_num_threads(threads);
 #endif
-    if (knn_degree == 0 || knn_degree > 128 || !start_lists) return -1;
+    if (knn_degree == 0 || knn_degree > 256 || !start_lists) return -1;
     const uint32_t W = go_nnd_extended_degree(knn_degree);
     std::vector<float> half(static_cast<size_t>(reorder_num) * dim), norms(reorder_num);
 #pragma omp parallel for schedule(static)
@@ -490,7 +490,7 @@ extern "C" int go_nnd_build_shipped(const float *reorder_data, uint32_t reorder_
 #ifdef _OPENMP
     if (threads > 0) omp_set_num_threads(threads);
 #endif
-    if (knn_degree == 0 || knn_degree > 128) return -1;
+    if (knn_degree == 0 || knn_degree > 256) return -1;
     std::vector<float> half(static_cast<size_t>(reorder_num) * dim), norms(reorder_num);
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < static_cast<int64_t>(reorder_num); i++) {

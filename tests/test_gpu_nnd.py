@@ -121,17 +121,18 @@ def test_nnd_termination_threshold(hip):
 def test_nnd_rejects_unsupported(hip):
     d = hip.DeviceArray(1024, np.float32)
     with pytest.raises(hip.GlideHipError) as e:
-        hip.nnd_build(d, 8, 128, d, d, 1, 129, 1, 0.0, 0, d, d, 1 << 30)      # list width above 192 (six sub-lists)
+        hip.nnd_build(d, 8, 128, d, d, 1, 257, 1, 0.0, 0, d, d, 1 << 30)      # above the widest degree the build searches take
     assert e.value.code == -1
     with pytest.raises(hip.GlideHipError) as e:
         hip.nnd_build(d, 8, 128, d, d, 1, 32, 1, 0.0, 0, d, d, 16)      # workspace too small
     assert e.value.code == -2
 
 
-@pytest.mark.parametrize("dim,k", [(4, 8), (36, 16), (100, 32), (132, 48), (260, 64), (1024, 24), (128, 96), (64, 128)])
+@pytest.mark.parametrize("dim,k", [(4, 8), (36, 16), (100, 32), (132, 48), (260, 64), (1024, 24), (128, 96), (64, 128), (128, 160), (96, 256)])
 def test_nnd_shapes(hip, dim, k):
-    """Dimensions that are not a multiple of the 64-dim chunk of the join (or of 8) and list widths 32, 64, 96, 128 and 192
-    (the reference accepts any degree, nn_descent.cuh:1423-1430; its evaluation runs degree 96)."""
+    """Dimensions that are not a multiple of the 64-dim chunk of the join (or of 8) and list widths 32, 64, 96, 128, 192,
+    224 and 352 (the reference accepts any degree, nn_descent.cuh:1423-1430; its evaluation runs degree 96; the build
+    searches that read the kNN graph take degrees up to 256)."""
     data = lowdim_data(3000, dim, latent=min(8, dim), seed=dim)
     seg_len = np.array([1800, 1200], dtype=np.uint32)
     seg_start = np.array([0, 1800], dtype=np.uint32)
