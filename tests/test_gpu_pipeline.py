@@ -184,3 +184,53 @@ def test_pipeline_matches_cpu_pipeline(hip, name, gen, num, dim, parts, degree, 
         else:
             assert se <= 0.02
             assert abs(diff.mean()) <= 0.005 + 2 * se
+
+
+def test_pipeline_with_a_knn_degree_above_128(hip):
+    """kNN degree 160 end to end: NN-descent with lists of 224 entries (seven id-keyed sub-lists, the merge step's widest
+    form), then the build searches over kNN rows of 160 ids (the two-half candidate sort).  From the GPU's kNN graph the
+    later stages are deterministic: the finished graph and the search results must be the CPU oracle's, bit for bit."""
+    from conftest import lowdim_data
+    from glide_amd import datasets as D, index as G
+    from oracle import oracle as O
+    num, dim, nq, parts, degree, knn_degree = 6000, 128, 200, 3, 32, 160
+    data, queries = lowdim_data(num, dim, seed=81), lowdim_data(nq, dim, seed=82)
+    pp = G.PartitionParameter(centroid_num=parts, boundary_factor=1.04, sample_factor=0.05, metric=0)
+    d_re, d_map, h_start, h_len, d_cent = G.preprocess(pp, hip.DeviceArray.from_numpy(data))
+    centroids, rdata, h_map = d_cent.numpy(), d_re.numpy(), d_map.numpy()
+    d_knn = G.build_nnd(G.NNDescentParameter(graph_degree=knn_degree, max_iterations=10, seed=0, termination_threshold=0.0), d_re, h_start, h_len)
+    knn = d_knn.numpy()
+    assert knn.shape == (rdata.shape[0], knn_degree)
+    for s, l in zip(h_start.tolist(), h_len.tolist()):
+        if l > 2 * knn_degree:
+            rows = knn[s:s + l]
+            assert (rows < l).all() and (np.sort(rows, axis=1)[:, 1:] != np.sort(rows, axis=1)[:, :-1]).all()      # local ids, no id twice
+    s, l = int(h_start[0]), int(h_len[0])
+    gt, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + 200], 32, exclude_self=True)
+    # at most 32 offers a round enter a list of 224 slots: after 10 rounds even its near end is still settling, in the
+    # CPU restatement alike, which is the bar
+    cpu = O.nnd_build(rdata, h_start, h_len, knn_degree, 10).astype(np.uint32)
+    r_gpu, r_cpu = D.recall(knn[s:s + 200, :32], gt, 32), D.recall(cpu[s:s + 200, :32], gt, 32)
+    print("recall@32 of the first 32 of 160: gpu %.4f cpu restatement %.4f" % (r_gpu, r_cpu), flush=True)
+    assert r_gpu >= 0.85 and r_gpu >= r_cpu - 0.01
+
+    index = G.GLIDE(degree, data, centroids, 0)
+    bp = G.IndexParameter(graph_degree=degree, knn_degree=knn_degree, relaxant_factor=1.05)
+    sp_b, sp_r = G.make_search_parameter(64, knn_degree), G.make_search_parameter(128, knn_degree)
+    local_sp, start_points = index.start_point_select(h_start, h_len, h_map, bp.seed)
+    index.build(bp, sp_b, sp_r, d_knn, h_start, h_len, d_map, d_re)
+    graph = index.d_graph.numpy()
+    ps = O.search_params(64, knn_degree)
+    g, _ = O.build_subgraph(rdata, num, knn, h_map, h_start, h_len, local_sp, degree, ps, 1.05, 0)
+    if rdata.shape[0] > num:
+        g, _ = O.build_boundary(rdata, num, knn, h_map, int(local_sp[parts]), g, ps, 1.05, 0)
+    g = O.reverse_edges(g)
+    g, _ = O.refine(data, g, centroids, start_points, O.search_params(128, knn_degree), 1.05, 0)
+    assert np.array_equal(g, graph)
+    sp = G.make_search_parameter(64, degree, 10)
+    ids, dists = index.search(sp, hip.DeviceArray.from_numpy(queries))
+    e_ids, e_dists, _ = O.search(data, graph, centroids, start_points, queries, 10, sp.beam, sp.max_iterations, sp.min_iterations,
+                                 sp.hash_bit, sp.hash_reset_interval, 0)
+    assert np.array_equal(ids, e_ids) and np.array_equal(dists, e_dists)
+    truth, _ = O.bruteforce_knn(data, queries, 10)
+    assert D.recall(ids, truth, 10) >= 0.95
