@@ -103,7 +103,7 @@ __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float
     // Steps in flight.  Rows of more than 512 dims are 2-4 KB each and a step holds only two of them: with one step in
     // flight a wavefront had 8 KB on its way, too little to cover the memory latency when a launch has about one
     // wavefront per SIMD (1 000 queries); four steps took the 960-dim beam-512 search from 16.8 to 13.2 ms.
-    constexpr int U = DIMV == 8 ? 4 : 2;   // rows of up to 2048 dims (DIMV 16) take 64 registers each: two steps
+    constexpr int U = DIMV == 8 ? 4 : 2;   // rows of more than 1024 dims (DIMV 16, 32) take 64 registers a lane each: two steps
     score_share<DIMV, U>(RefInRegs<DIMV>{ref}, data, dim, metric, first, count, lane, 0u, 1u, id_of, out);
 }
 

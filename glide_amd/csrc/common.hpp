@@ -136,11 +136,12 @@ __device__ __forceinline__ uint32_t hash_insert(uint32_t* table, uint32_t bitlen
 // serves 64/LPR rows.  DIMV selects the shape by row length (dim <= 128*DIMV):
 //   DIMV 1: 8 lanes x 4 loads (8 rows per wavefront)    DIMV 2: 16 lanes x 4 loads (4 rows)
 //   DIMV 4: 32 lanes x 4 loads (2 rows)                 DIMV 8 / 16: 32 lanes x 8 / 16 loads (2 rows)
+//   DIMV 32: 64 lanes x 16 loads (1 row; up to 4096 dims)
 template <int DIMV>
 struct RowShape {
-    static_assert(DIMV == 1 || DIMV == 2 || DIMV == 4 || DIMV == 8 || DIMV == 16, "row shape");
-    static constexpr int LPR = DIMV == 1 ? 8 : (DIMV == 2 ? 16 : 32);
-    static constexpr int NV = DIMV == 16 ? 16 : (DIMV == 8 ? 8 : 4);
+    static_assert(DIMV == 1 || DIMV == 2 || DIMV == 4 || DIMV == 8 || DIMV == 16 || DIMV == 32, "row shape");
+    static constexpr int LPR = DIMV == 1 ? 8 : (DIMV == 2 ? 16 : (DIMV == 32 ? 64 : 32));
+    static constexpr int NV = DIMV >= 16 ? 16 : (DIMV == 8 ? 8 : 4);
     static constexpr int ROWS = 64 / LPR;
     static __device__ __forceinline__ int lane_in_row(int lane) { return lane & (LPR - 1); }
     static __device__ __forceinline__ int row_of_lane(int lane) { return lane / LPR; }
@@ -187,6 +188,7 @@ __device__ __forceinline__ float row_sum(float v) {
     if constexpr (RowShape<DIMV>::LPR >= 16)
         v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));  // row_mirror
     if constexpr (RowShape<DIMV>::LPR >= 32) v += lane_xor<16>(v);
+    if constexpr (RowShape<DIMV>::LPR >= 64) v += lane_xor<32>(v);
     return v;
 }
 

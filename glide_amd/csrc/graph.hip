@@ -295,7 +295,8 @@ build_fn pick_build_dim(uint32_t dim) {
     if (dim <= 256) return build_kernel<MAX_CAND, MAX_BEAM, 2>;
     if (dim <= 512) return build_kernel<MAX_CAND, MAX_BEAM, 4>;
     if (dim <= 1024) return build_kernel<MAX_CAND, MAX_BEAM, 8>;
-    return build_kernel<MAX_CAND, MAX_BEAM, 16>;
+    if (dim <= 2048) return build_kernel<MAX_CAND, MAX_BEAM, 16>;
+    return build_kernel<MAX_CAND, MAX_BEAM, 32>;
 }
 template <int MAX_CAND>
 build_fn pick_build_beam(uint32_t beam, uint32_t dim) {
@@ -310,7 +311,8 @@ refine_fn pick_refine_dim(uint32_t dim) {
     if (dim <= 256) return refine_kernel<MAX_CAND, MAX_BEAM, 2>;
     if (dim <= 512) return refine_kernel<MAX_CAND, MAX_BEAM, 4>;
     if (dim <= 1024) return refine_kernel<MAX_CAND, MAX_BEAM, 8>;
-    return refine_kernel<MAX_CAND, MAX_BEAM, 16>;
+    if (dim <= 2048) return refine_kernel<MAX_CAND, MAX_BEAM, 16>;
+    return refine_kernel<MAX_CAND, MAX_BEAM, 32>;
 }
 template <int MAX_CAND>
 refine_fn pick_refine_beam(uint32_t beam, uint32_t dim) {
@@ -336,7 +338,7 @@ size_t prune_lds_bytes_refine(uint32_t beam, uint32_t degree) {
 int check_beam_sizes(uint32_t degree, uint32_t graph_degree, uint32_t beam, uint32_t dim, uint32_t hash_bit, int metric) {
     if (degree == 0 || graph_degree == 0 || beam == 0 || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
-    if (degree > kMaxDegree || graph_degree > kMaxDegree || beam > 512 || dim % 4 != 0 || dim > 2048 || hash_bit < 1 || hash_bit > 13)
+    if (degree > kMaxDegree || graph_degree > kMaxDegree || beam > 512 || dim % 4 != 0 || dim > 4096 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     return GLIDE_OK;
 }

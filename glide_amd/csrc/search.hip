@@ -84,7 +84,7 @@ constexpr int kTeam = 4;
 
 template <int DIMV>
 struct TeamShape {
-    static constexpr int U = DIMV == 16 ? 1 : (DIMV == 8 ? 2 : 4);   // row steps in flight per wavefront: 64 row registers either way
+    static constexpr int U = DIMV >= 16 ? 1 : (DIMV == 8 ? 2 : 4);   // row steps in flight per wavefront: 64 row registers either way
     static constexpr size_t query_bytes = sizeof(float4) * RowShape<DIMV>::NV * RowShape<DIMV>::LPR;
 };
 
@@ -476,7 +476,8 @@ sub_fn pick_sub_dim(uint32_t dim) {
     if (dim <= 256) return search_sub_kernel<MAX_CAND, MAX_BEAM, 2, WHOLE>;
     if (dim <= 512) return search_sub_kernel<MAX_CAND, MAX_BEAM, 4, WHOLE>;
     if (dim <= 1024) return search_sub_kernel<MAX_CAND, MAX_BEAM, 8, WHOLE>;
-    return search_sub_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
+    if (dim <= 2048) return search_sub_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
+    return search_sub_kernel<MAX_CAND, MAX_BEAM, 32, WHOLE>;
 }
 template <int MAX_CAND>
 sub_fn pick_sub_beam(uint32_t beam, uint32_t dim) {
@@ -498,13 +499,15 @@ search_fn pick_dim(uint32_t dim) {
     if (dim <= 256) return search_kernel<MAX_CAND, MAX_BEAM, 2, WHOLE>;
     if (dim <= 512) return search_kernel<MAX_CAND, MAX_BEAM, 4, WHOLE>;
     if (dim <= 1024) return search_kernel<MAX_CAND, MAX_BEAM, 8, WHOLE>;
-    return search_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
+    if (dim <= 2048) return search_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
+    return search_kernel<MAX_CAND, MAX_BEAM, 32, WHOLE>;
 }
 template <int MAX_CAND, int MAX_BEAM, bool WHOLE = false>
 search_fn pick_team_dim(uint32_t dim) {
     if (dim <= 512) return search_team_kernel<MAX_CAND, MAX_BEAM, 4, WHOLE>;
     if (dim <= 1024) return search_team_kernel<MAX_CAND, MAX_BEAM, 8, WHOLE>;
-    return search_team_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
+    if (dim <= 2048) return search_team_kernel<MAX_CAND, MAX_BEAM, 16, WHOLE>;
+    return search_team_kernel<MAX_CAND, MAX_BEAM, 32, WHOLE>;
 }
 template <int MAX_CAND>
 search_fn pick_team_beam(uint32_t beam, uint32_t dim) {
@@ -561,7 +564,7 @@ int launch_search(const float* data, uint32_t num, uint32_t dim, const uint32_t*
         return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0) return GLIDE_OK;
-    if (graph_degree > 256 || beam > 512 || centroid_num > 256 || dim % 4 != 0 || dim > 2048 || top_k > beam ||
+    if (graph_degree > 256 || beam > 512 || centroid_num > 256 || dim % 4 != 0 || dim > 4096 || top_k > beam ||
         hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     if (reinterpret_cast<uintptr_t>(data) % 16 || reinterpret_cast<uintptr_t>(queries) % 16 ||
@@ -598,7 +601,7 @@ int launch_search(const float* data, uint32_t num, uint32_t dim, const uint32_t*
     else fn = graph_degree <= 64 ? pick_beam<64>(beam, dim) : graph_degree <= 128 ? pick_beam<128>(beam, dim) : pick_beam<256>(beam, dim);
     const size_t lds_bytes = beam_lds_bytes(graph_degree) + round_up32(centroid_num) * sizeof(float) +
                              (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam, beam == 512) +
-                             (team ? (dim <= 512 ? TeamShape<4>::query_bytes : dim <= 1024 ? TeamShape<8>::query_bytes : TeamShape<16>::query_bytes) + 16 : 0);
+                             (team ? (dim <= 512 ? TeamShape<4>::query_bytes : dim <= 1024 ? TeamShape<8>::query_bytes : dim <= 2048 ? TeamShape<16>::query_bytes : TeamShape<32>::query_bytes) + 16 : 0);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     if (team) hipLaunchKernelGGL(fn, dim3(query_num), dim3(64 * kTeam), lds_bytes, as_stream(stream), a);
     else hipLaunchKernelGGL(fn, dim3(balanced_grid(query_num, beam, lds_bytes)), dim3(64), lds_bytes, as_stream(stream), a);
@@ -653,7 +656,7 @@ int launch_search_sub(const float* segment_data, uint32_t dim, const uint32_t* s
     if (dim == 0 || graph_degree == 0 || centroid_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0 || (query_list && list_len == 0)) return GLIDE_OK;
-    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 2048 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
+    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 4096 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;   // top_k buckets: kernel_config.cuh:312-323
     SubArgs a;
     a.data = segment_data;
@@ -764,7 +767,7 @@ extern "C" int glide_hip_search_partitions(const float* data, uint32_t dim, cons
     if (dim == 0 || graph_degree == 0 || segment_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0) return GLIDE_OK;
-    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 2048 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
+    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 4096 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     if (static_cast<unsigned long long>(query_num) * segment_num >= 0xffffffffull) return GLIDE_ERR_UNSUPPORTED;   // pairs are numbered with 32 bits
     const PartitionSearchLayout l = partition_search_layout(query_num, segment_num, top_k);

@@ -67,7 +67,7 @@ int glide_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* synchroni
  * kernel adds {beam iterations, data rows scored, graph rows read} into the stripe of each workgroup (one shared
  * address would serialise the launch); the sums over the stripes are the algorithmic-traffic tallies.
  * Limits (reference kernel_config.cuh:41-60): graph_degree <= 256, beam <= 512, centroid_num <= 256, dim % 4 == 0,
- * dim <= 2048, top_k <= beam.  Degrees above 128 and beams above 256 run the candidate sort / beam merge as two
+ * dim <= 4096, top_k <= beam.  Degrees above 128 and beams above 256 run the candidate sort / beam merge as two
  * half-wave networks, as the reference's two-warp branches do (search_kernel.cuh:38-94, :149-232). */
 int glide_hip_search(const float *data, uint32_t num, uint32_t dim, const uint32_t *graph, uint32_t graph_degree,
                      const float *centroids, uint32_t centroid_num, const uint32_t *start_points,
@@ -245,7 +245,7 @@ int glide_hip_nnd_finalize(uint32_t reorder_num, uint32_t dim, const uint32_t *s
 
 /* ---- graph construction (subsystem 3) ----------------------------------------------------------------------
  * All kernels give one point to one wavefront.  Limits as for glide_hip_search (knn_degree, graph_degree <= 256,
- * beam <= 512, dim % 4 == 0, dim <= 2048).  `counters` as in glide_hip_search (prune distances count as rows). */
+ * beam <= 512, dim % 4 == 0, dim <= 4096).  `counters` as in glide_hip_search (prune distances count as rows). */
 
 /* Replaces build_kernel (graph_kernel.cuh:249-316) as launched by GLIDE::subgraph_build_and_merge
  * (glide_impl.cuh:77-147): for every reorder id p < num, beam search on the partition-local kNN graph from the

@@ -10,7 +10,7 @@ INV = 0xFFFFFFFF
 
 def _cases():
     rng = np.random.default_rng(777)
-    dims = [4, 36, 128, 132, 256, 512, 960, 1536, 2048]
+    dims = [4, 36, 128, 132, 256, 512, 960, 1536, 2048, 3072, 4096]
     degrees = [8, 24, 32, 64, 96, 160]
     beams = [32, 64, 128, 256, 320]
     out = []

@@ -86,7 +86,7 @@ def test_nnd_k64_cosine_dim96(hip):
     assert r >= 0.93
 
 
-@pytest.mark.parametrize("dim", [960, 2048])
+@pytest.mark.parametrize("dim", [960, 2048, 4096])
 def test_nnd_long_rows(hip, dim):
     """Rows of 960 dims and of the longest length the beam kernels take, against the CPU restatement."""
     from oracle import oracle as O

@@ -98,7 +98,7 @@ def test_search_degree64_dim960(hip):
         assert np.array_equal(gids, eids) and np.array_equal(gdists, edists)
 
 
-@pytest.mark.parametrize("dim,deg", [(960, 64), (384, 32), (1024, 160), (1536, 32), (2048, 64)])
+@pytest.mark.parametrize("dim,deg", [(960, 64), (384, 32), (1024, 160), (1536, 32), (2048, 64), (3072, 32), (4096, 64)])
 def test_long_rows_small_and_large_batches_agree(hip, dim, deg):
     """Rows of more than 256 dims are searched by a team of four wavefronts per query while the batch is small and by one
     wavefront per query once it fills the chip; both forms must give the oracle's ids, distances and counters (integer
@@ -188,7 +188,7 @@ def test_search_rejects_unsupported_sizes(hip):
     base = dict(data=d, num=8, dim=128, graph=d, graph_degree=32, centroids=d, centroid_num=2, start_points=d, queries=d,
                 query_num=1, top_k=10, beam=64, max_iterations=10, min_iterations=0, hash_bit=8, hash_reset_interval=2,
                 metric=0, result_ids=d, result_dists=d)
-    for key, bad in (("beam", 544), ("graph_degree", 257), ("centroid_num", 300), ("dim", 130), ("dim", 2052), ("top_k", 65)):
+    for key, bad in (("beam", 544), ("graph_degree", 257), ("centroid_num", 300), ("dim", 130), ("dim", 4100), ("top_k", 65)):
         with pytest.raises(hip.GlideHipError) as e:
             hip.search(**{**base, key: bad})
         assert e.value.code == -1, key
