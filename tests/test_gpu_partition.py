@@ -32,7 +32,8 @@ def gpu_assign(hip, data, centroids, bf, metric=0):
                                             (3000, 128, 100, 0), (2500, 32, 200, 0), (1500, 960, 16, 0), (100, 128, 3, 0),
                                             (1000, 4, 7, 0), (1200, 36, 33, 0), (900, 1024, 256, 0), (700, 132, 64, 1),
                                             # at most 32 centroids of at most 128 dims: the kernel that keeps the centroids in LDS
-                                            (2222, 100, 32, 0), (1800, 64, 31, 0), (1300, 36, 2, 1), (4100, 124, 17, 0)])
+                                            (2222, 100, 32, 0), (1800, 64, 31, 0), (1300, 36, 2, 1), (4100, 124, 17, 0),
+                                            (800, 4096, 24, 0), (600, 3072, 40, 1)])
 def test_assign_matches_oracle(hip, n, dim, c, metric):
     from oracle import oracle as O
     data = lowdim_float_data(n, dim, seed=n) if metric == 1 else lowdim_data(n, dim, seed=n)

@@ -32,12 +32,14 @@ def test_copy_rows(hip, src_dim, dst_dim):
     hip.copy_rows(d_src, 0, src_dim, d_dst, dst_dim)      # no rows: nothing launched
 
 
-@pytest.mark.parametrize("dim", [25, 50, 101])
+@pytest.mark.parametrize("dim", [25, 50, 101, 3070])      # 3070: held as 3072, the row shape with a whole wavefront per row
 def test_pipeline_on_rows_of_any_length(hip, dim):
     from glide_amd import datasets as D, index as G
     from oracle import oracle as O
-    num, nq, parts, degree = 6000, 200, 3, 32
+    num, nq, parts, degree = (6000, 200, 3, 32) if dim < 1024 else (3000, 100, 3, 32)
     data, queries = lowdim_data(num, dim, seed=71), lowdim_data(nq, dim, seed=72)
+    if dim > 1024:      # values 0..8, so that sums of 3070 squared differences stay exact in float32
+        data, queries = np.rint(data / 32), np.rint(queries / 32)
     print("dim", dim, flush=True)
     held = (dim + 3) // 4 * 4
 
@@ -58,7 +60,7 @@ def test_pipeline_on_rows_of_any_length(hip, dim):
     knn = d_knn.numpy()
     s, l = int(h_start[0]), int(h_len[0])
     gt, _ = O.bruteforce_knn(rdata[s:s + l], rdata[s:s + 200], 32, exclude_self=True)
-    assert D.recall(knn[s:s + 200], gt, 32) >= 0.95
+    assert D.recall(knn[s:s + 200], gt, 32) >= (0.95 if dim < 1024 else 0.8)      # coarse values: many equal distances
 
     index = G.GLIDE(degree, data, centroids, 0)              # points and centroids in their own length: held padded
     assert index.dim() == held
@@ -84,6 +86,6 @@ def test_pipeline_on_rows_of_any_length(hip, dim):
                                      sp.hash_bit, sp.hash_reset_interval, 0)
         assert np.array_equal(ids, e_ids) and np.array_equal(dists, e_dists), beam
     truth, _ = O.bruteforce_knn(data, queries, 10)
-    assert D.recall(ids, truth, 10) >= 0.95
+    assert D.recall(ids, truth, 10) >= (0.95 if dim < 1024 else 0.8)
     with pytest.raises(ValueError):
         index.search(sp, hip.DeviceArray.from_numpy(queries[:, :dim - 4]))
