@@ -92,3 +92,41 @@ def test_degenerate_partitions_through_every_stage(boundary_factor):
     e_ids, e_d, _ = O.search(data, e_ref, centroids, start_points, queries, 10, **ssp)
     g_ids, g_d, _ = run_gpu_search(hip, data, e_ref, centroids, start_points, queries, 10, ssp)
     assert np.array_equal(g_ids, e_ids) and np.array_equal(g_d, e_d)
+
+
+def test_empty_inputs_are_no_ops():
+    """No points / no queries: every stage returns without touching its outputs (the partition stage reports zero
+    lengths), as a loop over nothing would; sentinels in the output buffers stay where they are."""
+    from glide_amd import capi as hip
+    from oracle import oracle as O
+    hip.set_device(0)
+    dim, c, D, K = 32, 3, 16, 16
+    buf = lambda shape, dtype=np.uint32: hip.DeviceArray.full(shape, 7, dtype)
+    d_rows, d_cent = hip.DeviceArray.from_numpy(lowdim_data(64, dim, seed=1)), hip.DeviceArray.from_numpy(lowdim_data(c, dim, seed=2))
+    sp = O.search_params(64, K)
+    beam_args = (sp["beam"], sp["max_iterations"], sp["min_iterations"], sp["hash_bit"], sp["hash_reset_interval"])
+
+    d_idx, d_len = buf((8, 3)), buf(c + 1)
+    wb = hip.partition_assign_workspace_bytes(8, c)
+    ws = hip.DeviceArray(wb // 4 + 1, np.uint32)
+    hip.partition_assign(d_rows, 0, dim, d_cent, c, 1.04, 0, d_idx, d_len, None, ws, wb)
+    hip.synchronize()
+    assert not d_len.numpy().any() and (d_idx.numpy() == 7).all()
+
+    d_re, d_map, d_starts = buf((8, dim), np.float32), buf(8), hip.DeviceArray.from_numpy(np.zeros(c + 1, np.uint32))
+    hip.reorder(d_rows, 0, dim, d_idx, d_starts, d_re, d_map)
+    hip.sample_rows(d_rows, dim, d_map, 0, d_re)
+
+    d_knn, d_graph, d_out, d_cnt, d_sp = buf((8, K)), buf((8, D)), buf((8, D)), buf(8), hip.DeviceArray.from_numpy(np.zeros(c + 1, np.uint32))
+    hip.build_subgraph(d_rows, 0, dim, d_knn, K, d_map, d_starts, d_starts, c + 1, d_sp, D, *beam_args, 1.05, 0, d_graph, None)
+    wb = hip.reverse_edges_workspace_bytes(8, D)
+    hip.reverse_edges(d_graph, 0, D, d_out, d_cnt, hip.DeviceArray(wb // 8 + 1, np.uint64), wb)
+    hip.insert_reverse(d_graph, d_out, d_cnt, 0, D)
+    hip.refine(d_rows, 0, dim, d_graph, d_out, D, d_cent, c, d_sp, *beam_args, 1.05, 0)
+    d_ids = buf((4, c))
+    hip.select_segments(d_rows, 0, dim, d_cent, c, 2, 1.1, 0, d_ids)
+    res_i, res_d = buf((4, 10)), buf((4, 10), np.float32)
+    hip.search(d_rows, 64, dim, d_graph, D, d_cent, c, d_sp, d_rows, 0, 10, *beam_args, 0, res_i, res_d)
+    hip.synchronize()
+    for d in (d_re, d_map, d_graph, d_out, d_cnt, d_ids, res_i, res_d):
+        assert (d.numpy() == 7).all()
