@@ -131,10 +131,11 @@ def test_long_rows_small_and_large_batches_agree(hip, dim, deg):
 
 @pytest.mark.parametrize("deg", [32, 64])
 def test_wide_beams_on_distinct_keys(hip, deg):
-    """Beams above 256 insert a few entering candidates by rank instead of running candidate sort and two-half merge when
-    every key involved is distinct.  Points on a line and queries beyond its ends make all distances of a search distinct
-    (and exact), so that path does the merging here; ids, distances and counters must be the oracle's.  A second data
-    set repeats every position once: beams with equal keys, where the networks must take over."""
+    """Beams of 288 to 480 insert a few entering candidates by rank instead of running candidate sort and two-half merge
+    when every key involved is distinct.  Points on a line and queries beyond its ends make all distances of a search
+    distinct (and exact), so that path does the merging here; ids, distances and counters must be the oracle's.  A second
+    data set repeats every position once: beams with equal keys, where the networks must take over.  Beam 512 runs the
+    kernel form that merges the whole beam in its registers, on the same two data sets."""
     from oracle import oracle as O
     rng = np.random.default_rng(deg)
     n = 3000
