@@ -31,13 +31,15 @@ struct BeamLds {  // per-wave LDS (the hash table follows, 1 << hash_bit words)
     uint32_t vlist[MAX_CAND];
 };
 
-// Host-side sizes of the dynamic LDS regions: the candidate lists for a degree bucket, and the staging area that the
-// beam merges of beams above 256 keep behind the hash table: 512 + 4 distances, as many ids, the turning points.
+// Beams the kernels take: up to 512 (the reference's widest bucket, kernel_config.cuh:41-48); above 256 a multiple of 16, so
+// that each half of the beam is whole lanes of eight entries (the reference's adjust_search_params, params.cuh:82-99, only
+// ever hands out multiples of 32).
+inline bool beam_supported(uint32_t beam) { return beam <= 512 && (beam <= 256 || beam % 16 == 0); }
+
+// Host-side size of the candidate lists for a degree bucket (the hash table follows them in the dynamic LDS).
 inline size_t beam_lds_bytes(uint32_t degree) {
     return degree <= 64 ? sizeof(BeamLds<64>) : degree <= 128 ? sizeof(BeamLds<128>) : sizeof(BeamLds<256>);
 }
-// A kernel that merges the whole of the widest beam in its registers (Beam<..., WHOLE>) stages nothing.
-inline size_t beam_stage_bytes(uint32_t beam, bool whole = false) { return beam > 256 && !whole ? (2 * (512 + 4) + 4) * sizeof(uint32_t) : 0; }
 
 __device__ __forceinline__ void wave_sync() { __syncthreads(); }  // workgroup == one wavefront
 // The same point in a wavefront that shares its workgroup with others (TEAM): a workgroup barrier would wait for them.
@@ -108,8 +110,8 @@ __device__ __forceinline__ void score_list(const RowRegs<DIMV>& ref, const float
 }
 
 // TEAM: the beam's wavefront is one of several in its workgroup (the others only score rows, see search_team_kernel).
-// WHOLE: the host promises beam == MAX_BEAM (asked for beams above 256 only, i.e. beam 512): the beam merge then stays in
-// the registers (merge_beam_full), and a kernel without the staged two-half merge needs 126 registers instead of 161.
+// WHOLE: the host promises beam == MAX_BEAM (asked for beams above 256 only, i.e. beam 512): the two-half merge of such a
+// beam needs no lane permutations (merge_beam_full), and the kernel 112 registers instead of 128.
 template <int MAX_CAND, int MAX_BEAM, int DIMV, bool TEAM = false, bool WHOLE = false>
 struct Beam {
     static_assert(!WHOLE || MAX_BEAM > 256, "beams up to 256 merge in the registers anyway");
@@ -123,23 +125,16 @@ struct Beam {
     RowRegs<DIMV> q;
     BeamLds<MAX_CAND>* lds;
     uint32_t* hash;
-    float* stage_dist;       // MAX_BEAM > 256 only: LDS copy of the beam for the two-warp merge (follows the hash table)
-    uint32_t* stage_id;
-    uint32_t* stage_ws;
     BeamParams p;
     BeamCounters cnt;
     int lane;
     uint32_t last_scored;   // rows scored by the latest expansion (wave-uniform)
-    uint32_t ranked_pause;  // beams above 256: merges left before the ranked insertion is tried again (wave-uniform)
 
     __device__ __forceinline__ void init(BeamLds<MAX_CAND>* lds_, uint32_t* hash_, const BeamParams& p_, const float* query) {
         lds = lds_;
         hash = hash_;
         p = p_;
         lane = lane_id();
-        stage_dist = reinterpret_cast<float*>(hash_ + (size_t{1} << p_.hash_bit));
-        stage_id = reinterpret_cast<uint32_t*>(stage_dist + MAX_BEAM + 4);
-        stage_ws = stage_id + MAX_BEAM + 4;
         load_row<DIMV>(q, query, p.dim, RowShape<DIMV>::lane_in_row(lane));
         hash_clear(hash, p.hash_bit, lane);
         wave_sync();
@@ -303,89 +298,6 @@ struct Beam {
         wave_sync();
     }
 
-    // Beam merge for beams above 256 (reference two-warp branch of sort_for_beam, search_kernel.cuh:149-232), on a copy
-    // of the beam in LDS: candidates displace larger entries from the tail, the two halves are compare-exchanged
-    // element by element, the smallest touched index of each half is tracked, and each 32-lane half of the wavefront
-    // merges one half of the beam laid out as [untouched prefix | padding | touched rest].  Returns false when no
-    // candidate entered (the beam is unchanged).
-    __device__ __forceinline__ bool merge_beam_two() {
-        constexpr int PER = MAX_BEAM / 2, N = PER / 32;
-        float* sd = stage_dist;
-        uint32_t* si = stage_id;
-        const uint32_t half = p.beam / 2;
-#pragma unroll
-        for (int r = 0; r < NB; r++) {
-            sd[NB * lane + r] = bk[r];
-            si[NB * lane + r] = bv[r];
-        }
-        if (lane < 3) stage_ws[lane] = half;
-        wave_sync();
-        bool replaced = false;
-        const uint32_t limit = p.degree < p.beam ? p.degree : p.beam;
-        for (uint32_t k = lane; k < limit; k += kWave) {
-            const uint32_t j = p.beam - 1 - k;
-            const float c = lds->cand_dist[k];
-            if (sd[j] > c) {
-                sd[j] = c;
-                si[j] = lds->cand_id[k];
-                if (j < half) atomicMin(&stage_ws[2], j);
-                else atomicMin(&stage_ws[1], j - half);
-                replaced = true;
-            }
-        }
-        if (ballot(replaced) == 0) return false;
-        wave_sync();
-        for (uint32_t j = lane; j < half; j += kWave) {
-            const uint32_t k = j + half;
-            const float k0 = sd[j], k1 = sd[k];
-            if (k0 > k1) {
-                sd[j] = k1;
-                sd[k] = k0;
-                const uint32_t v0 = si[j];
-                si[j] = si[k];
-                si[k] = v0;
-                atomicMin(&stage_ws[0], j);
-            }
-        }
-        wave_sync();
-        if (lane == 0 && stage_ws[2] < half) stage_ws[1] = stage_ws[2];
-        wave_sync();
-        const uint32_t w = lane >> 5, l = lane & 31;
-        const uint32_t turning = stage_ws[w];
-        float key[N];
-        uint32_t val[N];
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            uint32_t k = p.beam, j = N * l + i;
-            if (j < turning) {
-                k = j + half * w;
-            } else if (j >= PER - half) {
-                j -= PER - half;
-                if (turning <= j && j < half) k = j + half * w;
-            }
-            key[i] = k < p.beam ? sd[k] : FLT_MAX;
-            val[i] = k < p.beam ? si[k] : kInvalid;
-        }
-        wave_sync();
-        WaveNet<PER, 32>::merge(key, val, lane);
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            const uint32_t j = N * l + i;
-            if (j < half) {
-                sd[j + half * w] = key[i];
-                si[j + half * w] = val[i];
-            }
-        }
-        wave_sync();
-#pragma unroll
-        for (int r = 0; r < NB; r++) {
-            const uint32_t e = NB * lane + r;
-            bk[r] = e < p.beam ? sd[e] : FLT_MAX;
-            bv[r] = e < p.beam ? si[e] : kInvalid;
-        }
-        return true;
-    }
-
     // v of the lane 32 places away: one swap of the 32-lane halves of a register pair and a select
     template <class T>
     static __device__ __forceinline__ T other_half(T v, bool upper) {
@@ -394,11 +306,11 @@ struct Beam {
         return __builtin_bit_cast(T, upper ? s[0] : s[1]);
     }
 
-    // The same merge for a beam of exactly MAX_BEAM entries, in the registers.  Element NB * lane + r puts the two halves
-    // of the beam into the two 32-lane halves of the wavefront, each in the order its merge network wants, so the
-    // compare-exchange between the halves is a swap of register halves; and with half == PER the layout
-    // [untouched prefix | padding | touched rest] of a half is the half as it stands, whatever the turning points are,
-    // so they are not tracked.  No copy of the beam through LDS, no LDS atomics, no waits between the steps.
+    // Beam merge for a beam of exactly MAX_BEAM entries (beams above 256; the general form follows).  Element
+    // NB * lane + r puts the two halves of the beam into the two 32-lane halves of the wavefront, each in the order its
+    // merge network wants, so the compare-exchange between the halves is a swap of register halves; and with
+    // half == PER the layout [untouched prefix | padding | touched rest] of a half is the half as it stands, whatever
+    // the turning points are, so they are not tracked.
     __device__ __forceinline__ void merge_beam_full() {
         bool replaced = false;
 #pragma unroll
@@ -427,6 +339,92 @@ struct Beam {
         WaveNet<MAX_BEAM / 2, 32>::merge(bk, bv, lane);
     }
 
+    // Beam merge for beams above 256 (reference two-warp branch of sort_for_beam, search_kernel.cuh:149-232), on the beam
+    // where it sits; beam a multiple of 16, so that a half is whole lanes.  Half 0 of the beam is in lanes [0, H), half 1
+    // in lanes [H, 2H) (H = half / NB), pads behind.  The reference's steps, each of which decides where equal keys end
+    // up: candidates displace larger entries from the tail (the smallest touched index of each half, its "turning
+    // point", is found with a ballot: indices grow with the lane), the halves are compare-exchanged entry by entry (a
+    // lane permutation: same register, lane +-H), each 32-lane half of the wavefront gathers its half of the beam as
+    // [untouched prefix | padding | touched rest] -- the source of position q is the same register of another lane,
+    // because half and PER - half are multiples of NB -- and merges it, and the beam gathers the results back.  Three
+    // lane permutations of the beam's registers; the reference copies the beam through shared memory and finds the
+    // turning points with atomics.
+    __device__ __forceinline__ void merge_beam_general() {
+        constexpr int PER = MAX_BEAM / 2;
+        constexpr uint32_t kNone = 0xffffffffu;
+        const uint32_t half = p.beam / 2, H = half / NB;
+        uint32_t first = kNone;            // this lane's smallest element index that a candidate replaced
+#pragma unroll
+        for (int r = NB - 1; r >= 0; r--) {
+            const uint32_t e = NB * lane + r;
+            const uint32_t k = p.beam - 1 - e;
+            if (e < p.beam && k < p.degree) {
+                const float c = lds->cand_dist[k];
+                if (bk[r] > c) {
+                    bk[r] = c;
+                    bv[r] = lds->cand_id[k];
+                    first = e;
+                }
+            }
+        }
+        const uint64_t touched = ballot(first != kNone);
+        if (touched == 0) return;
+        const uint64_t lanes0 = (1ull << H) - 1;
+        const uint64_t touched0 = touched & lanes0, touched1 = touched >> H;
+        const uint32_t t2 = touched0 ? read_lane(first, __builtin_ctzll(touched0)) : half;
+        uint32_t t1 = touched1 ? read_lane(first, static_cast<int>(H) + __builtin_ctzll(touched1)) - half : half;
+
+        // the halves against each other: entry j of half 0 and entry j of half 1 change places when the first is larger
+        const bool lower = static_cast<uint32_t>(lane) < H, upper = !lower && static_cast<uint32_t>(lane) < 2 * H;
+        const int partner = lower ? lane + static_cast<int>(H) : (upper ? lane - static_cast<int>(H) : lane);
+        uint32_t moved = kNone;
+#pragma unroll
+        for (int r = NB - 1; r >= 0; r--) {
+            const float ok = shfl_f32(bk[r], partner);
+            const uint32_t ov = shfl_u32(bv[r], partner);
+            const bool take = lower ? bk[r] > ok : (upper && ok > bk[r]);
+            if (take && lower) moved = NB * lane + r;
+            bk[r] = take ? ok : bk[r];
+            bv[r] = take ? ov : bv[r];
+            __builtin_amdgcn_sched_barrier(0);   // one register at a time (interleaved, the permutations of a step hold the beam twice)
+        }
+        const uint64_t movers = ballot(moved != kNone);
+        const uint32_t t0 = movers ? read_lane(moved, __builtin_ctzll(movers)) : half;
+        if (t2 < half) t1 = t2;
+
+        // each 32-lane half gathers its half of the beam as [untouched prefix | padding | touched rest]; register i of a
+        // position comes from register i of another lane, so the beam's registers are rewritten in place
+        const uint32_t w = static_cast<uint32_t>(lane) >> 5, l = static_cast<uint32_t>(lane) & 31;
+        const uint32_t turning = w ? t1 : t0;
+        const uint32_t gap = PER - half;                       // the rest sits `gap` positions further on
+        const int from_prefix = static_cast<int>(l + H * w), from_rest = static_cast<int>(l + H * w) - static_cast<int>(gap / NB);
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const uint32_t q = NB * l + i;
+            const bool in_prefix = q < turning;
+            const bool in_rest = q >= gap && q - gap >= turning;     // q - gap < half holds for every q < PER
+            const int src = in_prefix ? from_prefix : (in_rest ? from_rest : lane);
+            const float k = shfl_f32(bk[i], src);
+            const uint32_t v = shfl_u32(bv[i], src);
+            bk[i] = in_prefix || in_rest ? k : FLT_MAX;
+            bv[i] = in_prefix || in_rest ? v : kInvalid;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        WaveNet<PER, 32>::merge(bk, bv, lane);
+        // back into beam order: the first `half` positions of half-wave w are elements [half * w, half * w + half)
+        const uint32_t w2 = static_cast<uint32_t>(lane) >= H ? 1u : 0u;
+        const int back = static_cast<int>(static_cast<uint32_t>(lane) - H * w2 + 32 * w2) & 63;
+        const bool live = static_cast<uint32_t>(lane) < 2 * H;
+#pragma unroll
+        for (int r = 0; r < NB; r++) {
+            const float k = shfl_f32(bk[r], back);
+            const uint32_t v = shfl_u32(bv[r], back);
+            bk[r] = live ? k : FLT_MAX;
+            bv[r] = live ? v : kInvalid;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
     // The candidates of the latest expansion that are below the last beam entry, as a lane mask (one candidate slot per
     // lane).  None: the beam stays as it is -- the half-cleaner of the merge replaces an entry only by a strictly smaller
     // candidate, entry `beam - 1 - k` by the k-th smallest, so if even the smallest candidate is not below the largest
@@ -447,111 +445,6 @@ struct Beam {
         return ballot(ck < tail);
     }
 
-    // Does the beam hold two equal keys (pads aside)?  Asked for beams above 256, where it decides whether the ranked
-    // insertion below is tried.  An entry without a distance that still names a point (the build kernels leave the point
-    // itself unscored) counts as a tie with the pads around it.
-    __device__ __forceinline__ bool beam_has_ties() const {
-        const float up = shfl_f32(bk[0], (lane + 1) & 63);   // first key of the next lane
-        bool t = false;
-#pragma unroll
-        for (int r = 0; r < NB; r++) {
-            const uint32_t e = NB * lane + r;
-            const float next = r + 1 < NB ? bk[r + 1 < NB ? r + 1 : r] : up;
-            t |= e + 1 < p.beam && bk[r] == next && bk[r] < FLT_MAX;
-            t |= e < p.beam && !(bk[r] < FLT_MAX) && bv[r] != kInvalid;
-        }
-        return ballot(t) != 0;
-    }
-
-    // x + 1 in the lanes whose bit is set in `mask`: the carry-in of an add, so one instruction per counter
-    static __device__ __forceinline__ uint32_t add_by_mask(uint32_t x, uint64_t mask) {
-        uint32_t out;
-        uint64_t carry_out;
-        asm("v_addc_co_u32_e64 %0, %1, %2, 0, %3" : "=v"(out), "=s"(carry_out) : "v"(x), "s"(mask));
-        return out;
-    }
-
-    // Beams above 256: candidate sort + two-half merge in one step when a few candidates enter a beam and every key
-    // involved is distinct.  The reference's networks then simply produce "the smallest `beam` of beam and candidates,
-    // ascending", and that can be had without sorting anything: a beam entry moves down by the number of entering
-    // candidates below it, a candidate goes to (beam entries not above it) + (entering candidates before it).  One pass over
-    // the entering candidates (a broadcast and a compare per beam register each) gives all of these counts; the entries
-    // are stored to their places in LDS and read back in beam order.  Equal keys are where the networks' result is their
-    // own business (they never exchange equal keys, and a merge network is not stable): entries ahead of the first
-    // candidate's place never move in either scheme, so ties there do not matter; from there to the first entry that
-    // drops out every two neighbours must differ, or the step reports failure and the caller runs the networks on the
-    // untouched beam.  `em`: lanes whose candidate (`ck`) enters.  Returns true when the beam is up to date.
-    static constexpr uint32_t kRankedLimit = 24;   // more entering candidates than this: the networks are cheaper
-    __device__ __forceinline__ bool insert_ranked(uint64_t em, float ck) {
-        if (static_cast<uint32_t>(__popcll(em)) > kRankedLimit) return false;
-        const bool enter = (em >> lane) & 1;
-        const uint32_t cv = lds->cand_id[lane];
-        uint32_t shift[NB];
-#pragma unroll
-        for (int r = 0; r < NB; r++) shift[r] = 0;
-        uint32_t crank = 0, below = 0, first_place = MAX_BEAM;
-        for (uint64_t rest = em; rest != 0; rest &= rest - 1) {
-            const int j = __builtin_ctzll(rest);
-            const float cj = read_lane(ck, j);
-            uint32_t greater = 0;                               // beam entries above candidate j (wave-uniform)
-#pragma unroll
-            for (int r = 0; r < NB; r++) {
-                const uint64_t g = ballot(cj < bk[r]);
-                shift[r] = add_by_mask(shift[r], g);
-                greater += static_cast<uint32_t>(__popcll(g));
-            }
-            // candidates in (key, lane) order: j goes before this lane's candidate if its key is smaller, or equal from a lower lane
-            const uint64_t lt = ballot(cj < ck), le = ballot(cj <= ck);
-            const uint64_t lanes_above = j == 63 ? 0ull : (~0ull << (j + 1));
-            crank = add_by_mask(crank, (le & lanes_above) | (lt & ~lanes_above));
-            const uint32_t place = MAX_BEAM - greater;          // beam entries not above it (pads count as above)
-            below = lane == j ? place : below;
-            first_place = place < first_place ? place : first_place;
-        }
-        // everything to its place; places 0 .. beam are each taken exactly once (place `beam` by the first entry to drop out)
-#pragma unroll
-        for (int r = 0; r < NB; r++) {
-            const uint32_t at = NB * lane + r + shift[r];
-            if (at <= p.beam) {
-                stage_dist[at] = bk[r];
-                stage_id[at] = bv[r];
-            }
-        }
-        if (enter) {
-            const uint32_t at = below + crank;
-            if (at <= p.beam) {
-                stage_dist[at] = ck;
-                stage_id[at] = cv;
-            }
-        }
-        wave_sync();
-        float nk[NB + 1];
-        uint32_t nv[NB + 1];
-#pragma unroll
-        for (int r = 0; r <= NB; r++) {
-            const uint32_t e = NB * lane + r;
-            nk[r] = e <= p.beam ? stage_dist[e] : FLT_MAX;
-            nv[r] = e <= p.beam ? stage_id[e] : kInvalid;
-        }
-        bool tie = false;
-#pragma unroll
-        for (int r = 0; r < NB; r++) {
-            const uint32_t e = NB * lane + r;
-            tie |= e + 1 >= first_place && e + 1 <= p.beam && nk[r] == nk[r + 1] && !(nv[r] == kInvalid && nv[r + 1] == kInvalid);
-        }
-        const bool clean = ballot(tie) == 0;
-        if (clean) {
-#pragma unroll
-            for (int r = 0; r < NB; r++) {
-                const uint32_t e = NB * lane + r;
-                bk[r] = e < p.beam ? nk[r] : FLT_MAX;
-                bv[r] = e < p.beam ? nv[r] : kInvalid;
-            }
-        }
-        wave_sync();   // the staging area is free again
-        return clean;
-    }
-
     // reference update_result_buffer: sort the candidates, then fold them into the beam
     __device__ __forceinline__ void absorb(bool first) {
         // No row scored: every candidate distance is FLT_MAX, the sort would not move anything (equal keys are never
@@ -562,20 +455,6 @@ struct Beam {
                 float ck;
                 const uint64_t em = entering(ck);
                 if (em == 0) return;
-                if constexpr (MAX_BEAM > 256 && !WHOLE) {
-                    // (A WHOLE kernel does without: its merge is cheap, and without the staging area four of its wavefronts
-                    // fit a SIMD's share of the LDS instead of three, which is worth more than the shortcut was.)
-                    // Only worth trying on a beam without equal keys (on integer-valued rows a beam of 512 rarely is): a
-                    // failed attempt is time lost on a path that is bound by the latency of its own steps.  After a beam
-                    // with equal keys, or an attempt that failed on a candidate's key, the next 16 merges go straight to
-                    // the networks.
-                    if (ranked_pause != 0) {
-                        ranked_pause--;
-                    } else {
-                        if (!beam_has_ties() && insert_ranked(em, ck)) return;
-                        ranked_pause = 16;
-                    }
-                }
             }
         }
         if constexpr (MAX_CAND > 128) sort_candidates_two();
@@ -588,10 +467,9 @@ struct Beam {
                 bk[r] = take ? lds->cand_dist[e] : FLT_MAX;
                 bv[r] = take ? lds->cand_id[e] : kInvalid;
             }
-            if constexpr (MAX_BEAM > 256) ranked_pause = 0;
         } else if constexpr (MAX_BEAM > 256) {
             if constexpr (WHOLE) merge_beam_full();
-            else merge_beam_two();
+            else merge_beam_general();
         } else {
             bool replaced = false;
 #pragma unroll

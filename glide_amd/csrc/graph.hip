@@ -338,7 +338,7 @@ size_t prune_lds_bytes_refine(uint32_t beam, uint32_t degree) {
 int check_beam_sizes(uint32_t degree, uint32_t graph_degree, uint32_t beam, uint32_t dim, uint32_t hash_bit, int metric) {
     if (degree == 0 || graph_degree == 0 || beam == 0 || dim == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
-    if (degree > kMaxDegree || graph_degree > kMaxDegree || beam > 512 || dim % 4 != 0 || dim > 4096 || hash_bit < 1 || hash_bit > 13)
+    if (degree > kMaxDegree || graph_degree > kMaxDegree || !beam_supported(beam) || dim % 4 != 0 || dim > 4096 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     return GLIDE_OK;
 }
@@ -346,8 +346,7 @@ int check_beam_sizes(uint32_t degree, uint32_t graph_degree, uint32_t beam, uint
 int launch_build(BuildArgs& a, hipStream_t stream) {
     build_fn fn = a.p.degree <= 64 ? pick_build_beam<64>(a.p.beam, a.p.dim)
                 : a.p.degree <= 128 ? pick_build_beam<128>(a.p.beam, a.p.dim) : pick_build_beam<256>(a.p.beam, a.p.dim);
-    const size_t lds_bytes = beam_lds_bytes(a.p.degree) + prune_lds_bytes(a.p.beam) + (size_t{1} << a.p.hash_bit) * sizeof(uint32_t) +
-                             beam_stage_bytes(a.p.beam);
+    const size_t lds_bytes = beam_lds_bytes(a.p.degree) + prune_lds_bytes(a.p.beam) + (size_t{1} << a.p.hash_bit) * sizeof(uint32_t);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(a.point_count), dim3(64), lds_bytes, stream, a);
     return launch_status();
@@ -476,8 +475,7 @@ int glide_hip_refine_segment(const float* segment_data, uint32_t num, uint32_t d
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
     refine_fn fn = graph_degree <= 64 ? pick_refine_beam<64>(beam, dim)
                  : graph_degree <= 128 ? pick_refine_beam<128>(beam, dim) : pick_refine_beam<256>(beam, dim);
-    const size_t lds_bytes = beam_lds_bytes(graph_degree) + prune_lds_bytes(beam) + (size_t{1} << hash_bit) * sizeof(uint32_t) +
-                             beam_stage_bytes(beam);
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + prune_lds_bytes(beam) + (size_t{1} << hash_bit) * sizeof(uint32_t);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
@@ -579,7 +577,7 @@ int launch_refine(const float* data, uint32_t num, uint32_t dim, const uint32_t*
     refine_fn fn = graph_degree <= 64 ? pick_refine_beam<64>(beam, dim)
                  : graph_degree <= 128 ? pick_refine_beam<128>(beam, dim) : pick_refine_beam<256>(beam, dim);
     const size_t lds_bytes = beam_lds_bytes(graph_degree) + prune_lds_bytes_refine(beam, graph_degree) + round_up32(centroid_num) * sizeof(float) +
-                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam);
+                             (size_t{1} << hash_bit) * sizeof(uint32_t);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();

@@ -58,8 +58,11 @@ __device__ __forceinline__ void search_body(const SearchArgs a) {
     }
 }
 
+// Beams above 256 on rows of up to 512 dims: held to the registers of four wavefronts per SIMD (the kernel asks for a
+// dozen more, which costs it the fourth wavefront and buys nothing: the vector ALU is the limit).
 template <int MAX_CAND, int MAX_BEAM, int DIMV, bool WHOLE = false>
-__global__ __launch_bounds__(64) void search_kernel(SearchArgs a) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(MAX_BEAM > 256 && DIMV <= 4 ? 4 : 1)))
+void search_kernel(SearchArgs a) {
     search_body<MAX_CAND, MAX_BEAM, DIMV, WHOLE>(a);
 }
 // The beam-256 kernels are bound by the vector ALU (sorting networks) and need 103 registers, one wavefront per SIMD
@@ -228,7 +231,7 @@ int launch_search(const float* data, uint32_t num, uint32_t dim, const uint32_t*
         return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0) return GLIDE_OK;
-    if (graph_degree > 256 || beam > 512 || centroid_num > 256 || dim % 4 != 0 || dim > 4096 || top_k > beam ||
+    if (graph_degree > 256 || !beam_supported(beam) || centroid_num > 256 || dim % 4 != 0 || dim > 4096 || top_k > beam ||
         hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     if (reinterpret_cast<uintptr_t>(data) % 16 || reinterpret_cast<uintptr_t>(queries) % 16 ||
@@ -264,7 +267,7 @@ int launch_search(const float* data, uint32_t num, uint32_t dim, const uint32_t*
     if (team) fn = graph_degree <= 64 ? pick_team_beam<64>(beam, dim) : graph_degree <= 128 ? pick_team_beam<128>(beam, dim) : pick_team_beam<256>(beam, dim);
     else fn = graph_degree <= 64 ? pick_beam<64>(beam, dim) : graph_degree <= 128 ? pick_beam<128>(beam, dim) : pick_beam<256>(beam, dim);
     const size_t lds_bytes = beam_lds_bytes(graph_degree) + round_up32(centroid_num) * sizeof(float) +
-                             (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam, beam == 512) +
+                             (size_t{1} << hash_bit) * sizeof(uint32_t) +
                              (team ? (dim <= 512 ? TeamShape<4>::query_bytes : dim <= 1024 ? TeamShape<8>::query_bytes : dim <= 2048 ? TeamShape<16>::query_bytes : TeamShape<32>::query_bytes) + 16 : 0);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     if (team) hipLaunchKernelGGL(fn, dim3(query_num), dim3(64 * kTeam), lds_bytes, as_stream(stream), a);

@@ -375,7 +375,7 @@ int launch_search_sub(const float* segment_data, uint32_t dim, const uint32_t* s
     if (dim == 0 || graph_degree == 0 || centroid_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0 || (query_list && list_len == 0)) return GLIDE_OK;
-    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 4096 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
+    if (graph_degree > 256 || !beam_supported(beam) || dim % 4 != 0 || dim > 4096 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;   // top_k buckets: kernel_config.cuh:312-323
     SubArgs a;
     a.data = segment_data;
@@ -401,7 +401,7 @@ int launch_search_sub(const float* segment_data, uint32_t dim, const uint32_t* s
     a.max_topk = top_k <= 32 ? 32 : (top_k <= 64 ? 64 : 128);
     a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
     sub_fn fn = graph_degree <= 64 ? pick_sub_beam<64>(beam, dim) : graph_degree <= 128 ? pick_sub_beam<128>(beam, dim) : pick_sub_beam<256>(beam, dim);
-    const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam, beam == 512);
+    const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t);
     GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
     hipLaunchKernelGGL(fn, dim3(query_list ? list_len : query_num), dim3(64), lds_bytes, as_stream(stream), a);
     return launch_status();
@@ -486,7 +486,7 @@ extern "C" int glide_hip_search_partitions(const float* data, uint32_t dim, cons
     if (dim == 0 || graph_degree == 0 || segment_num == 0 || beam == 0 || top_k == 0 || max_iterations == 0) return GLIDE_ERR_BAD_ARGUMENT;
     if (metric != GLIDE_METRIC_EUCLIDEAN && metric != GLIDE_METRIC_COSINE) return GLIDE_ERR_BAD_ARGUMENT;
     if (query_num == 0) return GLIDE_OK;
-    if (graph_degree > 256 || beam > 512 || dim % 4 != 0 || dim > 4096 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
+    if (graph_degree > 256 || !beam_supported(beam) || dim % 4 != 0 || dim > 4096 || top_k > beam || top_k > 128 || hash_bit < 1 || hash_bit > 13)
         return GLIDE_ERR_UNSUPPORTED;
     if (static_cast<unsigned long long>(query_num) * segment_num >= 0xffffffffull) return GLIDE_ERR_UNSUPPORTED;   // pairs are numbered with 32 bits
     const PartitionSearchLayout l = partition_search_layout(query_num, segment_num, top_k);
@@ -536,7 +536,7 @@ extern "C" int glide_hip_search_partitions(const float* data, uint32_t dim, cons
         a.list_len = pairs;
         a.p = BeamParams{beam, graph_degree, dim, hash_bit, hash_reset_interval ? hash_reset_interval : 1, max_iterations, min_iterations, metric};
         sub_fn fn = graph_degree <= 64 ? pick_sub_beam<64>(beam, dim) : graph_degree <= 128 ? pick_sub_beam<128>(beam, dim) : pick_sub_beam<256>(beam, dim);
-        const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t) + beam_stage_bytes(beam, beam == 512);
+        const size_t lds_bytes = beam_lds_bytes(graph_degree) + 128 * 8 + (size_t{1} << hash_bit) * sizeof(uint32_t);
         GLIDE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
         hipLaunchKernelGGL(fn, dim3(pairs), dim3(64), lds_bytes, s, a);
     }

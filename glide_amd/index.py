@@ -117,7 +117,7 @@ def make_search_parameter(beam, degree, top_k=10):
 
 def _check_sizes(beam, degree):
     # kernel_config.cuh:48,60: std::invalid_argument("Unsupported beam" / "Unsupported graph_degree")
-    if beam > 512:
+    if beam > 512 or (beam > 256 and beam % 16):     # the second: adjust_search_params rounds beams to multiples of 32
         raise ValueError("Unsupported beam")
     if degree > 256:
         raise ValueError("Unsupported graph_degree")

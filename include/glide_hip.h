@@ -67,8 +67,9 @@ int glide_hip_event_elapsed_ms(void *start, void *stop, float *ms); /* synchroni
  * kernel adds {beam iterations, data rows scored, graph rows read} into the stripe of each workgroup (one shared
  * address would serialise the launch); the sums over the stripes are the algorithmic-traffic tallies.
  * Limits (reference kernel_config.cuh:41-60): graph_degree <= 256, beam <= 512, centroid_num <= 256, dim % 4 == 0,
- * dim <= 4096, top_k <= beam.  Degrees above 128 and beams above 256 run the candidate sort / beam merge as two
- * half-wave networks, as the reference's two-warp branches do (search_kernel.cuh:38-94, :149-232). */
+ * dim <= 4096, top_k <= beam; a beam above 256 is a multiple of 16 (params.cuh:82-99 rounds beams to multiples of 32).
+ * Degrees above 128 and beams above 256 run the candidate sort / beam merge as two half-wave networks, as the
+ * reference's two-warp branches do (search_kernel.cuh:38-94, :149-232). */
 int glide_hip_search(const float *data, uint32_t num, uint32_t dim, const uint32_t *graph, uint32_t graph_degree,
                      const float *centroids, uint32_t centroid_num, const uint32_t *start_points,
                      const float *queries, uint32_t query_num, uint32_t top_k, uint32_t beam,

@@ -131,11 +131,11 @@ def test_long_rows_small_and_large_batches_agree(hip, dim, deg):
 
 @pytest.mark.parametrize("deg", [32, 64])
 def test_wide_beams_on_distinct_keys(hip, deg):
-    """Beams of 288 to 480 insert a few entering candidates by rank instead of running candidate sort and two-half merge
-    when every key involved is distinct.  Points on a line and queries beyond its ends make all distances of a search
-    distinct (and exact), so that path does the merging here; ids, distances and counters must be the oracle's.  A second
-    data set repeats every position once: beams with equal keys, where the networks must take over.  Beam 512 runs the
-    kernel form that merges the whole beam in its registers, on the same two data sets."""
+    """Beams above 256 on keys that are all distinct, and on keys that repeat.  Points on a line and queries beyond its
+    ends make all distances of a search distinct (and exact); a second data set repeats every position once, so that
+    beams hold equal keys, where the order the reference's two-half merge leaves is the network's own.  Beams 288 and 448
+    run the merge with its lane permutations, beam 512 the whole-beam form; ids, distances and counters must be the
+    oracle's."""
     from oracle import oracle as O
     rng = np.random.default_rng(deg)
     n = 3000
@@ -189,7 +189,7 @@ def test_search_rejects_unsupported_sizes(hip):
     base = dict(data=d, num=8, dim=128, graph=d, graph_degree=32, centroids=d, centroid_num=2, start_points=d, queries=d,
                 query_num=1, top_k=10, beam=64, max_iterations=10, min_iterations=0, hash_bit=8, hash_reset_interval=2,
                 metric=0, result_ids=d, result_dists=d)
-    for key, bad in (("beam", 544), ("graph_degree", 257), ("centroid_num", 300), ("dim", 130), ("dim", 4100), ("top_k", 65)):
+    for key, bad in (("beam", 544), ("beam", 300), ("graph_degree", 257), ("centroid_num", 300), ("dim", 130), ("dim", 4100), ("top_k", 65)):
         with pytest.raises(hip.GlideHipError) as e:
             hip.search(**{**base, key: bad})
         assert e.value.code == -1, key
