@@ -245,7 +245,8 @@ __device__ __forceinline__ void merge_result(const float* beam_dist, const uint3
 
 // search_on_sub_kernel (search_kernel.cuh:653-765)
 template <int MAX_CAND, int MAX_BEAM, int DIMV, bool WHOLE = false>
-__global__ __launch_bounds__(64) void search_sub_kernel(SubArgs a) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(MAX_BEAM > 256 && DIMV <= 4 ? 4 : 1)))   // as search_kernel
+void search_sub_kernel(SubArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     auto* lds = reinterpret_cast<BeamLds<MAX_CAND>*>(smem);
     float* head_dist = reinterpret_cast<float*>(smem + sizeof(BeamLds<MAX_CAND>));   // beam head staged for the merge (128 pairs)

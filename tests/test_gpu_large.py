@@ -77,7 +77,7 @@ def test_select_segments_bit_exact(hip, c, min_seg, bf):
     assert ((want != INV).sum(1) >= min(min_seg, c)).all()
 
 
-@pytest.mark.parametrize("top_k,beam", [(10, 64), (40, 128), (100, 256)])
+@pytest.mark.parametrize("top_k,beam", [(10, 64), (40, 128), (100, 256), (10, 320), (64, 448), (128, 512)])
 def test_search_over_partitions_bit_exact(hip, large_index, top_k, beam):
     from glide_amd.datasets import recall
     from oracle import oracle as O
