@@ -12,7 +12,7 @@ def _cases():
     rng = np.random.default_rng(777)
     dims = [4, 36, 128, 132, 256, 512, 960, 1536, 2048, 3072, 4096]
     degrees = [8, 24, 32, 64, 96, 160]
-    beams = [32, 64, 128, 256, 320]
+    beams = [32, 64, 128, 256, 320, 448, 512]
     out = []
     for i in range(28):
         out.append((i, int(rng.choice(dims)), int(rng.choice(degrees)), int(rng.choice(degrees)), int(rng.choice(beams)), int(rng.choice(beams)),
