@@ -11,7 +11,7 @@ def _cases():
     rng = np.random.default_rng(20240)
     dims = [4, 8, 36, 100, 128, 132, 256, 260, 512, 960, 1024, 1028, 1536, 2048, 2052, 3072, 4096]
     degrees = [8, 16, 24, 32, 40, 64, 72, 96, 128, 160, 256]
-    beams = [32, 64, 96, 128, 192, 256, 320, 512]
+    beams = [32, 64, 96, 128, 192, 256, 288, 320, 448, 480, 512]
     out = []
     for i in range(72):
         dim, deg, beam = int(rng.choice(dims)), int(rng.choice(degrees)), int(rng.choice(beams))
