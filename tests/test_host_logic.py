@@ -25,6 +25,11 @@ def test_unsupported_sizes_raise_like_the_reference():
     import pytest
     with pytest.raises(ValueError, match="Unsupported beam"):
         G._check_sizes(513, 32)
+    with pytest.raises(ValueError, match="Unsupported beam"):
+        G._check_sizes(300, 32)        # above 256 a beam is a multiple of 16; adjust_search_params never hands out another
+    for beam in (1, 50, 255, 256, 288, 320, 448, 480, 512):
+        G._check_sizes(beam, 32)
+    assert all(G.adjust_search_params(0, 0, b)[1] % 32 == 0 for b in range(1, 513))
     with pytest.raises(ValueError, match="Unsupported graph_degree"):
         G._check_sizes(64, 257)
 
