@@ -154,6 +154,7 @@ def parse():
     ap.add_argument("--details-file", default=os.path.join("gpurun_out", "bench_full.json"),
                     help="where the per-workload details are written as one JSON file (relative to the repository root)")
     ap.add_argument("--queries", type=int, default=0, help="use only the first N queries of the workload (small-batch measurements)")
+    ap.add_argument("--extra-beams", default="", help="comma-separated beams to add to the sweep, e.g. 288,320,384,448,480")
     ap.add_argument("--partition-only", type=int, default=0, metavar="C",
                     help="only time partition assignment of 1M x 128 rows against C centroids (fp32 matrix-core tile) and exit")
     return ap.parse_args()
@@ -283,6 +284,9 @@ def run_workload(args, workload, torch, want_cpu):
         return rec
 
     recalls = {beam: measure(beam) for beam in SWEEP_BEAMS}
+    for beam in sorted({int(b) for b in args.extra_beams.split(",") if b} - set(SWEEP_BEAMS)):
+        measure(beam)
+    sweep.sort(key=lambda s: s["beam"])
     # "the smallest beam reaching the target": where a power of two reaches it and the one before does not, the three
     # beams between them (steps of an eighth of the larger one) are measured as well
     if workload not in NAMED_BEAMS:
