@@ -489,12 +489,14 @@ struct Beam {
             // network (strict comparisons) is the identity on it.
             if (ballot(replaced) != 0) {
                 WaveNet<MAX_BEAM>::merge(bk, bv, lane);
+                if (p.beam < MAX_BEAM) {   // a beam that fills its bucket has nothing behind it (and the lane masks of this loop are not held)
 #pragma unroll
-                for (int r = 0; r < NB; r++) {
-                    const uint32_t e = NB * lane + r;
-                    if (e >= p.beam) {
-                        bk[r] = FLT_MAX;
-                        bv[r] = kInvalid;
+                    for (int r = 0; r < NB; r++) {
+                        const uint32_t e = NB * lane + r;
+                        if (e >= p.beam) {
+                            bk[r] = FLT_MAX;
+                            bv[r] = kInvalid;
+                        }
                     }
                 }
             }
@@ -504,12 +506,11 @@ struct Beam {
 
     // first unexplored beam entry (reference select_current_point); marks it explored
     __device__ __forceinline__ uint32_t select_parent() {
+        // entries behind the beam are pads (kInvalid), which carry the explored bit like every unfilled entry
         int rsel = NB;
 #pragma unroll
-        for (int r = NB - 1; r >= 0; r--) {
-            const uint32_t e = NB * lane + r;
-            if (e < p.beam && (bv[r] & kExplored) == 0) rsel = r;
-        }
+        for (int r = NB - 1; r >= 0; r--)
+            if ((bv[r] & kExplored) == 0) rsel = r;
         const uint64_t m = ballot(rsel < NB);
         if (m == 0) return kInvalid;
         const int src = __builtin_ctzll(m);
