@@ -437,10 +437,15 @@ struct Beam {
         // below `beam` (written as a maximum: a chain of selects between the registers becomes a run-time index, which
         // moves the beam out of the registers).  Keys are not negative.
         const uint32_t last = p.beam - 1;
-        float mine = bk[0];
+        float tail;
+        if (p.beam == MAX_BEAM) {   // a beam that fills its bucket ends in the last register of the last lane
+            tail = read_lane(bk[NB - 1], 63);
+        } else {
+            float mine = bk[0];
 #pragma unroll
-        for (int r = 1; r < NB; r++) mine = fmaxf(mine, NB * lane + r <= static_cast<int>(last) ? bk[r] : 0.f);
-        const float tail = read_lane(mine, static_cast<int>(last / NB));
+            for (int r = 1; r < NB; r++) mine = fmaxf(mine, NB * lane + r <= static_cast<int>(last) ? bk[r] : 0.f);
+            tail = read_lane(mine, static_cast<int>(last / NB));
+        }
         ck = static_cast<uint32_t>(lane) < p.degree ? lds->cand_dist[lane] : FLT_MAX;
         return ballot(ck < tail);
     }
